@@ -1,0 +1,48 @@
+"""ctypes binding of libnq_moe_hip.so (the C ABI in include/nq_moe_hip.h).
+
+There is no fallback: if the library is missing, `lib()` raises. Build it with `python -m nestquant_amd.build`.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libnq_moe_hip.so")
+_lib = None
+
+_vp, _i, _i64p, _i32p = C.c_void_p, C.c_int, C.c_void_p, C.c_void_p
+
+# name -> (restype, argtypes); every symbol declared in include/nq_moe_hip.h
+SIGNATURES = {
+    "nq_abi_version": (C.c_int, []),
+    "nq_last_error": (C.c_char_p, []),
+    "nq_codes": (C.c_int, [C.POINTER(C.c_uint32)]),
+    "nq_validate_row": (C.c_int, [C.POINTER(C.c_int64), _i, _i]),
+    "nq_dequant": (C.c_int, [_i64p, _i, _i, _i, _i, _vp, _vp]),
+    "nq_pf_decode": (C.c_int, [_i64p, _i32p, _i, _vp, _vp, _i, _i, _vp]),
+}
+
+
+def lib():
+    """the loaded library; raises RuntimeError when it has not been built"""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(f"{LIB_PATH} is missing: run `python -m nestquant_amd.build` (there is no CPU fallback)")
+        L = C.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(L, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = L
+    return _lib
+
+
+def check(rc):
+    """raise the library's last error as RuntimeError (the reference raises RuntimeError from TORCH_CHECK)"""
+    if rc:
+        raise RuntimeError(lib().nq_last_error().decode())
+
+
+def stream_ptr():
+    """raw hipStream_t of torch's current stream"""
+    import torch
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)

@@ -1,0 +1,52 @@
+"""Build libnq_moe_hip.so for gfx950 with hipcc (in-tree; `python -m nestquant_amd.build`).
+
+Replaces the reference's JIT build (sm120/build.py:7-12): explicit hipcc, one object per .hip file compiled in parallel,
+linked into nestquant_amd/libnq_moe_hip.so. Cross-compiles without a GPU.
+"""
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "libnq_moe_hip.so")
+OBJ = os.path.join(HERE, "build")
+ARCH = "gfx950"
+FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-ffp-contract=off",
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
+
+
+def sources():
+    return sorted(f for f in os.listdir(CSRC) if f.endswith(".hip"))
+
+
+def _run(cmd):
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "is not a recognized feature for this target"
+    err = "\n".join(l for l in r.stderr.splitlines() if noise not in l)
+    if r.returncode:
+        raise RuntimeError("build failed: " + " ".join(cmd) + "\n" + err)
+    return err
+
+
+def build(verbose=False, jobs=None):
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    os.makedirs(OBJ, exist_ok=True)
+    srcs = sources()
+    objs = [os.path.join(OBJ, s[:-4] + ".o") for s in srcs]
+
+    def one(i):
+        cmd = [hipcc] + FLAGS + ["-c", os.path.join(CSRC, srcs[i]), "-o", objs[i]]
+        out = _run(cmd)
+        if verbose and out.strip():
+            print(out, file=sys.stderr)
+
+    with ThreadPoolExecutor(max_workers=jobs or min(8, len(srcs))) as ex:
+        list(ex.map(one, range(len(srcs))))
+    _run([hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", LIB] + objs)
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build(verbose=True))

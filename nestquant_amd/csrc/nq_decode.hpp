@@ -1,0 +1,243 @@
+// Nested-trellis decode primitives for gfx950 (wave64). Header shared by the dequant, decode-GEMV and prefill kernels.
+//
+// Format being decoded (reference sm120/nqmoe.cu:14-25, sm120/ref15_spec.py:3-24):
+//   unit   = 16 rows x 128 columns = 8 tail-biting rings x 256 weights; ring g = records of lanes 4g..4g+3
+//   record = one lane's 64 weights in one plane; base record = 128 bits (2 bits / step); residual record = RBITS bits
+//   state(j) = 16-bit window of the lane's record (extended by the ring neighbour's first word) at step_off(j)
+//   hash     x = state * 0x83DCD12D mod 2^32 ; S = byte sum of x
+//   level 2  w = fp16(A * (1024 + S_b) + B)                                      A = 0x1eee, B = 0xc931
+//   level 3/4 F = (Mb S_b + N S_r + 128) >> 8 ; w = fp16(A' * (1024 + F) + C)   block word Mb | N << 8 per unit
+//
+// gfx950 instruction choices:
+//   * the hash multiply is split into two full-rate 16-bit multiplies (v_mad_u32_u16 + v_pk_mad_u16 with op_sel), which
+//     read only a 16-bit half of their source, so a window needs no masking and every second window (offset + 16) is
+//     the high half of a register that was already produced for its partner: half a v_alignbit per weight;
+//   * v_sad_u8 / v_sad_hi_u8 give the byte sums of two weights already packed as the fp16 pair (1024 + S);
+//   * v_dot4_u32_u8 folds Mb * S_b + N * S_r with the rounding constant in its accumulator; v_perm_b32 packs a pair.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace nq {
+
+constexpr int TBL_W = 20;                       // int64 words per table row (reference sm120/moe.py:6)
+constexpr uint32_t HASH_LO = 0xD12Du;           // 0x83DCD12D = HASH_HI << 16 | HASH_LO
+constexpr uint32_t HASH_HI_SHL = 0x83DC0000u;   // high multiplier in the upper half, zero in the lower half
+constexpr uint32_t MUL1_A2 = 0x1eee1eeeu;       // fp16 A twice
+constexpr uint32_t MUL1_B2 = 0xc931c931u;       // fp16 B twice
+constexpr int CODE_L3 = 10, CODE_L4N = 11;      // nested planes of this build: K=1 plane; P3 record || P4 record
+constexpr int NCODES = 12;
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+
+// ---- window patterns (reference sm120/moe.py:10-12, sm120/nqmoe.cu:128-138) ----------------------------------------
+template <int CODE> struct Pat;
+template <> struct Pat<0>  { static constexpr int KA = 2, M = 0x0000; static constexpr bool SPLIT = false; };
+template <> struct Pat<1>  { static constexpr int KA = 1, M = 0xEEEE; static constexpr bool SPLIT = false; };
+template <> struct Pat<2>  { static constexpr int KA = 2, M = 0xAAAA; static constexpr bool SPLIT = false; };
+template <> struct Pat<3>  { static constexpr int KA = 2, M = 0x8888; static constexpr bool SPLIT = false; };
+template <> struct Pat<4>  { static constexpr int KA = 3, M = 0x0000; static constexpr bool SPLIT = false; };
+template <> struct Pat<5>  { static constexpr int KA = 1, M = 0xAAAA; static constexpr bool SPLIT = false; };
+template <> struct Pat<6>  { static constexpr int KA = 1, M = 0xFFFE; static constexpr bool SPLIT = false; };
+template <> struct Pat<7>  { static constexpr int KA = 2, M = 0x9248; static constexpr bool SPLIT = false; };
+template <> struct Pat<8>  { static constexpr int KA = 1, M = 0xFEFE; static constexpr bool SPLIT = false; };
+template <> struct Pat<9>  { static constexpr int KA = 2, M = 0xD5AA; static constexpr bool SPLIT = false; };
+template <> struct Pat<10> { static constexpr int KA = 1, M = 0x0000; static constexpr bool SPLIT = false; };
+template <> struct Pat<11> { static constexpr int KA = 2, M = 0x0000; static constexpr bool SPLIT = true; };
+
+__host__ __device__ constexpr int popc16(int m) { int c = 0; for (int i = 0; i < 16; ++i) c += (m >> i) & 1; return c; }
+__host__ __device__ constexpr int step_off(int j, int KA, int M)
+{
+    int s = (j >> 4) * (16 * KA + popc16(M));
+    for (int i = 0; i < (j & 15); ++i) s += KA + ((M >> i) & 1);
+    return s;
+}
+template <int CODE> struct Rec
+{
+    static constexpr int KA = Pat<CODE>::KA, M = Pat<CODE>::M;
+    static constexpr int BITS = 4 * (16 * KA + popc16(M));
+    static constexpr int NW = (BITS + 31) / 32;
+    static constexpr int off(int j) { return step_off(j, KA, M); }
+};
+__host__ inline int rec_bits(int code)
+{
+    constexpr int ka[NCODES] = {2, 1, 2, 2, 3, 1, 1, 2, 1, 2, 1, 2};
+    constexpr int mk[NCODES] = {0, 0xEEEE, 0xAAAA, 0x8888, 0, 0xAAAA, 0xFFFE, 0x9248, 0xFEFE, 0xD5AA, 0, 0};
+    return 4 * (16 * ka[code] + popc16(mk[code]));
+}
+
+// ---- record loads ---------------------------------------------------------------------------------------------------
+// Residual plane = sub-arrays uint4 x n4 | uint2 | uint | ushort, each contiguous over all nrec records, then a tail of
+// BITS % 16 bits per record bit-packed over records (reference sm120/moe.py:36-49, sm120/nqmoe.cu:17-20).
+// Code 11 stores its 128-bit record as uint2 (plane P3) | uint2 (plane P4).
+template <int CODE>
+__device__ __forceinline__ void load_record(uint32_t* w, const uint8_t* __restrict__ p, size_t rec, size_t nrec)
+{
+    constexpr int BITS = Rec<CODE>::BITS;
+    if constexpr (Pat<CODE>::SPLIT)
+    {
+        const uint2 a = ((const uint2*)p)[rec], b = ((const uint2*)(p + nrec * 8))[rec];
+        w[0] = a.x; w[1] = a.y; w[2] = b.x; w[3] = b.y;
+    }
+    else
+    {
+        constexpr int n4 = BITS / 128, r1 = BITS % 128, n2 = r1 / 64, r2 = r1 % 64, n1 = r2 / 32, nh = (r2 % 32) / 16;
+        constexpr int T = BITS % 16;
+        int k = 0;
+#pragma unroll
+        for (int i = 0; i < n4; ++i)
+        {
+            const uint4 v = ((const uint4*)p)[rec * n4 + i];
+            w[k++] = v.x; w[k++] = v.y; w[k++] = v.z; w[k++] = v.w;
+        }
+        p += nrec * 16 * n4;
+        if constexpr (n2) { const uint2 v = ((const uint2*)p)[rec]; w[k++] = v.x; w[k++] = v.y; p += nrec * 8; }
+        if constexpr (n1) { w[k++] = ((const uint32_t*)p)[rec]; p += nrec * 4; }
+        if constexpr (nh) { w[k++] = ((const uint16_t*)p)[rec]; p += nrec * 2; }
+        if constexpr (T)
+        {
+            const size_t b = rec * T;
+            const uint32_t* q = (const uint32_t*)p + (b >> 5);
+            const int sh = (int)(b & 31);
+            uint32_t v;
+            if constexpr (32 % T) v = __builtin_amdgcn_alignbit(q[1], q[0], sh);   // q[1] lies inside the 4-byte pad
+            else v = q[0] >> sh;
+            v &= (1u << T) - 1u;
+            if constexpr (((BITS - T) & 31) == 16) w[k - 1] |= v << 16; else w[k++] = v;
+        }
+    }
+}
+
+// stream bits [BITS, BITS + 32) of a lane = first word of the next lane of its ring (tail-biting)
+template <int BITS, int NW>
+__device__ __forceinline__ void ext_words(uint32_t* w, uint32_t nb)
+{
+    constexpr int T = BITS % 32;
+    if constexpr (T == 0) { w[NW] = nb; w[NW + 1] = 0; }
+    else
+    {
+        w[NW - 1] = (w[NW - 1] & ((1u << T) - 1u)) | (nb << T);
+        w[NW] = nb >> (32 - T);
+        w[NW + 1] = 0;
+    }
+}
+
+// ---- hash -----------------------------------------------------------------------------------------------------------
+// x = st * 0x83DCD12D mod 2^32 with st = the low (HI = false) or high (HI = true) 16 bits of r; other bits ignored.
+template <bool HI>
+__device__ __forceinline__ uint32_t hash16(uint32_t r)
+{
+    uint32_t y, x;
+    const uint32_t klo = HASH_LO, khi = HASH_HI_SHL;
+    if constexpr (!HI)
+    {
+        asm("v_mad_u32_u16 %0, %1, %2, 0" : "=v"(y) : "v"(r), "s"(klo));
+        asm("v_pk_mad_u16 %0, %1, %2, %3 op_sel:[0,0,0] op_sel_hi:[0,1,1]" : "=v"(x) : "v"(r), "s"(khi), "v"(y));
+    }
+    else
+    {
+        asm("v_mad_u32_u16 %0, %1, %2, 0 op_sel:[1,0,0,0]" : "=v"(y) : "v"(r), "s"(klo));
+        asm("v_pk_mad_u16 %0, %1, %2, %3 op_sel:[1,0,0] op_sel_hi:[1,1,1]" : "=v"(x) : "v"(r), "s"(khi), "v"(y));
+    }
+    return x;
+}
+// hash of the 16-bit window at bit offset O of the extended record w[]. Windows O and O + 16 share one register.
+template <int O>
+__device__ __forceinline__ uint32_t hash_at(const uint32_t* w)
+{
+    constexpr bool HI = (O & 31) >= 16;
+    constexpr int o = HI ? O - 16 : O, i = o >> 5, s = o & 31;
+    uint32_t r;
+    if constexpr (s == 0) r = w[i]; else r = __builtin_amdgcn_alignbit(w[i + 1], w[i], s);
+    return hash16<HI>(r);
+}
+
+// ---- per-unit constants ---------------------------------------------------------------------------------------------
+struct FoldK { uint32_t Mrep, Nrep, A2, C2; };      // Mb and N replicated into 4 bytes; fp16 A', C replicated twice
+
+// IEEE 1.0f / i, i = 1..255 (entry 0 unused)
+struct RcpTable { float v[256]; };
+constexpr RcpTable make_rcp() { RcpTable t{}; t.v[0] = 0.f; for (int i = 1; i < 256; ++i) t.v[i] = 1.0f / (float)i; return t; }
+static __device__ __constant__ const RcpTable c_rcp = make_rcp();
+
+// level-2 constants with the ring's sign (sgm = 0x80008000 negates exactly)
+__device__ __forceinline__ FoldK consts_l2(uint32_t sgm) { return FoldK{0u, 0u, MUL1_A2 ^ sgm, MUL1_B2 ^ sgm}; }
+// fold constants, fp32 operations in the spec's order without contraction (reference sm120/ref15_spec.py:79-84)
+__device__ __forceinline__ FoldK consts_fold(uint32_t dw, uint32_t sgm)
+{
+    const uint32_t Mb = dw & 0xFFu, N = (dw >> 8) & 0xFFu;
+    const float rc = c_rcp.v[Mb];
+    const _Float16 Ah = (_Float16)__fmul_rn(1.732421875f, rc);
+    const float t = __fadd_rn(__fmul_rn(__fmul_rn((float)N, rc), -3.453125f), -3.453125f);
+    const _Float16 Ch = (_Float16)__fsub_rn(t, __fmul_rn(1024.f, (float)Ah));
+    const uint32_t a = (uint32_t)__builtin_bit_cast(uint16_t, Ah), c = (uint32_t)__builtin_bit_cast(uint16_t, Ch);
+    return FoldK{Mb * 0x01010101u, N * 0x01010101u, (a * 0x00010001u) ^ sgm, (c * 0x00010001u) ^ sgm};
+}
+
+__device__ __forceinline__ uint32_t pk_fma(uint32_t h, uint32_t a, uint32_t c)
+{
+    const half2_t r = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, h), __builtin_bit_cast(half2_t, a),
+                                                __builtin_bit_cast(half2_t, c));
+    return __builtin_bit_cast(uint32_t, r);
+}
+
+// ---- pair decode ----------------------------------------------------------------------------------------------------
+// fp16 pair (1024 + S or 1024 + F) of lane weights JA (low half) and JB (high half); exact integers in fp16.
+// RES = false: base only. wb: extended base record (6 words); wr: extended residual record.
+template <bool RES, int CODE, int JA, int JB>
+__device__ __forceinline__ uint32_t code_pair(const uint32_t* wb, const uint32_t* wr, const FoldK& k)
+{
+    const uint32_t xa = hash_at<2 * JA>(wb), xb = hash_at<2 * JB>(wb);
+    if constexpr (!RES)
+    {
+        const uint32_t t = __builtin_amdgcn_sad_u8(xa, 0u, 0x64006400u);
+        return __builtin_amdgcn_sad_hi_u8(xb, 0u, t);
+    }
+    else
+    {
+        uint32_t ta = __builtin_amdgcn_udot4(xa, k.Mrep, 0x640080u, false);
+        uint32_t tb = __builtin_amdgcn_udot4(xb, k.Mrep, 0x640080u, false);
+        ta = __builtin_amdgcn_udot4(hash_at<Rec<CODE>::off(JA)>(wr), k.Nrep, ta, false);
+        tb = __builtin_amdgcn_udot4(hash_at<Rec<CODE>::off(JB)>(wr), k.Nrep, tb, false);
+        return __builtin_amdgcn_perm(tb, ta, 0x06050201u);          // bits [8, 24) of ta, then of tb
+    }
+}
+// decoded fp16 weight pair (bit-exact values)
+template <bool RES, int CODE, int JA, int JB>
+__device__ __forceinline__ uint32_t weight_pair(const uint32_t* wb, const uint32_t* wr, const FoldK& k)
+{
+    return pk_fma(code_pair<RES, CODE, JA, JB>(wb, wr, k), k.A2, k.C2);
+}
+
+// ---- table row ------------------------------------------------------------------------------------------------------
+// int64[20] per expert (reference sm120/moe.py:216-229, sm120/nqmoe.cu:26-45):
+//   [0] level 0/2/3/4  [1..4] gate|up base, residual plane, block words, flags  [5..8] down  [9] sign/scale vector
+//   [10],[11] residual window code of gate|up, down  [12],[13] sign-variant planes  [14..17] low-rank plane (unsupported)
+//   [18] in_had_down (unsupported unless 0/128)  [19] base codes (unsupported unless 0)
+struct Planes { const uint4* base; const uint8_t* res; const uint32_t* dw; const uint8_t* var; int code; };
+__device__ __forceinline__ Planes planes_of(const int64_t* ent, int mode)
+{
+    const int o = mode == 0 ? 1 : 5;
+    Planes P;
+    P.base = (const uint4*)ent[o]; P.res = (const uint8_t*)ent[o + 1]; P.dw = (const uint32_t*)ent[o + 2];
+    P.var = (const uint8_t*)ent[mode == 0 ? 12 : 13]; P.code = (int)ent[10 + mode];
+    return P;
+}
+
+// compile-time dispatch over the residual code; F is a generic lambda taking std::integral_constant<int, CODE>
+template <int C> struct CodeTag { static constexpr int value = C; };
+template <class F>
+__device__ __forceinline__ void dispatch_code(int code, F&& f)
+{
+    switch (code)
+    {
+        case 1: f(CodeTag<1>{}); break;   case 2: f(CodeTag<2>{}); break;   case 3: f(CodeTag<3>{}); break;
+        case 4: f(CodeTag<4>{}); break;   case 5: f(CodeTag<5>{}); break;   case 6: f(CodeTag<6>{}); break;
+        case 7: f(CodeTag<7>{}); break;   case 8: f(CodeTag<8>{}); break;   case 9: f(CodeTag<9>{}); break;
+        case 10: f(CodeTag<10>{}); break; case 11: f(CodeTag<11>{}); break; default: f(CodeTag<0>{}); break;
+    }
+}
+
+}  // namespace nq

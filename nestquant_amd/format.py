@@ -1,0 +1,225 @@
+"""Plane format of NestQuant expert weights: window-pattern codes, record sizes, sub-array packing, synthetic planes.
+
+Host-side mirror of the format half of the reference's sm120/moe.py (RKP/RK_OF :10-12, rbits :17, step_off :18-20,
+proj_sizes :23-26, pack_words/unpack_words :36-66, Proj :76-107, Expert :177-195). Same names and argument meaning, so
+loaders and tests written against the reference read the same here. Mask mode (nm) and base codes other than 0 are not
+implemented and raise.
+
+Nested levels of this build (the reference serves levels 0/2/4 only): an expert built with nested=True also carries
+P3 (64 bits / record, K=1 windows, code 10) with block words d3, and P4 (64 bits / record) with block words d4n. Level 3
+decodes base + P3; nested level 4 decodes base + the 128-bit record P3 || P4 read with K=2 windows (code 11). In device
+memory P4's uint2 sub-array follows P3's, so promotion 3 -> 4 uploads only P4 and d4n.
+"""
+import torch
+
+TBL_W = 20
+# window-pattern code -> (KA, MASK): step p carries KA + ((MASK >> (p % 16)) & 1) bits
+RKP = {0: (2, 0), 1: (1, 0xEEEE), 2: (2, 0xAAAA), 3: (2, 0x8888), 4: (3, 0), 5: (1, 0xAAAA), 6: (1, 0xFFFE),
+       7: (2, 0x9248), 8: (1, 0xFEFE), 9: (2, 0xD5AA), 10: (1, 0), 11: (2, 0)}
+RK_OF = {2: 0, 1.75: 1, 2.5: 2, 2.25: 3, 3: 4, 1.5: 5, 1.9375: 6, 2.3125: 7, 1.875: 8, 2.5625: 9}
+CODE_L3, CODE_L4N = 10, 11
+
+
+def popc(m):
+    return bin(m).count("1")
+
+
+def rbits(rk):
+    ka, mask = RKP[rk]
+    return 4 * (16 * ka + popc(mask))
+
+
+def step_off(p, KA, MASK):
+    per = [sum(KA + ((MASK >> i) & 1) for i in range(r)) for r in range(16)]
+    p = torch.as_tensor(p)
+    return (p >> 4) * (16 * KA + popc(MASK)) + torch.tensor(per, device=p.device)[p & 15]
+
+
+def split_bits(bits):
+    """(#uint4, uint2?, uint?, ushort?, tail bits) of a record of `bits` bits"""
+    rem = bits % 128
+    return bits // 128, rem // 64, (rem % 64) // 32, (rem % 32) // 16, bits % 16
+
+
+def proj_sizes(N, K, nm=None, rk=0, bk=0):
+    """bytes per plane of a projection [N, K]; nm (mask mode) is not implemented"""
+    if nm is not None:
+        raise NotImplementedError("mask mode (nm) is not implemented")
+    S, C = N // 16, K // 128
+    pad = lambda code: 4 if rbits(code) % 16 else 0
+    return dict(S=S, C=C, nm=None, rk=rk, bk=bk, base=S * C * 32 * rbits(bk) // 8 + pad(bk),
+                p4=S * C * 32 * rbits(rk) // 8 + pad(rk), d4=S * C * 4, flags=0, nrec_r=S * C * 32,
+                p3=S * C * 32 * 8, d3=S * C * 4)
+
+
+def _bytes_le(t, nb):
+    return torch.stack([(t >> (8 * i)) & 255 for i in range(nb)], -1).to(torch.uint8).reshape(-1)
+
+
+def pack_words(w, bits):
+    """w [nrec, NW] int64 (uint32 values) -> int32 tensor in the sub-array layout uint4 x n4 | uint2 | uint | ushort |
+    tail (bits % 16 bits per record, bit-packed over records, + 4 bytes of padding)"""
+    n4, n2, n1, nh, T = split_bits(bits)
+    parts, k = [], 0
+    if n4:
+        parts.append(_bytes_le(w[:, :4 * n4], 4)); k = 4 * n4
+    if n2:
+        parts.append(_bytes_le(w[:, k:k + 2], 4)); k += 2
+    if n1:
+        parts.append(_bytes_le(w[:, k], 4)); k += 1
+    if nh:
+        parts.append(_bytes_le(w[:, k] & 0xFFFF, 2))
+    if T:
+        a = bits - T
+        t = (w[:, a // 32] >> (a % 32)) & ((1 << T) - 1)
+        b = ((t[:, None] >> torch.arange(T, device=w.device)) & 1).reshape(-1)
+        b = torch.cat([b, torch.zeros(32, dtype=b.dtype, device=w.device)])
+        b = b[: b.numel() // 8 * 8].view(-1, 8)
+        parts.append((b << torch.arange(8, device=w.device)).sum(1).to(torch.uint8))
+    return torch.cat(parts).view(torch.int32)
+
+
+def unpack_words(t, nrec, bits):
+    """inverse of pack_words -> [nrec, NW] int64 (uint32 values)"""
+    n4, n2, n1, nh, T = split_bits(bits)
+    dev = t.device
+    b = t.contiguous().view(torch.uint8).long()
+    w = torch.zeros(nrec, (bits + 31) // 32, dtype=torch.int64, device=dev)
+    pos = 0
+
+    def take(nwords, nb):
+        nonlocal pos
+        x = b[pos:pos + nrec * nwords * nb].view(nrec, nwords, nb)
+        pos += nrec * nwords * nb
+        return (x << (8 * torch.arange(nb, device=dev))).sum(-1)
+
+    k = 0
+    if n4:
+        w[:, :4 * n4] = take(4 * n4, 4); k = 4 * n4
+    if n2:
+        w[:, k:k + 2] = take(2, 4); k += 2
+    if n1:
+        w[:, k] = take(1, 4)[:, 0]; k += 1
+    if nh:
+        w[:, k] = take(1, 2)[:, 0]
+    if T:
+        a = bits - T
+        bb = b[pos:pos + (nrec * T + 7) // 8]
+        bit = ((bb[:, None] >> torch.arange(8, device=dev)) & 1).reshape(-1)[: nrec * T].view(nrec, T)
+        w[:, a // 32] |= (bit << torch.arange(T, device=dev)).sum(-1) << (a % 32)
+    return w
+
+
+_MBN = None
+
+
+def all_MbN():
+    """every valid block word (Mb, N): 1 <= Mb <= 255, 0 <= N <= 255, Mb + N <= 257"""
+    global _MBN
+    if _MBN is None:
+        _MBN = torch.tensor([(m, n) for m in range(1, 256) for n in range(0, min(255, 257 - m) + 1)])
+    return _MBN
+
+
+def _block_words(nb, gen, mbn, dev):
+    """'rand': realistic delta = N / Mb ~ 0.1-0.8 plus 5% random extremes; ('exh', offset): cycle through all_MbN()"""
+    if mbn == "rand":
+        kw = dict(generator=gen, device=dev)
+        Mb = torch.randint(120, 256, (nb,), **kw)
+        Nn = (torch.rand(nb, **kw) * 0.8 * Mb).round().long()
+        ext = torch.rand(nb, **kw) < 0.05
+        Mb2 = torch.randint(1, 256, (nb,), **kw)
+        N2 = (torch.rand(nb, **kw) * (torch.clamp(257 - Mb2, max=255) + 1)).floor().long()
+        Mb = torch.where(ext, Mb2, Mb)
+        Nn = torch.minimum(torch.where(ext, N2, Nn), 257 - Mb)
+    else:
+        L = all_MbN().to(dev)
+        idx = (torch.arange(nb, device=dev) + mbn[1]) % len(L)
+        Mb, Nn = L[idx, 0], L[idx, 1]
+    return Mb, Nn
+
+
+class Proj:
+    """Random packed planes of one projection of one expert, each plane its own tensor so it can live in a pool.
+    base int32 [nrec*4]; p4 int32 (packed sub-arrays of residual code rk), d4 int32 (Mb | N << 8 per unit);
+    nested=True adds p3 / d3 and p4n / d4n (int32, uint2 per record) drawn after everything else, so the other planes
+    do not depend on it. The draws before that follow the reference's order (sm120/moe.py:80-103), so a CPU generator
+    with the same seed yields the same planes as the reference's Proj."""
+
+    def __init__(s, N, K, gen, nm=None, rk=0, mbn="rand", var=False, bk=0, nested=False):
+        if nm is not None or bk != 0:
+            raise NotImplementedError("mask mode and base codes other than 0 are not implemented")
+        dev = gen.device
+        z = proj_sizes(N, K, None, rk, bk)
+        s.z, s.N, s.K, s.rk, s.bk, s.nested = z, N, K, rk, bk, nested
+        S, C = z["S"], z["C"]
+        nr, nb = S * C * 32, S * C
+        bits = rbits(rk); nw = (bits + 31) // 32
+        s.base = torch.randint(-2**31, 2**31 - 1, (nr * 4,), generator=gen, dtype=torch.int32, device=dev)
+        w = torch.randint(0, 2**32, (nr, nw), generator=gen, dtype=torch.int64, device=dev)
+        if bits % 32:
+            w[:, -1] &= (1 << (bits % 32)) - 1
+        s.p4w, s.p4 = w, pack_words(w, bits)
+        s.Mb, s.Nn = _block_words(nb, gen, mbn, dev)
+        s.d4 = (s.Mb | (s.Nn << 8)).to(torch.int32)
+        s.var = torch.randint(0, 256, (nb,), generator=gen, dtype=torch.int64, device=dev).to(torch.uint8) if var else None
+        s.flags = s.fl = None
+        s.p3 = s.d3 = s.p4n = s.d4n = s.p3w = s.p4nw = None
+        if nested:
+            s.p3w = torch.randint(0, 2**32, (nr, 2), generator=gen, dtype=torch.int64, device=dev)
+            s.p4nw = torch.randint(0, 2**32, (nr, 2), generator=gen, dtype=torch.int64, device=dev)
+            s.p3, s.p4n = pack_words(s.p3w, 64), pack_words(s.p4nw, 64)
+            s.Mb3, s.N3 = _block_words(nb, gen, "rand", dev)
+            s.Mb4n, s.N4n = _block_words(nb, gen, "rand", dev)
+            s.d3 = (s.Mb3 | (s.N3 << 8)).to(torch.int32)
+            s.d4n = (s.Mb4n | (s.N4n << 8)).to(torch.int32)
+
+    _TENSORS = ["base", "p4", "d4", "p4w", "Mb", "Nn", "var", "p3", "d3", "p4n", "d4n", "p3w", "p4nw"]
+
+    def to(s, dev):
+        for k in s._TENSORS:
+            if getattr(s, k, None) is not None:
+                setattr(s, k, getattr(s, k).to(dev))
+        return s
+
+    def drop_host_words(s):
+        """free the unpacked word tensors (only tests need them)"""
+        s.p4w = s.p3w = s.p4nw = None
+        return s
+
+    def nested_plane(s):
+        """device layout of the nested two-plane record: P3's uint2 sub-array followed by P4's"""
+        return torch.cat([s.p3, s.p4n])
+
+
+class Expert:
+    """Synthetic expert: gate|up [2I, H] and down [H, I] planes + fp16 sign vector
+    [H su_g | I sv_g | I sv_u | I su_d | H sv_o | H su_u] (reference sm120/moe.py:177-183)."""
+
+    def __init__(s, H, I, seed, nm_gu=None, nm_dn=None, dev="cuda", rk_gu=0, rk_dn=0, mbn="rand", var=False,
+                 bk_gu=0, bk_dn=0, nested=False, gen_dev="cpu"):
+        gen = torch.Generator(device=gen_dev).manual_seed(seed)
+        mbn_dn = mbn if mbn == "rand" else ("exh", mbn[1] + (2 * I // 16) * (H // 128))
+        s.gu = Proj(2 * I, H, gen, nm_gu, rk_gu, mbn, var, bk_gu, nested).to(dev)
+        s.dn = Proj(H, I, gen, nm_dn, rk_dn, mbn_dn, var, bk_dn, nested).to(dev)
+        sg = torch.randint(0, 2, (2 * H + 3 * I,), generator=gen, device=gen_dev) * 2 - 1
+        su_u = torch.randint(0, 2, (H,), generator=gen, device=gen_dev) * 2 - 1
+        s.signs = torch.cat([sg, su_u]).half().to(dev)
+        s.H, s.I, s.nested = H, I, nested
+        s.lr = s.lr4 = None
+        s.rg = s.rd = 0
+        if nested:                                       # slot image: [P3 | P4] per projection, contiguous
+            s.gu.slot = s.gu.nested_plane(); s.dn.slot = s.dn.nested_plane()
+
+    def bytes(s, level):
+        """plane bytes a layer call reads for this expert at `level` (the reference's GB/s numerator, sm120/moe.py:190-195)"""
+        b = 0
+        for p in (s.gu, s.dn):
+            b += p.base.numel() * 4 + (0 if p.var is None else p.var.numel())
+            if level == 3:
+                b += (p.p3.numel() + p.d3.numel()) * 4
+            elif level >= 4 and s.nested:
+                b += (p.p3.numel() + p.p4n.numel() + p.d4n.numel()) * 4
+            elif level >= 4:
+                b += (p.p4.numel() + p.d4.numel()) * 4
+        return b

@@ -1,0 +1,100 @@
+"""Writes the golden fixtures of tests/golden/ by running the REFERENCE's own CPU decoder once, in the build container.
+
+Run only where /root/reference exists:   python tests/golden/make_fixtures.py
+It imports sm120/ref15_spec.py (numpy only) and sm120/moe.py (torch CPU; its `build` import is replaced by an empty
+stub the way the reference's own sm120/verify_res2.py:9-15 does) and stores inputs + outputs as small .npz files.
+The fixtures pin what closed forms cannot: lane-minor ring concatenation, bit order of the ring streams, the dense
+row/column scatter, sub-array order and tail packing, the gate|up row order, and the layer math conventions.
+Nothing here is read at test time except the .npz files it wrote.
+"""
+import os
+import sys
+import types
+
+import numpy as np
+import torch
+
+REF = "/root/reference/sm120"
+OUT = os.path.dirname(os.path.abspath(__file__))
+
+
+def main():
+    sys.modules["build"] = types.SimpleNamespace(get=lambda *a, **k: None, get_sal=lambda *a, **k: None)
+    sys.path.insert(0, REF)
+    import moe as R          # reference torch decoder (CPU)
+    import ref15_spec as SP  # reference numpy bit-level spec
+    # The reference's Proj.to() reads s.bw, which Proj.__init__ only sets for base codes != 0 (sm120/moe.py:84-88,105);
+    # a class-level default lets its Expert constructor run for the K=2 base used everywhere here.
+    R.Proj.bw = None
+
+    # 1. projections: planes from the reference generator, dense decode by the reference at levels 2 and 4
+    for rk in (0, 3, 6, 7, 8, 9):
+        for var in (False, True):
+            if var and rk not in (0, 7):
+                continue
+            seed = 1000 + 10 * rk + int(var)
+            gen = torch.Generator().manual_seed(seed)
+            p = R.Proj(32, 256, gen, None, rk, ("exh", 4000 * rk + 17), var=var)
+            W2 = R.dense_W(p, 2, 4, torch.float16)
+            W4 = R.dense_W(p, 4, 4, torch.float16)
+            np.savez_compressed(
+                os.path.join(OUT, f"proj_rk{rk}_var{int(var)}.npz"), seed=seed, N=32, K=256, rk=rk,
+                mbn_offset=4000 * rk + 17, base=p.base.numpy(), p4=p.p4.numpy(), d4=p.d4.numpy(),
+                var=(p.var.numpy() if var else np.zeros(0, np.uint8)),
+                W2=W2.numpy().view(np.uint16), W4=W4.numpy().view(np.uint16))
+
+    # 2. nested levels through the reference's generic (KA, MASK) decoder: K=1 plane, and K=2 over P3 || P4
+    rng = np.random.default_rng(7)
+    units = []
+    for u in range(4):
+        base = rng.integers(0, 2**32, (32, 4), dtype=np.uint64).astype(np.uint32)
+        p3 = rng.integers(0, 2**32, (32, 2), dtype=np.uint64).astype(np.uint32)
+        p4 = rng.integers(0, 2**32, (32, 2), dtype=np.uint64).astype(np.uint32)
+        Mb3, N3 = int(rng.integers(1, 256)), 0
+        N3 = int(rng.integers(0, min(255, 257 - Mb3) + 1))
+        Mb4 = int(rng.integers(120, 256)); N4 = int(rng.integers(0, 257 - Mb4 + 1))
+        bs = SP.rings_from_lane_words(base, 128)
+        r3 = SP.rings_from_lane_words(p3, 64)
+        r4 = SP.rings_from_lane_words(np.concatenate([p3, p4], 1), 128)
+        Q2, Q3 = SP.decode_unit(bs, r3, Mb3, N3, Kb=2, Kr=(1, 0))
+        _, Q4 = SP.decode_unit(bs, r4, Mb4, N4, Kb=2, Kr=2)
+        units.append(dict(base=base, p3=p3, p4=p4, d3=Mb3 | N3 << 8, d4=Mb4 | N4 << 8,
+                          U2=SP.to_unit(Q2).T.astype(np.float16).view(np.uint16),      # [16 rows, 128 cols]
+                          U3=SP.to_unit(Q3).T.astype(np.float16).view(np.uint16),
+                          U4=SP.to_unit(Q4).T.astype(np.float16).view(np.uint16)))
+    np.savez_compressed(os.path.join(OUT, "nested_units.npz"),
+                        **{k: np.stack([np.asarray(u[k]) for u in units]) for k in units[0]})
+
+    # 3. layer math: reference Expert.ref / moe_ref on CPU (H = I = 256, 4 experts, levels 2/4/4/0, var on expert 2)
+    H = I = 256
+    ex = [R.Expert(H, I, seed=300 + i, dev="cpu", rk_gu=(0, 3, 7, 0)[i], rk_dn=(0, 7, 0, 0)[i], var=(i == 2)) for i in range(4)]
+    levels = [2, 4, 4, 0]
+    g = torch.Generator().manual_seed(5)
+    x = (torch.randn(3, H, generator=g) * 0.05).half()
+    sel = torch.tensor([[0, 1, 2, 3], [2, 0, 1, 3], [1, 2, 0, 3]])
+    rw = (torch.rand(3, 4, generator=g) + 0.1)
+    rw = (rw / rw.sum(1, keepdim=True)).half()
+    rw[2, 1] = 0                                                     # a pick with zero weight is skipped
+    y = R.moe_ref(ex, levels, x, sel, rw)
+    y1 = ex[1].ref(x.float(), 4)
+    np.savez_compressed(os.path.join(OUT, "layer_small.npz"), H=H, I=I, seeds=np.arange(300, 304), levels=np.array(levels),
+                        rk_gu=np.array([0, 3, 7, 0]), rk_dn=np.array([0, 7, 0, 0]), var=np.array([0, 0, 1, 0]),
+                        x=x.numpy().view(np.uint16), sel=sel.numpy(), rw=rw.numpy().view(np.uint16),
+                        y=y.numpy(), y_expert1_level4=y1.numpy(), signs1=ex[1].signs.numpy().view(np.uint16))
+
+    # 4. the reference's residual packer on every code (sub-array order and tail bits)
+    g = torch.Generator().manual_seed(0)
+    packs = {}
+    for c in range(10):
+        b = R.rbits(c); nw = (b + 31) // 32
+        w = torch.randint(0, 2**32, (96, nw), generator=g, dtype=torch.int64)
+        if b % 32:
+            w[:, -1] &= (1 << (b % 32)) - 1
+        packs[f"w{c}"] = w.numpy().astype(np.uint32)
+        packs[f"p{c}"] = R.pack_words(w, b).numpy()
+    np.savez_compressed(os.path.join(OUT, "pack_words.npz"), **packs)
+    print("fixtures written to", OUT)
+
+
+if __name__ == "__main__":
+    main()

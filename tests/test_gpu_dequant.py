@@ -1,0 +1,137 @@
+"""HIP decoder (nq_dequant / nq_pf_decode through the C ABI) against the oracle and the golden fixtures: bit-exact fp16,
++0 and -0 identified (the reference's own rule, sm120/verify_ext.py:55)."""
+import glob
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from nestquant_amd import _lib, format as F, moe as M
+from oracle import nq_oracle as O
+from tests.util import oracle_plane, same_f16
+
+pytestmark = pytest.mark.gpu
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+DEV = "cuda"
+
+
+class _Ex:
+    """duck-typed expert with one real projection (the other side is a tiny dummy) for single-projection decodes"""
+
+    def __init__(s, p, mode, H, I):
+        s.H, s.I, s.nested = H, I, p.nested
+        s.gu = s.dn = p
+        s.signs = torch.zeros(8, dtype=torch.float16, device=DEV)
+        s.mode = mode
+        s.lr = None
+
+
+def gpu_dense(p, level, N, K, mode=0):
+    """decode projection p (already on the device) as gate|up (mode 0: N = 2I, K = H) or down (mode 1)"""
+    H, I = (K, N // 2) if mode == 0 else (N, K)
+    ex = _Ex(p, mode, H, I)
+    if p.nested:
+        p.slot = p.nested_plane()
+    row = M.entry(ex, level)
+    M.validate_row(row, 128, 128)                                 # field checks only; a lone projection may be small
+    W = M.dequant(row.to(DEV), mode, H, I)
+    torch.cuda.synchronize()
+    return W.cpu().numpy()
+
+
+@pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(GOLD, "proj_rk*_var*.npz"))), ids=lambda p: os.path.basename(p)[:-4])
+def test_golden_projections(path):
+    z = np.load(path)
+    gen = torch.Generator().manual_seed(int(z["seed"]))
+    p = F.Proj(int(z["N"]), int(z["K"]), gen, None, int(z["rk"]), ("exh", int(z["mbn_offset"])), var=bool(z["var"].size)).to(DEV)
+    for mode in (0, 1):
+        assert same_f16(gpu_dense(p, 2, p.N, p.K, mode), z["W2"].view(np.float16)) == 0
+        assert same_f16(gpu_dense(p, 4, p.N, p.K, mode), z["W4"].view(np.float16)) == 0
+
+
+def test_golden_nested_units():
+    z = np.load(os.path.join(GOLD, "nested_units.npz"))
+    n = z["base"].shape[0]
+    gen = torch.Generator().manual_seed(0)
+    p = F.Proj(16, 128 * n, gen, nested=True)
+    p.base = torch.from_numpy(z["base"].reshape(-1).view(np.int32).copy())
+    p.p3 = F.pack_words(torch.from_numpy(z["p3"].reshape(-1, 2).astype(np.int64)), 64)
+    p.p4n = F.pack_words(torch.from_numpy(z["p4"].reshape(-1, 2).astype(np.int64)), 64)
+    p.d3 = torch.from_numpy(z["d3"].astype(np.int32)); p.d4n = torch.from_numpy(z["d4"].astype(np.int32))
+    p.to(DEV)
+    for lv, key in ((2, "U2"), (3, "U3"), (4, "U4")):
+        W = gpu_dense(p, lv, 16, 128 * n, mode=1)
+        for u in range(n):
+            assert same_f16(W[:, 128 * u:128 * (u + 1)], z[key][u].view(np.float16)) == 0, (lv, u)
+
+
+@pytest.mark.parametrize("rk", range(10))
+@pytest.mark.parametrize("var", [False, True])
+def test_every_residual_code(rk, var):
+    """4 strips x 4 chunks as the reference's verify_ext.py (a): every code, sign planes on and off"""
+    gen = torch.Generator().manual_seed(rk)
+    p = F.Proj(64, 512, gen, None, rk, ("exh", rk * 1000), var=var)
+    op = oracle_plane(p)
+    p.to(DEV)
+    for lv in (2, 4):
+        assert same_f16(gpu_dense(p, lv, 64, 512, mode=rk % 2), O.dense_W(op, lv)) == 0, (rk, var, lv)
+
+
+def test_exhaustive_block_words():
+    """every one of the 33149 valid (Mb, N) words goes through the device's constant computation"""
+    seen = set()
+    for i in range(17):
+        gen = torch.Generator().manual_seed(900 + i)
+        p = F.Proj(2048, 2048, gen, None, 0, ("exh", i * 2048))
+        seen |= set((p.Mb * 256 + p.Nn).tolist())
+        op = oracle_plane(p)
+        p.to(DEV)
+        assert same_f16(gpu_dense(p, 4, 2048, 2048, mode=1), O.dense_W(op, 4)) == 0, i
+    assert len(seen) == 33149
+
+
+def test_odd_unit_count_and_level0():
+    gen = torch.Generator().manual_seed(5)
+    p = F.Proj(48, 128, gen, None, 3, "rand", var=True)          # 3 units: the last wave decodes a single unit
+    op = oracle_plane(p); p.to(DEV)
+    assert same_f16(gpu_dense(p, 4, 48, 128, mode=1), O.dense_W(op, 4)) == 0
+    assert same_f16(gpu_dense(p, 2, 48, 128, mode=1), O.dense_W(op, 2)) == 0
+    ex = _Ex(p, 1, 48, 128)
+    row = M.entry(ex, 0).to(DEV)
+    out = torch.full((48, 128), float("nan"), dtype=torch.float16, device=DEV)
+    M.dequant(row, 1, 48, 128, out=out)
+    assert not out.any()                                          # level 0 decodes to zeros
+
+
+def test_full_shape_nested_expert_and_pf_decode():
+    """one full-size expert (H 6144, I 2048) at levels 2/3/4 and the multi-expert prefill decode on top of it"""
+    H, I = 6144, 2048
+    ex = F.Expert(H, I, seed=77, dev="cpu", nested=True)
+    og, od = oracle_plane(ex.gu), oracle_plane(ex.dn)
+    for p in (ex.gu, ex.dn):
+        p.to(DEV); p.slot = p.nested_plane()
+    ex.signs = ex.signs.to(DEV)
+    want = {}
+    for lv in (2, 3, 4):
+        want[lv] = (O.dense_W(og, lv, nested=True), O.dense_W(od, lv, nested=True))
+        assert same_f16(M.dense_W(ex, 0, lv).cpu().numpy(), want[lv][0]) == 0, lv
+        assert same_f16(M.dense_W(ex, 1, lv).cpu().numpy(), want[lv][1]) == 0, lv
+    table = torch.stack([M.entry(ex, lv) for lv in (4, 0, 2, 3)]).to(DEV)
+    ids = torch.tensor([3, 1, 0], dtype=torch.int32, device=DEV)
+    Wgu = torch.empty(3, 2 * I, H, dtype=torch.float16, device=DEV); Wdn = torch.empty(3, H, I, dtype=torch.float16, device=DEV)
+    _lib.check(_lib.lib().nq_pf_decode(table.data_ptr(), ids.data_ptr(), 3, Wgu.data_ptr(), Wdn.data_ptr(), H, I,
+                                       _lib.stream_ptr()))
+    torch.cuda.synchronize()
+    assert same_f16(Wgu[0].cpu().numpy(), want[3][0]) == 0 and same_f16(Wdn[0].cpu().numpy(), want[3][1]) == 0
+    assert not Wgu[1].any() and not Wdn[1].any()
+    assert same_f16(Wgu[2].cpu().numpy(), want[4][0]) == 0 and same_f16(Wdn[2].cpu().numpy(), want[4][1]) == 0
+
+
+def test_bad_arguments_raise():
+    row = torch.zeros(F.TBL_W, dtype=torch.int64, device=DEV)
+    out = torch.empty(256, 256, dtype=torch.float16, device=DEV)
+    with pytest.raises(RuntimeError, match="whole 16x128 units"):
+        M.dequant(row, 0, 100, 128, out=out)
+    with pytest.raises(RuntimeError, match="proj"):
+        _lib.check(_lib.lib().nq_dequant(row.data_ptr(), 2, 0, 128, 128, out.data_ptr(), None))

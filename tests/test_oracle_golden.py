@@ -1,0 +1,111 @@
+"""Oracle and host format code against the golden fixtures written by tests/golden/make_fixtures.py
+(outputs of the reference's own CPU decoder: sm120/moe.py dense_W / Expert.ref / moe_ref / pack_words and
+sm120/ref15_spec.py decode_unit). CPU only."""
+import glob
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from nestquant_amd import format as F
+from oracle import nq_oracle as O
+from tests.util import oracle_plane, rel_err, same_f16, u32
+
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+PROJ_FILES = sorted(glob.glob(os.path.join(GOLD, "proj_rk*_var*.npz")))
+
+
+def test_fixture_inventory():
+    assert len(PROJ_FILES) == 8
+    for f in ("nested_units.npz", "layer_small.npz", "pack_words.npz"):
+        assert os.path.exists(os.path.join(GOLD, f))
+
+
+@pytest.mark.parametrize("path", PROJ_FILES, ids=[os.path.basename(p)[:-4] for p in PROJ_FILES])
+def test_dense_decode_matches_reference(path):
+    z = np.load(path)
+    N, K, rk = int(z["N"]), int(z["K"]), int(z["rk"])
+    nrec = (N // 16) * (K // 128) * 32
+    var = z["var"] if z["var"].size else None
+    res = O.unpack_words(z["p4"], nrec, O.rbits(rk))
+    p = O.Plane(N, K, u32(torch.from_numpy(z["base"])).reshape(-1, 4), rk=rk, res=res, d4=u32(torch.from_numpy(z["d4"])), var=var)
+    W2 = O.dense_W(p, 2); W4 = O.dense_W(p, 4)
+    assert same_f16(W2, z["W2"].view(np.float16)) == 0
+    assert same_f16(W4, z["W4"].view(np.float16)) == 0
+    # a decoder that ignored the residual plane, or the sign plane, must not pass by accident
+    assert same_f16(W2, z["W4"].view(np.float16)) > 1000
+    if var is not None:
+        q = O.Plane(N, K, p.base, rk=rk, res=res, d4=p.d4, var=None)
+        assert same_f16(O.dense_W(q, 2), z["W2"].view(np.float16)) > 1000
+
+
+@pytest.mark.parametrize("path", PROJ_FILES, ids=[os.path.basename(p)[:-4] for p in PROJ_FILES])
+def test_package_generator_reproduces_reference_planes(path):
+    """nestquant_amd.format.Proj draws in the reference's order: same seed -> same planes, block words and signs"""
+    z = np.load(path)
+    gen = torch.Generator().manual_seed(int(z["seed"]))
+    p = F.Proj(int(z["N"]), int(z["K"]), gen, None, int(z["rk"]), ("exh", int(z["mbn_offset"])), var=bool(z["var"].size))
+    assert np.array_equal(p.base.numpy(), z["base"]) and np.array_equal(p.p4.numpy(), z["p4"])
+    assert np.array_equal(p.d4.numpy(), z["d4"])
+    if z["var"].size:
+        assert np.array_equal(p.var.numpy(), z["var"])
+    assert p.p4.numel() * 4 == F.proj_sizes(p.N, p.K, None, p.rk)["p4"]
+
+
+def test_pack_words_matches_reference():
+    z = np.load(os.path.join(GOLD, "pack_words.npz"))
+    for c in range(10):
+        w = z[f"w{c}"]; want = z[f"p{c}"]
+        bits = O.rbits(c)
+        assert np.array_equal(O.pack_words(w, bits).view(np.int32), want)
+        got = F.pack_words(torch.from_numpy(w.astype(np.int64)), bits)
+        assert np.array_equal(got.numpy(), want)
+        assert np.array_equal(F.unpack_words(torch.from_numpy(want), 96, bits).numpy().astype(np.uint32), w)
+        assert np.array_equal(O.unpack_words(want, 96, bits), w)
+
+
+def test_nested_levels_match_reference_generic_decoder():
+    """level 3 (K=1 plane) and nested level 4 (K=2 over P3 || P4) through the reference's decode_unit(Kr=(KA, MASK))"""
+    z = np.load(os.path.join(GOLD, "nested_units.npz"))
+    n = z["base"].shape[0]
+    base = z["base"].reshape(n * 32, 4); p3 = z["p3"].reshape(n * 32, 2); p4 = z["p4"].reshape(n * 32, 2)
+    p = O.Plane(16, 128 * n, base, p3=p3, d3=z["d3"].astype(np.uint32), p4n=p4, d4n=z["d4"].astype(np.uint32))
+    for lv, key in ((2, "U2"), (3, "U3"), (4, "U4")):
+        W = O.dense_W(p, lv, nested=True)
+        for u in range(n):
+            assert same_f16(W[:, 128 * u:128 * (u + 1)], z[key][u].view(np.float16)) == 0, (lv, u)
+    assert same_f16(O.dense_W(p, 3, nested=True), O.dense_W(p, 4, nested=True)) > 1000
+
+
+def _small_layer():
+    z = np.load(os.path.join(GOLD, "layer_small.npz"))
+    H, I = int(z["H"]), int(z["I"])
+    ex = [F.Expert(H, I, seed=int(z["seeds"][i]), dev="cpu", rk_gu=int(z["rk_gu"][i]), rk_dn=int(z["rk_dn"][i]),
+                   var=bool(z["var"][i])) for i in range(4)]
+    return z, H, I, ex
+
+
+def test_expert_and_layer_math_match_reference():
+    z, H, I, ex = _small_layer()
+    levels = z["levels"].tolist()
+    assert np.array_equal(ex[1].signs.numpy().view(np.uint16), z["signs1"])
+    x = z["x"].view(np.float16); rw = z["rw"].view(np.float16); sel = z["sel"]
+
+    def dense(e):
+        return (O.dense_W(oracle_plane(ex[e].gu), levels[e]).astype(np.float32),
+                O.dense_W(oracle_plane(ex[e].dn), levels[e]).astype(np.float32))
+
+    y1 = O.expert_forward(x.astype(np.float32), *dense(1), ex[1].signs.numpy())
+    assert rel_err(y1, z["y_expert1_level4"]) < 2e-6
+    y = O.moe_forward(dense, levels, lambda e: ex[e].signs.numpy(), x, sel, rw)
+    # row-by-row and batched fp32 matmuls differ in summation order; where that flips one of the fp16 activation
+    # roundings an element moves by one fp16 ulp, so the layer bar is the reference's own kernel-vs-ref band (<= 1e-4)
+    assert rel_err(y, z["y"]) < 1e-4
+    # sensitivity: dropping the zero-weight rule or the level-0 rule, or swapping gate and up, must fail this bar
+    Wgu, Wdn = dense(1)
+    swapped = np.concatenate([Wgu[I:], Wgu[:I]])
+    assert rel_err(O.expert_forward(x.astype(np.float32), swapped, Wdn, ex[1].signs.numpy()), z["y_expert1_level4"]) > 1e-2
+    # distance to the pipeline without the two fp16 activation roundings stays inside the 1e-3 budget
+    y_pure = O.moe_forward(dense, levels, lambda e: ex[e].signs.numpy(), x, sel, rw, round_acts=False)
+    assert 0 < rel_err(y, y_pure) < 1e-3
