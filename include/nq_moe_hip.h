@@ -46,6 +46,37 @@ int nq_dequant(const int64_t* row, int proj, int level, int H, int I, void* out_
 int nq_pf_decode(const int64_t* table, const int32_t* experts, int G, void* Wgu_f16, void* Wdn_f16, int H, int I,
                  void* stream);
 
+/* One decode-path MoE layer call, B <= 8 tokens, B * topk <= 64 picks (reference moe_forward, sm120/nqmoe.cu:858-907).
+ * cfg = {cpw, sb, nst, 0}: k-slice = cpw * nst chunks of 128 columns per block, sb wavefronts per block (each wavefront
+ * decodes two 16-row strips), as the reference's {chunks per warp, warps per block, stages}. Workspaces hold k-slice
+ * partial sums (no atomics, no zero-on-entry contract): acc_gu >= (H/128/(cpw*nst)) * B*topk * 2I floats,
+ * acc_d >= (I/128/(cpw*nst)) * B*topk * H floats, h >= B*topk * I halfs. Picks with rw == 0, level <= 0 or an expert id
+ * outside [0, E) contribute nothing. which: bit 0 = gate|up launches, bit 1 = down launches. hits: optional int32[E]
+ * pick counters (device or host-mapped memory), incremented once per pick with rw != 0 (reference :784-787). */
+typedef struct NqMoeArgs
+{
+    const void* x;            /* fp16 [B][H] */
+    const int64_t* sel;       /* int64 [B][topk] */
+    const void* rw;           /* fp16 [B][topk] */
+    const int64_t* table;     /* int64 [E][NQ_TBL_W] */
+    void* out;                /* fp32 [B][H] */
+    void* acc_gu;             /* fp32 workspace */
+    void* h;                  /* fp16 workspace */
+    void* acc_d;              /* fp32 workspace */
+    int32_t* hits;            /* optional, may be NULL */
+    int64_t acc_gu_elems, acc_d_elems, h_elems, out_elems;   /* capacities, checked against the shapes above */
+    int32_t B, topk, E, H, I;
+    int32_t cfg_gu[4], cfg_dn[4];
+    int32_t force_level;      /* 0, or a level that overrides every active row's level (debug) */
+    int32_t which;
+} NqMoeArgs;
+int nq_moe_forward(const NqMoeArgs* args, void* stream);
+
+/* table[e] <- stage[e] for every e with seq[e] != applied[e]; then applied[e] <- seq[e], mirrored to applied_host
+ * [host-mapped, optional]. Replaces mailbox (reference sm120/nqmoe.cu:908-929). */
+int nq_mailbox(int64_t* table, const int64_t* stage, const int32_t* seq, int32_t* applied, int32_t* applied_host, int E,
+               void* stream);
+
 #ifdef __cplusplus
 }
 #endif

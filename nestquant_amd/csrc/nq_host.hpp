@@ -20,7 +20,18 @@ inline int set_error(const char* fmt, ...)
 #define NQ_LAUNCH_CHECK(what) do { hipError_t e_ = hipGetLastError(); \
     if (e_ != hipSuccess) return nq::set_error("%s: %s", what, hipGetErrorString(e_)); } while (0)
 
+// arguments of one decode-path layer call (device pointers; see NqMoeArgs in include/nq_moe_hip.h)
+struct MoeArgs
+{
+    const _Float16* x; const int64_t* sel; const _Float16* rw; int B, topk;
+    const int64_t* table; int E, H, I;
+    float* part_gu; _Float16* h; float* part_d; float* out;
+    int force_level; int* hits;
+};
+
 // kernel launchers defined next to their kernels
+int launch_moe(const MoeArgs& a, const int* cfg_gu, const int* cfg_dn, int which, hipStream_t st);
+int launch_mailbox(int64_t* table, const int64_t* stage, const int32_t* seq, int32_t* applied, int32_t* applied_host, int E, hipStream_t st);
 int launch_dequant(const int64_t* row, int proj, int level, int H, int I, void* out, hipStream_t st);
 int launch_pf_decode(const int64_t* table, const int32_t* experts, int G, void* Wgu, void* Wdn, int H, int I, hipStream_t st);
 

@@ -1,0 +1,338 @@
+// Decode-path MoE layer for 1..8 tokens (reference sm120/nqmoe.cu:375-449 route, :493-771 do_item, :858-907 moe_forward,
+// :908-929 mailbox). Four launches on one stream, every routing / level / pointer decision read on the device:
+//
+//   nq_gemv_k<0>  gate|up: grid (strip-pair blocks, k-slices, runs). A run = one distinct routed expert + the tokens that
+//                 picked it. The block rotates those tokens' x (x * su -> Hadamard-128 -> fp16) into LDS, then every
+//                 wavefront decodes the records of two strips chunk by chunk straight into MFMA A operands
+//                 (v_mfma_f32_16x16x32_f16, tokens as the N dimension) and writes its k-slice partial sums.
+//   nq_fin_gu_k   per (slot, 128-column group): sum the k-slice partials, Hadamard * sv, SwiGLU, * su_d, Hadamard -> h fp16.
+//   nq_gemv_k<1>  down: same kernel on h.
+//   nq_fin_dn_k   per (token, 128-row group): out[b] = sum_k rw[b,k] * sv_o (.) Hadamard(sum of partials).
+//
+// Lane mapping of the GEMV (wave64): lane = 16 * t4 + 8 * ss + g decodes the record of lane (4 g + t4) of unit
+// (strip0 + ss, chunk); it holds 32 weights of row g and 32 of row g + 8, in columns 16 t + 2 t4 + {0,1,8,9}. An MFMA
+// 16x16x32 takes 8 fp16 per lane: lanes with equal (ss, g) and different t4 are the k-groups of one A row, so the decoded
+// pairs are A operands as they leave the decoder, with no cross-lane movement. The B operand (tokens) comes from LDS,
+// staged in the matching column order. Partial sums instead of atomics make the layer output bitwise repeatable and
+// need no zeroed workspace.
+#include "nq_decode.hpp"
+#include "nq_host.hpp"
+#include <utility>
+
+namespace nq {
+
+constexpr int MAXTOK = 16;                     // MFMA N: tokens of one run (B <= 8 -> at most 8 with distinct top-k ids)
+struct RunInfo { int e, level, ntok, nruns; int slot[MAXTOK]; const int64_t* ent; };
+
+// ---- routing dedup: picks -> runs, numbered by first occurrence; slots in pick order ---------------------------------
+// called by one full wavefront; lane s owns pick s (S <= 64). Fills run z.
+__device__ __forceinline__ void route(const MoeArgs& a, int z, RunInfo* R, int lane)
+{
+    const int S = a.B * a.topk;
+    int e = -1; bool ok = false;
+    if (lane < S)
+    {
+        const long long ee = a.sel[lane];
+        if (ee >= 0 && ee < a.E)
+        {
+            e = (int)ee;
+            ok = (float)a.rw[lane] != 0.f && a.table[(size_t)e * TBL_W] > 0;
+        }
+    }
+    unsigned long long rem = __ballot(ok);
+    const unsigned long long below = (1ull << lane) - 1ull;
+    int r = 0;
+    while (rem)
+    {
+        const int leader = __ffsll((long long)rem) - 1;
+        const int ev = __shfl(e, leader);
+        const unsigned long long m = __ballot(ok && e == ev);
+        if (r == z && ((m >> lane) & 1ull))
+        {
+            const int pos = __popcll(m & below);
+            if (pos < MAXTOK) R->slot[pos] = lane;
+            if (pos == 0)
+            {
+                R->e = e; R->ent = a.table + (size_t)e * TBL_W;
+                const int lv = (int)R->ent[0];
+                R->level = a.force_level ? a.force_level : lv;
+                const int n = __popcll(m);
+                R->ntok = n < MAXTOK ? n : MAXTOK;
+            }
+        }
+        rem &= ~m; ++r;
+    }
+    if (lane == 0) R->nruns = r;
+}
+
+// ---- Hadamard-128 on one wavefront: lane holds elements 2 lane, 2 lane + 1 --------------------------------------------
+__device__ __forceinline__ void wht128(float& a, float& b, int lane)
+{
+    const float s = a + b, d = a - b; a = s; b = d;
+#pragma unroll
+    for (int m = 1; m < 64; m <<= 1)
+    {
+        const float oa = __shfl_xor(a, m), ob = __shfl_xor(b, m);
+        a = (lane & m) ? oa - a : a + oa;
+        b = (lane & m) ? ob - b : b + ob;
+    }
+    a *= 0.08838834764f; b *= 0.08838834764f;
+}
+
+// LDS position (in halfs) of column c of a 128-column chunk in the B-operand order:
+// 16-byte block (mm, kg) holds, for i = 0..3, columns 32 mm + 2 kg + 8 (i >> 1) + (i & 1) and that + 16
+__device__ __forceinline__ int bop_index(int c)
+{
+    const int mm = c >> 5, hi = (c >> 4) & 1, kg = (c >> 1) & 3, i = 2 * ((c >> 3) & 1) + (c & 1);
+    return (mm * 4 + kg) * 8 + 2 * i + hi;
+}
+
+template <int... Is, class F> __device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, Is...>) { (f(CodeTag<Is>{}), ...); }
+template <int N, class F> __device__ __forceinline__ void static_for(F&& f) { static_for_impl(f, std::make_integer_sequence<int, N>{}); }
+
+// A operand of MFMA (MM, RHO): rows g + 8 RHO, columns of t = 2 MM and 2 MM + 1
+template <bool RES, int CODE, int MM, int RHO>
+__device__ __forceinline__ half8_t a_operand(const uint32_t* wb, const uint32_t* wr, const FoldK& k)
+{
+    constexpr int J = 16 * MM + 2 * RHO;
+    uint32_t u[4];
+    u[0] = weight_pair<RES, CODE, J + 0, J + 8>(wb, wr, k);
+    u[1] = weight_pair<RES, CODE, J + 1, J + 9>(wb, wr, k);
+    u[2] = weight_pair<RES, CODE, J + 4, J + 12>(wb, wr, k);
+    u[3] = weight_pair<RES, CODE, J + 5, J + 13>(wb, wr, k);
+    return __builtin_bit_cast(half8_t, *(uint4*)u);
+}
+
+struct LaneCtx
+{
+    size_t rec0;          // record index of this lane in chunk 0 of its k-slice: (unit0) * 32 + 4 g + t4
+    size_t unit0;         // unit index (strip * C + chunk0)
+    size_t nrec;          // records of the whole projection (sub-array stride)
+    int src;              // lane holding the next record of the ring
+    int g;                // ring index (sign-variant bit)
+    const char* xs;       // this lane's B-operand base in LDS (bytes), kg folded in
+    int xstep;            // bytes per chunk (0 for lanes without a token)
+};
+
+template <bool RES, int CODE>
+__device__ __forceinline__ void gemv_chunks(const Planes& P, const LaneCtx& L, int NC, float4_t* acc)
+{
+    constexpr int NW = RES ? Rec<CODE>::NW : 1;
+    uint4 nb = P.base[L.rec0];
+    uint32_t nr[NW + 2] = {0}, ndw = 0, nvar = 0;
+    if constexpr (RES) { load_record<CODE>(nr, P.res, L.rec0, L.nrec); ndw = P.dw[L.unit0]; }
+    if (P.var) nvar = P.var[L.unit0];
+    for (int c = 0; c < NC; ++c)
+    {
+        uint32_t wb[6], wr[NW + 2];
+        wb[0] = nb.x; wb[1] = nb.y; wb[2] = nb.z; wb[3] = nb.w;
+#pragma unroll
+        for (int i = 0; i < NW; ++i) wr[i] = nr[i];
+        const uint32_t dw = ndw, var = nvar;
+        if (c + 1 < NC)                                         // prefetch the next chunk's records
+        {
+            nb = P.base[L.rec0 + (size_t)(c + 1) * 32];
+            if constexpr (RES) { load_record<CODE>(nr, P.res, L.rec0 + (size_t)(c + 1) * 32, L.nrec); ndw = P.dw[L.unit0 + c + 1]; }
+            if (P.var) nvar = P.var[L.unit0 + c + 1];
+        }
+        ext_words<128, 4>(wb, __shfl(wb[0], L.src));
+        const uint32_t sgm = ((var >> L.g) & 1u) * 0x80008000u;
+        FoldK k;
+        if constexpr (RES)
+        {
+            ext_words<Rec<CODE>::BITS, Rec<CODE>::NW>(wr, __shfl(wr[0], L.src));
+            k = consts_fold(dw, sgm);
+        }
+        else k = consts_l2(sgm);
+        const char* xp = L.xs + c * L.xstep;
+        static_for<4>([&](auto mm) {
+            constexpr int MM = decltype(mm)::value;
+            const half8_t b = *(const half8_t*)(xp + MM * 64);
+            acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_operand<RES, CODE, MM, 0>(wb, wr, k), b, acc[0], 0, 0, 0);
+            acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_operand<RES, CODE, MM, 1>(wb, wr, k), b, acc[1], 0, 0, 0);
+        });
+    }
+}
+
+// MODE 0: gate|up (N = 2I, K = H, input x rotated here). MODE 1: down (N = H, K = I, input h).
+// grid (N / 32 / SB, C / NC, S); block 64 * SB threads; dynamic LDS = ntokmax * (NC * 256 + 16) + 256 bytes
+template <int MODE>
+__global__ void __launch_bounds__(512) nq_gemv_k(MoeArgs a, int NC)
+{
+    extern __shared__ __align__(16) char smem[];
+    __shared__ RunInfo R;
+    const int lane = threadIdx.x & 63, warp = threadIdx.x >> 6, SB = blockDim.x >> 6;
+    if (warp == 0) route(a, blockIdx.z, &R, lane);
+    if (MODE == 0 && a.hits && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x < a.B * a.topk)
+    {
+        const long long ee = a.sel[threadIdx.x];
+        if ((float)a.rw[threadIdx.x] != 0.f && ee >= 0 && ee < a.E)
+            __hip_atomic_fetch_add(a.hits + ee, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+    __syncthreads();
+    if ((int)blockIdx.z >= R.nruns) return;                      // block-uniform
+    const int N = MODE == 0 ? 2 * a.I : a.H, K = MODE == 0 ? a.H : a.I, C = K / 128;
+    const int ntok = R.ntok, chunk0 = blockIdx.y * NC, k0 = chunk0 * 128;
+    const int rowstride = NC * 256 + 16;                         // bytes per staged token (+16: spread tokens over banks)
+    char* zero = smem + ntok * rowstride;                      // 256 zero bytes after the token rows
+    const _Float16* signs = (const _Float16*)R.ent[9];
+
+    // ---- stage the run's tokens for this k-slice in B-operand order
+    if constexpr (MODE == 0)
+    {
+        const bool up = (int)(blockIdx.x * SB * 32) >= a.I;      // gate rows use su_g, up rows su_u
+        const _Float16* su = up ? signs + 2 * a.H + 3 * a.I : signs;
+        for (int task = warp; task < ntok * NC; task += SB)
+        {
+            const int j = task / NC, c = task % NC, kk = k0 + c * 128 + 2 * lane;
+            const int tok = R.slot[j] / a.topk;
+            const half2_t xv = *(const half2_t*)(a.x + (size_t)tok * a.H + kk), sv = *(const half2_t*)(su + kk);
+            float v0 = (float)xv.x * (float)sv.x, v1 = (float)xv.y * (float)sv.y;
+            wht128(v0, v1, lane);
+            _Float16* dst = (_Float16*)(smem + j * rowstride + c * 256);
+            dst[bop_index(2 * lane)] = (_Float16)v0; dst[bop_index(2 * lane + 1)] = (_Float16)v1;
+        }
+    }
+    else
+    {
+        for (int i = threadIdx.x; i < ntok * NC * 64; i += blockDim.x)
+        {
+            const int j = i / (NC * 64), r = i % (NC * 64), c = r >> 6, p = r & 63;
+            const half2_t hv = *(const half2_t*)(a.h + (size_t)R.slot[j] * a.I + k0 + c * 128 + 2 * p);
+            _Float16* dst = (_Float16*)(smem + j * rowstride + c * 256);
+            dst[bop_index(2 * p)] = hv.x; dst[bop_index(2 * p + 1)] = hv.y;
+        }
+    }
+    if (threadIdx.x < 64) ((uint32_t*)zero)[threadIdx.x] = 0u;
+    __syncthreads();
+
+    // ---- decode + MFMA over the k-slice
+    const int t4 = lane >> 4, ss = (lane >> 3) & 1, g = lane & 7, n = lane & 15;
+    const int strip = 2 * (blockIdx.x * SB + warp) + ss;
+    const Planes P = planes_of(R.ent, MODE);
+    LaneCtx L;
+    L.unit0 = (size_t)strip * C + chunk0; L.rec0 = L.unit0 * 32 + 4 * g + t4;
+    L.nrec = (size_t)(N / 16) * C * 32;
+    L.src = (lane + 16) & 63; L.g = g;
+    L.xs = (n < ntok ? smem + n * rowstride : zero) + t4 * 16; L.xstep = n < ntok ? 256 : 0;
+    float4_t acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+    if (R.level == 2) gemv_chunks<false, 0>(P, L, NC, acc);
+    else dispatch_code(P.code, [&](auto tag) { gemv_chunks<true, decltype(tag)::value>(P, L, NC, acc); });
+
+    // ---- k-slice partial sums: lane (t4, n) holds rows 16 (strip0 + t4 / 2) + 4 (t4 & 1) + i (+ 8 for acc[1]) of token n
+    if (n < ntok)
+    {
+        const int S = a.B * a.topk;
+        float* part = (MODE == 0 ? a.part_gu : a.part_d) + ((size_t)blockIdx.y * S + R.slot[n]) * N;
+        const int row = 16 * (2 * (blockIdx.x * SB + warp) + (t4 >> 1)) + 4 * (t4 & 1);
+        *(float4_t*)(part + row) = acc[0];
+        *(float4_t*)(part + row + 8) = acc[1];
+    }
+}
+
+// per (slot, 128-column group): h[slot] = fp16(WHT(silu(g) * u * su_d)), g = WHT(sum_ky part_g) * sv_g, u likewise
+// grid (I / 128 / 4, S), block 256 (wave = one column group)
+__global__ void __launch_bounds__(256) nq_fin_gu_k(MoeArgs a, int NY)
+{
+    const int lane = threadIdx.x & 63, grp = blockIdx.x * 4 + (threadIdx.x >> 6), s = blockIdx.y;
+    if (grp >= a.I / 128) return;
+    const long long ee = a.sel[s];
+    if (ee < 0 || ee >= a.E || (float)a.rw[s] == 0.f) return;
+    const int64_t* ent = a.table + (size_t)ee * TBL_W;
+    if (ent[0] <= 0) return;
+    const _Float16* signs = (const _Float16*)ent[9];
+    const _Float16 *sv_g = signs + a.H, *sv_u = sv_g + a.I, *su_d = sv_u + a.I;
+    const int S = a.B * a.topk, col = grp * 128 + 2 * lane;
+    float g0 = 0.f, g1 = 0.f, u0 = 0.f, u1 = 0.f;
+    for (int y = 0; y < NY; ++y)
+    {
+        const float* p = a.part_gu + ((size_t)y * S + s) * 2 * a.I + col;
+        const float2 pg = *(const float2*)p, pu = *(const float2*)(p + a.I);
+        g0 += pg.x; g1 += pg.y; u0 += pu.x; u1 += pu.y;
+    }
+    wht128(g0, g1, lane); wht128(u0, u1, lane);
+    const half2_t svg = *(const half2_t*)(sv_g + col), svu = *(const half2_t*)(sv_u + col), sud = *(const half2_t*)(su_d + col);
+    g0 *= (float)svg.x; g1 *= (float)svg.y; u0 *= (float)svu.x; u1 *= (float)svu.y;
+    float v0 = g0 / (1.f + __expf(-g0)) * u0 * (float)sud.x, v1 = g1 / (1.f + __expf(-g1)) * u1 * (float)sud.y;
+    wht128(v0, v1, lane);
+    half2_t hv; hv.x = (_Float16)v0; hv.y = (_Float16)v1;
+    *(half2_t*)(a.h + (size_t)s * a.I + col) = hv;
+}
+
+// per (token, 128-row group): out[b] = sum_k rw[b,k] * sv_o[e] (.) WHT(sum_ky part_d[slot]); grid (H / 128 / 4, B)
+__global__ void __launch_bounds__(256) nq_fin_dn_k(MoeArgs a, int NY)
+{
+    const int lane = threadIdx.x & 63, grp = blockIdx.x * 4 + (threadIdx.x >> 6), b = blockIdx.y;
+    if (grp >= a.H / 128) return;
+    const int S = a.B * a.topk, col = grp * 128 + 2 * lane;
+    float o0 = 0.f, o1 = 0.f;
+    for (int k = 0; k < a.topk; ++k)
+    {
+        const int s = b * a.topk + k;
+        const long long ee = a.sel[s];
+        const float w = (float)a.rw[s];
+        if (ee < 0 || ee >= a.E || w == 0.f) continue;
+        const int64_t* ent = a.table + (size_t)ee * TBL_W;
+        if (ent[0] <= 0) continue;
+        float v0 = 0.f, v1 = 0.f;
+        for (int y = 0; y < NY; ++y)
+        {
+            const float2 p = *(const float2*)(a.part_d + ((size_t)y * S + s) * a.H + col);
+            v0 += p.x; v1 += p.y;
+        }
+        wht128(v0, v1, lane);
+        const half2_t sv = *(const half2_t*)((const _Float16*)ent[9] + a.H + 3 * a.I + col);
+        o0 += w * (v0 * (float)sv.x); o1 += w * (v1 * (float)sv.y);
+    }
+    *(float2*)(a.out + (size_t)b * a.H + col) = make_float2(o0, o1);
+}
+
+// table[e] <- stage[e] where seq[e] != applied[e]; publish applied (device copy and optional host-mapped mirror)
+__global__ void nq_mailbox_k(int64_t* table, const int64_t* stage, const int32_t* seq, int32_t* applied, int32_t* applied_host, int E)
+{
+    const int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= E) return;
+    const int32_t sq = __hip_atomic_load(seq + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    if (sq == applied[e]) return;
+#pragma unroll
+    for (int i = 0; i < TBL_W; ++i)
+        table[(size_t)e * TBL_W + i] = __hip_atomic_load(stage + (size_t)e * TBL_W + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    __threadfence();
+    applied[e] = sq;
+    if (applied_host) __hip_atomic_store(applied_host + e, sq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+int launch_moe(const MoeArgs& a, const int* cfg_gu, const int* cfg_dn, int which, hipStream_t st)
+{
+    const int S = a.B * a.topk;
+    for (int mode = 0; mode < 2; ++mode)
+    {
+        if (!((which >> mode) & 1)) continue;
+        const int* cf = mode == 0 ? cfg_gu : cfg_dn;
+        const int NC = cf[0] * cf[2], SB = cf[1];
+        const int N = mode == 0 ? 2 * a.I : a.H, K = mode == 0 ? a.H : a.I, C = K / 128;
+        const int NX = N / 32 / SB, NY = C / NC;
+        const int shm = MAXTOK * (NC * 256 + 16) + 256;
+        auto kern = mode == 0 ? nq_gemv_k<0> : nq_gemv_k<1>;
+        if (shm > 48 * 1024)
+        {
+            hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, shm);
+            if (e != hipSuccess) return set_error("moe_forward: LDS %d bytes: %s", shm, hipGetErrorString(e));
+        }
+        kern<<<dim3(NX, NY, S), 64 * SB, shm, st>>>(a, NC);
+        NQ_LAUNCH_CHECK("moe_forward gemv");
+        if (mode == 0) nq_fin_gu_k<<<dim3((a.I / 128 + 3) / 4, S), 256, 0, st>>>(a, NY);
+        else nq_fin_dn_k<<<dim3((a.H / 128 + 3) / 4, a.B), 256, 0, st>>>(a, NY);
+        NQ_LAUNCH_CHECK("moe_forward finisher");
+    }
+    return 0;
+}
+
+int launch_mailbox(int64_t* table, const int64_t* stage, const int32_t* seq, int32_t* applied, int32_t* applied_host, int E, hipStream_t st)
+{
+    nq_mailbox_k<<<(E + 127) / 128, 128, 0, st>>>(table, stage, seq, applied, applied_host, E);
+    NQ_LAUNCH_CHECK("nq_mailbox");
+    return 0;
+}
+
+}  // namespace nq

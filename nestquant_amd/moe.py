@@ -104,3 +104,114 @@ def dense_W(ex, proj, level, dtype=torch.float16):
     validate_row(row, ex.H, ex.I)
     row = row.to(ex.signs.device)
     return dequant(row, proj, ex.H, ex.I).to(dtype)
+
+
+class MoELayer:
+    """Device table [E, TBL_W] + workspaces for up to Bmax tokens; table rows are flipped in place (graph-safe).
+
+    Same constructor, attributes and call signature as the reference's MoELayer (sm120/moe.py:231-260). Differences that
+    a caller can observe: acc_gu / acc_d hold per-k-slice partial sums ([NY, S, 2I] and [NY, S, H]) instead of
+    atomically accumulated [S, 2I] / [S, H], so they are not zero between calls and outputs are bitwise repeatable;
+    cnt_gu, cnt_d, wq, zd, cnt_h exist for attribute compatibility and stay zero."""
+
+    def __init__(s, E, H, I, nm_gu=0, nm_dn=0, Bmax=4, topk=8, G=4, dev="cuda", mod=None):
+        if G != 4:
+            raise NotImplementedError("rings of G=4 lanes only")
+        s.M = mod or _lib.lib()
+        s.E, s.H, s.I, s.nm_gu, s.nm_dn, s.G, s.Bmax, s.topk = E, H, I, nm_gu, nm_dn, G, Bmax, topk
+        s.table = torch.zeros(E, TBL_W, dtype=torch.int64, device=dev)
+        S = Bmax * topk
+        f32, i32 = torch.float32, torch.int32
+        s.cfg_gu, s.cfg_dn = s.default_cfg(H, I)
+        s.h = torch.zeros(S, I, dtype=torch.float16, device=dev)
+        s.cnt_gu = torch.zeros(S * (I // 128), dtype=i32, device=dev); s.cnt_d = torch.zeros(H // 128, dtype=i32, device=dev)
+        s.wq = torch.zeros(4, dtype=i32, device=dev)
+        s.zd = torch.zeros(S * (I // 128) * 4, dtype=f32, device=dev); s.cnt_h = torch.zeros(S * (I // 128), dtype=i32, device=dev)
+        s.out = torch.zeros(Bmax, H, dtype=f32, device=dev)
+        s.hits_ptr = 0
+        s._alloc_partials()
+
+    @staticmethod
+    def default_cfg(H, I):
+        """[cpw, sb, nst]: k-slice of cpw * nst chunks, sb wavefronts per block"""
+        def pick(C, N, want):
+            nc = max(d for d in range(1, want + 1) if C % d == 0)
+            sb = max(d for d in (4, 2, 1) if (N // 32) % d == 0 and (I // 32) % d == 0)
+            return [1, sb, nc]
+        return pick(H // 128, 2 * I, 6), pick(I // 128, H, 4)
+
+    def _ny(s, cfg, C):
+        return C // (cfg[0] * cfg[2])
+
+    def _alloc_partials(s, cfg_gu=None, cfg_dn=None):
+        S, dev = s.Bmax * s.topk, s.table.device
+        ny_gu, ny_dn = s._ny(cfg_gu or s.cfg_gu, s.H // 128), s._ny(cfg_dn or s.cfg_dn, s.I // 128)
+        if getattr(s, "acc_gu", None) is None or s.acc_gu.shape[0] < ny_gu:
+            s.acc_gu = torch.zeros(ny_gu, S, 2 * s.I, dtype=torch.float32, device=dev)
+        if getattr(s, "acc_d", None) is None or s.acc_d.shape[0] < ny_dn:
+            s.acc_d = torch.zeros(ny_dn, S, s.H, dtype=torch.float32, device=dev)
+
+    def set_cfg(s, cfg_gu=None, cfg_dn=None):
+        """change the default tilings (re-sizes the partial-sum workspaces; not graph-safe)"""
+        s.cfg_gu, s.cfg_dn = list(cfg_gu or s.cfg_gu), list(cfg_dn or s.cfg_dn)
+        s._alloc_partials()
+
+    def set(s, e, ex, level):
+        row = entry(ex, level)
+        validate_row(row, s.H, s.I)
+        s.table[e].copy_(row.to(s.table.device), non_blocking=False)
+
+    def __call__(s, x, sel, rw, out=None, force_level=0, which=3, cfg_gu=None, cfg_dn=None, table=None):
+        """x fp16 [B, H], sel int64 [B, topk], rw fp16 [B, topk] -> fp32 [B, H] (s.out[:B] unless `out` is given).
+        table: optional [E, TBL_W] override. Everything is enqueued on torch's current stream; nothing syncs."""
+        assert x.dtype == torch.float16 and rw.dtype == torch.float16 and sel.dtype == torch.int64, (x.dtype, rw.dtype, sel.dtype)
+        assert x.is_contiguous() and sel.is_contiguous() and rw.is_contiguous()
+        B, topk = sel.shape
+        out = s.out[:B] if out is None else out
+        tb = s.table if table is None else table
+        cg, cd = list(cfg_gu or s.cfg_gu), list(cfg_dn or s.cfg_dn)
+        s._alloc_partials(cg, cd)                    # grows only when a call brings a finer k-split than any before
+        a = _lib.NqMoeArgs()
+        a.x, a.sel, a.rw, a.table, a.out = x.data_ptr(), sel.data_ptr(), rw.data_ptr(), tb.data_ptr(), out.data_ptr()
+        a.acc_gu, a.h, a.acc_d, a.hits = s.acc_gu.data_ptr(), s.h.data_ptr(), s.acc_d.data_ptr(), s.hits_ptr or None
+        a.acc_gu_elems, a.acc_d_elems, a.h_elems, a.out_elems = s.acc_gu.numel(), s.acc_d.numel(), s.h.numel(), out.numel()
+        a.B, a.topk, a.E, a.H, a.I = B, topk, tb.shape[0], x.shape[1], s.I
+        a.cfg_gu = (C.c_int32 * 4)(*(cg + [0] * (4 - len(cg)))); a.cfg_dn = (C.c_int32 * 4)(*(cd + [0] * (4 - len(cd))))
+        a.force_level, a.which = force_level, which
+        _lib.check(s.M.nq_moe_forward(C.byref(a), _lib.stream_ptr()))
+        return out
+
+
+class Mailbox:
+    """Graph-safe table updates (reference sm120/moe.py:329-342): call apply() on the compute stream before the layer;
+    stage rows from a side stream with post(). One outstanding op per expert."""
+
+    def __init__(s, layer):
+        E, dev = layer.E, layer.table.device
+        s.L = layer
+        s.stage = torch.zeros(E, TBL_W, dtype=torch.int64, device=dev)
+        s.seq = torch.zeros(E, dtype=torch.int32, device=dev)
+        s.applied = torch.zeros(E, dtype=torch.int32, device=dev)
+        s.applied_host = torch.zeros(E, dtype=torch.int32).pin_memory()
+        s.hseq = [0] * E
+        s.pins = []
+
+    def apply(s):
+        _lib.check(s.L.M.nq_mailbox(s.L.table.data_ptr(), s.stage.data_ptr(), s.seq.data_ptr(), s.applied.data_ptr(),
+                                    s.applied_host.data_ptr(), s.L.E, _lib.stream_ptr()))
+
+    def post(s, e, row, stream):
+        """enqueue on `stream`, after any plane copy already enqueued there: stage[e] = row; seq[e] += 1"""
+        assert s.done(e), "one outstanding op per expert"
+        validate_row(row, s.L.H, s.L.I)
+        s.hseq[e] += 1
+        r = row.pin_memory(); q = torch.tensor([s.hseq[e]], dtype=torch.int32).pin_memory()
+        s.pins += [r, q]
+        if len(s.pins) > 4096:                       # rows whose copies completed long ago
+            del s.pins[:2048]
+        with torch.cuda.stream(stream):
+            s.stage[e].copy_(r, non_blocking=True)
+            s.seq[e:e + 1].copy_(q, non_blocking=True)
+
+    def done(s, e):
+        return int(s.applied_host[e]) == s.hseq[e]

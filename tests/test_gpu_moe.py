@@ -1,0 +1,196 @@
+"""Decode-path MoE layer (nq_moe_forward through the C ABI) against the oracle's layer math.
+
+Tolerances: 1e-4 relative (L2) against the oracle pipeline with the same two fp16 activation roundings -- the band the
+reference's own kernel shows against its torch reference (1.4e-5 .. 9.8e-5, sm120/results/check_I512.txt) -- and 1e-3
+against an fp32 pipeline without those roundings (the north-star gate)."""
+import random
+
+import numpy as np
+import pytest
+import torch
+
+from nestquant_amd import format as F, moe as M, routing as RT
+from oracle import nq_oracle as O
+from tests.util import oracle_plane, rel_err
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def experts_on_gpu(H, I, n, seed0, nested_ids=(), rk=None, var_ids=()):
+    ex = []
+    for i in range(n):
+        rg, rd = (0, 0) if rk is None else rk[i]
+        ex.append(F.Expert(H, I, seed=seed0 + i, dev="cpu", rk_gu=rg, rk_dn=rd, nested=i in nested_ids, var=i in var_ids))
+    return ex
+
+
+def to_dev(ex):
+    for e in ex:
+        e.gu.to(DEV); e.dn.to(DEV); e.signs = e.signs.to(DEV)
+        if e.nested:
+            e.gu.slot = e.gu.nested_plane(); e.dn.slot = e.dn.nested_plane()
+    return ex
+
+
+def oracle_layer(ex_cpu_planes, levels, signs, x, sel, rw, **kw):
+    def dense(e):
+        pg, pd, nested = ex_cpu_planes[e]
+        return (O.dense_W(pg, levels[e], nested=nested).astype(np.float32), O.dense_W(pd, levels[e], nested=nested).astype(np.float32))
+    return O.moe_forward(dense, levels, lambda e: signs[e], x.cpu().numpy(), sel.cpu().numpy(), rw.cpu().numpy(), **kw)
+
+
+def test_small_layer_all_levels_and_codes_vs_full_oracle():
+    """H 512, I 256: decode AND layer math from the oracle; levels 0/2/3/4, wide-plane codes, sign planes, zero weights"""
+    H, I, NE = 512, 256, 10
+    rk = [(0, 0), (3, 7), (6, 9), (8, 3), (0, 0), (1, 2), (4, 5), (0, 0), (7, 6), (0, 0)]
+    nested = (4, 7, 9)
+    ex = experts_on_gpu(H, I, NE, 40, nested_ids=nested, rk=rk, var_ids=(1, 4))
+    planes = [(oracle_plane(e.gu), oracle_plane(e.dn), e.nested) for e in ex]
+    signs = [e.signs.numpy() for e in ex]
+    levels = [2, 4, 4, 4, 3, 4, 4, 4, 2, 0]
+    to_dev(ex)
+    L = M.MoELayer(NE, H, I, Bmax=8, topk=4)
+    for e in range(NE):
+        L.set(e, ex[e], levels[e])
+    rng = random.Random(1)
+    g = torch.Generator().manual_seed(2)
+    for B in (1, 2, 3, 5, 8):
+        rows = RT.make_sel(B, range(NE), "recency", p=0.5, rng=rng, topk=4)
+        sel, rw = RT.routing_tensors(rows, seed=B)
+        if B == 3:
+            rw[1, 2] = 0
+        x = (torch.randn(B, H, generator=g) * 0.05).half().to(DEV)
+        want = oracle_layer(planes, levels, signs, x, sel, rw)
+        for cg, cd in (([1, 4, 2], [1, 4, 2]), ([1, 1, 1], [2, 2, 1]), ([2, 8, 2], [1, 8, 1])):
+            y = L(x, sel, rw, cfg_gu=cg, cfg_dn=cd).clone()
+            y2 = L(x, sel, rw, cfg_gu=cg, cfg_dn=cd).clone()
+            torch.cuda.synchronize()
+            assert rel_err(y.cpu().numpy(), want) < 1e-4, (B, cg, cd)
+            assert torch.equal(y, y2)                              # partial sums, no atomics: bitwise repeatable
+        pure = oracle_layer(planes, levels, signs, x, sel, rw, round_acts=False)
+        assert rel_err(y.cpu().numpy(), pure) < 1e-3
+
+
+def test_golden_layer_fixture(golden_dir):
+    """the reference's own moe_ref output on the small golden layer (levels 2/4/4/0, codes 3/7, a sign plane, rw == 0)"""
+    z = np.load(f"{golden_dir}/layer_small.npz")
+    H, I = int(z["H"]), int(z["I"])
+    ex = to_dev([F.Expert(H, I, seed=int(z["seeds"][i]), dev="cpu", rk_gu=int(z["rk_gu"][i]), rk_dn=int(z["rk_dn"][i]),
+                          var=bool(z["var"][i])) for i in range(4)])
+    L = M.MoELayer(4, H, I, Bmax=4, topk=4)
+    for e in range(4):
+        L.set(e, ex[e], int(z["levels"][e]))
+    x = torch.from_numpy(z["x"].view(np.float16).copy()).to(DEV)
+    sel = torch.from_numpy(z["sel"]).to(DEV); rw = torch.from_numpy(z["rw"].view(np.float16).copy()).to(DEV)
+    y = L(x, sel, rw)
+    torch.cuda.synchronize()
+    assert rel_err(y.cpu().numpy(), z["y"]) < 1e-4
+
+
+def _dense_from_gpu(ex, levels):
+    """dense weights through the HIP decoder (proved bit-exact in test_gpu_dequant) for full-shape layer checks"""
+    cache = {}
+
+    def dense(e):
+        if e not in cache:
+            cache[e] = (M.dense_W(ex[e], 0, levels[e]).float().cpu().numpy(), M.dense_W(ex[e], 1, levels[e]).float().cpu().numpy())
+        return cache[e]
+    return dense
+
+
+def test_full_shape_layer_like_reference_check():
+    """H 6144, I 2048, 12 experts at mixed levels, B 1..4 x {recency, distinct, same} x tilings (reference sm120/check.py)"""
+    H, I, NE = 6144, 2048, 12
+    levels = [2, 4, 4, 2, 3, 4, 2, 4, 3, 4, 2, 0]
+    nested = tuple(i for i in range(NE) if levels[i] == 3 or i in (5, 9))
+    ex = to_dev(experts_on_gpu(H, I, NE, 100, nested_ids=nested, rk=[(6, 7) if i in (1, 2) else (0, 0) for i in range(NE)]))
+    L = M.MoELayer(NE, H, I, Bmax=4)
+    for e in range(NE):
+        L.set(e, ex[e], levels[e])
+    dense = _dense_from_gpu(ex, levels)
+    signs = [e.signs.cpu().numpy() for e in ex]
+    rng = random.Random(0)
+    worst = 0.0
+    for B in (1, 2, 3, 4):
+        for mode in ("recency", "distinct", "same"):
+            if mode == "same":
+                rows = [RT.make_sel(1, range(NE), rng=rng)[0]] * B
+            elif mode == "distinct" and B * 8 > NE:
+                rows = RT.make_sel(B, range(NE), "recency", p=0.0, rng=rng)
+            else:
+                rows = RT.make_sel(B, range(NE), mode, p=0.5, rng=rng)
+            sel, rw = RT.routing_tensors(rows, seed=B)
+            x = (torch.randn(B, H, device=DEV) * 0.05).half()
+            want = O.moe_forward(dense, levels, lambda e: signs[e], x.cpu().numpy(), sel.cpu().numpy(), rw.cpu().numpy())
+            for cg, cd in (([1, 4, 6], [1, 4, 4]), ([2, 8, 4], [2, 8, 4]), ([1, 2, 12], [1, 8, 2])):
+                y = L(x, sel, rw, cfg_gu=cg, cfg_dn=cd)
+                torch.cuda.synchronize()
+                err = rel_err(y.cpu().numpy(), want)
+                worst = max(worst, err)
+                assert err < 1e-4, (B, mode, cg, cd, err)
+    print("worst rel err", worst)
+
+
+def test_force_level_which_hits_and_out_of_range_ids():
+    H, I, NE = 256, 256, 6
+    ex = to_dev(experts_on_gpu(H, I, NE, 7, nested_ids=range(NE)))
+    L = M.MoELayer(NE, H, I, Bmax=2, topk=4)
+    for e in range(NE):
+        L.set(e, ex[e], 4)
+    sel = torch.tensor([[0, 1, 2, 3], [3, 4, 5, 0]], device=DEV); rw = torch.full((2, 4), 0.25, device=DEV).half()
+    x = (torch.randn(2, H, device=DEV) * 0.05).half()
+    signs = [e.signs.cpu().numpy() for e in ex]
+    for lv in (2, 4):                                            # rows are level 4; force_level = 2 must read the base only
+        dense = _dense_from_gpu(ex, [lv] * NE)
+        want = O.moe_forward(dense, [lv] * NE, lambda e: signs[e], x.cpu().numpy(), sel.cpu().numpy(), rw.cpu().numpy())
+        y = L(x, sel, rw, force_level=lv)
+        torch.cuda.synchronize()
+        assert rel_err(y.cpu().numpy(), want) < 1e-4, lv
+    # which = 1 then which = 2 equals which = 3
+    y3 = L(x, sel, rw).clone()
+    L(x, sel, rw, which=1); y12 = L(x, sel, rw, which=2).clone()
+    assert torch.equal(y3, y12)
+    # hits: one count per pick with rw != 0 (device buffer here)
+    hits = torch.zeros(NE, dtype=torch.int32, device=DEV)
+    L.hits_ptr = hits.data_ptr()
+    rw2 = rw.clone(); rw2[0, 1] = 0
+    L(x, sel, rw2); L(x, sel, rw2)
+    torch.cuda.synchronize()
+    assert hits.tolist() == [4, 0, 2, 4, 2, 2]
+    L.hits_ptr = 0
+    # an expert id outside [0, E) contributes nothing and does not fault
+    selbad = sel.clone(); selbad[1, 3] = 99
+    rwz = rw.clone(); rwz[1, 3] = 0
+    assert torch.equal(L(x, selbad, rw).clone(), L(x, sel, rwz).clone())
+
+
+def test_argument_errors():
+    L = M.MoELayer(4, 256, 256, Bmax=2, topk=4)
+    x = torch.zeros(2, 256, dtype=torch.float16, device=DEV); sel = torch.zeros(2, 4, dtype=torch.int64, device=DEV)
+    rw = torch.zeros(2, 4, dtype=torch.float16, device=DEV)
+    with pytest.raises(RuntimeError, match="bad cfg"):
+        L(x, sel, rw, cfg_gu=[1, 4, 3])
+    with pytest.raises(RuntimeError, match="persistent"):
+        L(x, sel, rw, cfg_gu=[1, 4, 2, 1])
+    with pytest.raises(RuntimeError, match="B="):
+        L(torch.zeros(9, 256, dtype=torch.float16, device=DEV), torch.zeros(9, 4, dtype=torch.int64, device=DEV),
+          torch.zeros(9, 4, dtype=torch.float16, device=DEV), out=torch.zeros(9, 256, device=DEV))
+    with pytest.raises(AssertionError):
+        L(x.float(), sel, rw)
+    y = L(x, sel, rw)                                            # all weights zero -> zeros, no fault
+    assert not y.any()
+
+
+def test_mailbox_kernel_matches_state_machine():
+    L = M.MoELayer(8, 256, 256, Bmax=1, topk=2)
+    MB = M.Mailbox(L)
+    table = torch.randint(0, 1000, (8, F.TBL_W), dtype=torch.int64); stage = torch.randint(0, 1000, (8, F.TBL_W), dtype=torch.int64)
+    seq = torch.tensor([0, 1, 0, 2, 5, 0, 0, 1], dtype=torch.int32); applied = torch.tensor([0, 0, 0, 2, 4, 0, 0, 1], dtype=torch.int32)
+    L.table.copy_(table); MB.stage.copy_(stage); MB.seq.copy_(seq); MB.applied.copy_(applied)
+    MB.apply(); torch.cuda.synchronize()
+    t, a = table.numpy().copy(), applied.numpy().copy()
+    n = O.mailbox_apply(t, stage.numpy(), seq.numpy(), a)
+    assert n == 2
+    assert np.array_equal(L.table.cpu().numpy(), t) and np.array_equal(MB.applied.cpu().numpy(), a)
+    assert MB.applied_host.numpy()[[1, 4]].tolist() == [1, 5]
