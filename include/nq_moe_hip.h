@@ -51,7 +51,8 @@ int nq_pf_decode(const int64_t* table, const int32_t* experts, int G, void* Wgu_
  * decodes two 16-row strips), as the reference's {chunks per warp, warps per block, stages}. Workspaces hold k-slice
  * partial sums (no atomics, no zero-on-entry contract): acc_gu >= (H/128/(cpw*nst)) * B*topk * 2I floats,
  * acc_d >= (I/128/(cpw*nst)) * B*topk * H floats, h >= B*topk * I halfs. Picks with rw == 0, level <= 0 or an expert id
- * outside [0, E) contribute nothing. which: bit 0 = gate|up launches, bit 1 = down launches. hits: optional int32[E]
+ * outside [0, E) contribute nothing. which: bit 0 = gate|up launches, bit 1 = down launches, bit 2 = skip the two
+ * finisher launches (timing the decode+GEMV kernels alone; h and out are then not produced). hits: optional int32[E]
  * pick counters (device or host-mapped memory), incremented once per pick with rw != 0 (reference :784-787). */
 typedef struct NqMoeArgs
 {

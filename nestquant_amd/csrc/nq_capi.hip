@@ -81,7 +81,7 @@ extern "C" int nq_moe_forward(const NqMoeArgs* p, void* stream)
     NQ_REQUIRE(p->B >= 1 && p->B <= 8 && p->topk >= 1 && p->B * p->topk <= 64, "nq_moe_forward: B=%d topk=%d (B <= 8, B*topk <= 64)", p->B, p->topk);
     NQ_REQUIRE(p->E >= 1, "nq_moe_forward: E=%d", p->E);
     NQ_REQUIRE(shape_ok(p->H, p->I), "nq_moe_forward: H=%d I=%d must be positive multiples of 128", p->H, p->I);
-    NQ_REQUIRE((p->which & ~3) == 0, "nq_moe_forward: which=%d", p->which);
+    NQ_REQUIRE((p->which & ~7) == 0, "nq_moe_forward: which=%d", p->which);
     NQ_REQUIRE(p->force_level == 0 || p->force_level == 2 || p->force_level == 3 || p->force_level == 4, "nq_moe_forward: force_level=%d", p->force_level);
     const int64_t S = (int64_t)p->B * p->topk;
     for (int mode = 0; mode < 2; ++mode)

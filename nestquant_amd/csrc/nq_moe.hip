@@ -321,6 +321,7 @@ int launch_moe(const MoeArgs& a, const int* cfg_gu, const int* cfg_dn, int which
         }
         kern<<<dim3(NX, NY, S), 64 * SB, shm, st>>>(a, NC);
         NQ_LAUNCH_CHECK("moe_forward gemv");
+        if (which & 4) continue;                                  // profiling: GEMV launches only
         if (mode == 0) nq_fin_gu_k<<<dim3((a.I / 128 + 3) / 4, S), 256, 0, st>>>(a, NY);
         else nq_fin_dn_k<<<dim3((a.H / 128 + 3) / 4, a.B), 256, 0, st>>>(a, NY);
         NQ_LAUNCH_CHECK("moe_forward finisher");

@@ -211,15 +211,30 @@ class Expert:
         if nested:                                       # slot image: [P3 | P4] per projection, contiguous
             s.gu.slot = s.gu.nested_plane(); s.dn.slot = s.dn.nested_plane()
 
+    def compact(s):
+        """drop everything a layer call does not read (unpacked words; for nested experts the wide plane and the separate
+        P3 / P4 tensors, whose bytes live on in `slot`)"""
+        for p in (s.gu, s.dn):
+            p.drop_host_words()
+            p.Mb = p.Nn = None
+            if s.nested:
+                p._nbytes = dict(p3=p.p3.numel() * 4, p4n=p.p4n.numel() * 4, p4=p.p4.numel() * 4)
+                p.p4 = p.d4 = p.p3 = p.p4n = None
+                for k in ("Mb3", "N3", "Mb4n", "N4n"):
+                    setattr(p, k, None)
+        return s
+
     def bytes(s, level):
         """plane bytes a layer call reads for this expert at `level` (the reference's GB/s numerator, sm120/moe.py:190-195)"""
         b = 0
         for p in (s.gu, s.dn):
             b += p.base.numel() * 4 + (0 if p.var is None else p.var.numel())
+            nb = getattr(p, "_nbytes", None) or dict(p3=0 if p.p3 is None else p.p3.numel() * 4,
+                                                      p4n=0 if p.p4n is None else p.p4n.numel() * 4)
             if level == 3:
-                b += (p.p3.numel() + p.d3.numel()) * 4
+                b += nb["p3"] + p.d3.numel() * 4
             elif level >= 4 and s.nested:
-                b += (p.p3.numel() + p.p4n.numel() + p.d4n.numel()) * 4
+                b += nb["p3"] + nb["p4n"] + p.d4n.numel() * 4
             elif level >= 4:
                 b += (p.p4.numel() + p.d4.numel()) * 4
         return b
