@@ -47,13 +47,14 @@ int nq_pf_decode(const int64_t* table, const int32_t* experts, int G, void* Wgu_
                  void* stream);
 
 /* One decode-path MoE layer call, B <= 8 tokens, B * topk <= 64 picks (reference moe_forward, sm120/nqmoe.cu:858-907).
- * cfg = {cpw, sb, nst, 0}: k-slice = cpw * nst chunks of 128 columns per block, sb wavefronts per block (each wavefront
- * decodes two 16-row strips), as the reference's {chunks per warp, warps per block, stages}. Workspaces hold k-slice
- * partial sums (no atomics, no zero-on-entry contract): acc_gu >= (H/128/(cpw*nst)) * B*topk * 2I floats,
- * acc_d >= (I/128/(cpw*nst)) * B*topk * H floats, h >= B*topk * I halfs. Picks with rw == 0, level <= 0 or an expert id
- * outside [0, E) contribute nothing. which: bit 0 = gate|up launches, bit 1 = down launches, bit 2 = skip the two
- * finisher launches (timing the decode+GEMV kernels alone; h and out are then not produced). hits: optional int32[E]
- * pick counters (device or host-mapped memory), incremented once per pick with rw != 0 (reference :784-787). */
+ * cfg = {cpw, sb, nst, 0}: k-slice = cpw * nst chunks of 128 columns per block; sb = 1, 2 or 4 wavefronts per block (each
+ * wavefront decodes two 16-row strips, so sb = 4 covers the reference's largest block of 128 rows); the 4th entry
+ * (persistent mode) must be 0. Workspaces: acc_gu / acc_d hold k-slice partial sums (plain stores, no float atomics):
+ * acc_gu >= (H/128/(cpw*nst)) * B*topk * 2I floats, acc_d >= (I/128/(cpw*nst)) * B*topk * H floats, h >= B*topk * I
+ * halfs; cnt_gu >= B*topk * I/128 and cnt_d >= H/128 int32 arrival counters, zero on entry and zero again on exit (the
+ * reference's workspace contract, sm120/nqmoe.cu:855-857). Picks with rw == 0, level <= 0 or an expert id outside
+ * [0, E) contribute nothing. which: bit 0 = gate|up launch, bit 1 = down launch. hits: optional int32[E] pick counters
+ * (device or host-mapped memory), incremented once per pick with rw != 0 (reference :784-787). */
 typedef struct NqMoeArgs
 {
     const void* x;            /* fp16 [B][H] */
@@ -64,8 +65,10 @@ typedef struct NqMoeArgs
     void* acc_gu;             /* fp32 workspace */
     void* h;                  /* fp16 workspace */
     void* acc_d;              /* fp32 workspace */
+    int32_t* cnt_gu;          /* int32 workspace, zero on entry */
+    int32_t* cnt_d;           /* int32 workspace, zero on entry */
     int32_t* hits;            /* optional, may be NULL */
-    int64_t acc_gu_elems, acc_d_elems, h_elems, out_elems;   /* capacities, checked against the shapes above */
+    int64_t acc_gu_elems, acc_d_elems, h_elems, out_elems, cnt_gu_elems, cnt_d_elems;   /* capacities, checked */
     int32_t B, topk, E, H, I;
     int32_t cfg_gu[4], cfg_dn[4];
     int32_t force_level;      /* 0, or a level that overrides every active row's level (debug) */

@@ -14,8 +14,10 @@ _vp, _i, _i64p, _i32p = C.c_void_p, C.c_int, C.c_void_p, C.c_void_p
 class NqMoeArgs(C.Structure):
     """mirror of struct NqMoeArgs in include/nq_moe_hip.h"""
     _fields_ = [("x", C.c_void_p), ("sel", C.c_void_p), ("rw", C.c_void_p), ("table", C.c_void_p), ("out", C.c_void_p),
-                ("acc_gu", C.c_void_p), ("h", C.c_void_p), ("acc_d", C.c_void_p), ("hits", C.c_void_p),
+                ("acc_gu", C.c_void_p), ("h", C.c_void_p), ("acc_d", C.c_void_p), ("cnt_gu", C.c_void_p), ("cnt_d", C.c_void_p),
+                ("hits", C.c_void_p),
                 ("acc_gu_elems", C.c_int64), ("acc_d_elems", C.c_int64), ("h_elems", C.c_int64), ("out_elems", C.c_int64),
+                ("cnt_gu_elems", C.c_int64), ("cnt_d_elems", C.c_int64),
                 ("B", C.c_int32), ("topk", C.c_int32), ("E", C.c_int32), ("H", C.c_int32), ("I", C.c_int32),
                 ("cfg_gu", C.c_int32 * 4), ("cfg_dn", C.c_int32 * 4), ("force_level", C.c_int32), ("which", C.c_int32)]
 

@@ -77,11 +77,11 @@ extern "C" int nq_pf_decode(const int64_t* table, const int32_t* experts, int G,
 extern "C" int nq_moe_forward(const NqMoeArgs* p, void* stream)
 {
     NQ_REQUIRE(p, "nq_moe_forward: null args");
-    NQ_REQUIRE(p->x && p->sel && p->rw && p->table && p->out && p->acc_gu && p->h && p->acc_d, "nq_moe_forward: null pointer");
+    NQ_REQUIRE(p->x && p->sel && p->rw && p->table && p->out && p->acc_gu && p->h && p->acc_d && p->cnt_gu && p->cnt_d, "nq_moe_forward: null pointer");
     NQ_REQUIRE(p->B >= 1 && p->B <= 8 && p->topk >= 1 && p->B * p->topk <= 64, "nq_moe_forward: B=%d topk=%d (B <= 8, B*topk <= 64)", p->B, p->topk);
     NQ_REQUIRE(p->E >= 1, "nq_moe_forward: E=%d", p->E);
     NQ_REQUIRE(shape_ok(p->H, p->I), "nq_moe_forward: H=%d I=%d must be positive multiples of 128", p->H, p->I);
-    NQ_REQUIRE((p->which & ~7) == 0, "nq_moe_forward: which=%d", p->which);
+    NQ_REQUIRE((p->which & ~3) == 0, "nq_moe_forward: which=%d", p->which);
     NQ_REQUIRE(p->force_level == 0 || p->force_level == 2 || p->force_level == 3 || p->force_level == 4, "nq_moe_forward: force_level=%d", p->force_level);
     const int64_t S = (int64_t)p->B * p->topk;
     for (int mode = 0; mode < 2; ++mode)
@@ -90,17 +90,18 @@ extern "C" int nq_moe_forward(const NqMoeArgs* p, void* stream)
         const int N = mode == 0 ? 2 * p->I : p->H, K = mode == 0 ? p->H : p->I, C = K / 128;
         NQ_REQUIRE(cf[0] >= 1 && cf[1] >= 1 && cf[2] >= 1 && cf[3] == 0, "bad cfg: {%d,%d,%d,%d} (cpw, sb, nst >= 1; persistent mode is not implemented)", cf[0], cf[1], cf[2], cf[3]);
         const int NC = cf[0] * cf[2], SB = cf[1];
-        NQ_REQUIRE(C % NC == 0 && SB <= 8 && (N / 32) % SB == 0 && (mode == 1 || (p->I / 32) % SB == 0) && NC <= 48,
-                   "bad cfg: k-slice %d chunks of %d, %d wavefronts per block for N=%d", NC, C, SB, N);
+        NQ_REQUIRE(C % NC == 0 && (SB == 1 || SB == 2 || SB == 4) && NC <= 48,
+                   "bad cfg: k-slice %d chunks of %d, %d wavefronts per block for N=%d (sb must be 1, 2 or 4)", NC, C, SB, N);
         const int64_t need = (int64_t)(C / NC) * S * N, have = mode == 0 ? p->acc_gu_elems : p->acc_d_elems;
         NQ_REQUIRE(have >= need, "workspace too small: %s holds %lld floats, needs %lld", mode == 0 ? "acc_gu" : "acc_d", (long long)have, (long long)need);
     }
     NQ_REQUIRE(p->h_elems >= S * p->I && p->out_elems >= (int64_t)p->B * p->H, "workspace too small: h or out");
+    NQ_REQUIRE(p->cnt_gu_elems >= S * (p->I / 128) && p->cnt_d_elems >= p->H / 128, "workspace too small: cnt_gu or cnt_d");
     MoeArgs a{};
     a.x = (const _Float16*)p->x; a.sel = p->sel; a.rw = (const _Float16*)p->rw; a.B = p->B; a.topk = p->topk;
     a.table = p->table; a.E = p->E; a.H = p->H; a.I = p->I;
     a.part_gu = (float*)p->acc_gu; a.h = (_Float16*)p->h; a.part_d = (float*)p->acc_d; a.out = (float*)p->out;
-    a.force_level = p->force_level; a.hits = p->hits;
+    a.force_level = p->force_level; a.hits = p->hits; a.cnt_gu = p->cnt_gu; a.cnt_d = p->cnt_d;
     return launch_moe(a, p->cfg_gu, p->cfg_dn, p->which, (hipStream_t)stream);
 }
 

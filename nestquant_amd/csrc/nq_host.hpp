@@ -27,6 +27,7 @@ struct MoeArgs
     const int64_t* table; int E, H, I;
     float* part_gu; _Float16* h; float* part_d; float* out;
     int force_level; int* hits;
+    int* cnt_gu; int* cnt_d;          // arrival counters [S * I/128] and [H/128]: zero on entry, zero on exit
 };
 
 // kernel launchers defined next to their kernels

@@ -1,20 +1,21 @@
 // Decode-path MoE layer for 1..8 tokens (reference sm120/nqmoe.cu:375-449 route, :493-771 do_item, :858-907 moe_forward,
-// :908-929 mailbox). Four launches on one stream, every routing / level / pointer decision read on the device:
+// :908-929 mailbox). Two launches on one stream, every routing / level / pointer decision read on the device:
 //
 //   nq_gemv_k<0>  gate|up: grid (strip-pair blocks, k-slices, runs). A run = one distinct routed expert + the tokens that
 //                 picked it. The block rotates those tokens' x (x * su -> Hadamard-128 -> fp16) into LDS, then every
 //                 wavefront decodes the records of two strips chunk by chunk straight into MFMA A operands
-//                 (v_mfma_f32_16x16x32_f16, tokens as the N dimension) and writes its k-slice partial sums.
-//   nq_fin_gu_k   per (slot, 128-column group): sum the k-slice partials, Hadamard * sv, SwiGLU, * su_d, Hadamard -> h fp16.
-//   nq_gemv_k<1>  down: same kernel on h.
-//   nq_fin_dn_k   per (token, 128-row group): out[b] = sum_k rw[b,k] * sv_o (.) Hadamard(sum of partials).
+//                 (v_mfma_f32_16x16x32_f16, tokens as the N dimension) and writes its k-slice partial sums. The block
+//                 that arrives last at a (run, 128-column group) counter sums the partials and finishes them:
+//                 Hadamard * sv, SwiGLU, * su_d, Hadamard -> h fp16.
+//   nq_gemv_k<1>  down: same kernel on h; the last block of a 128-row output group (counter over all runs) combines:
+//                 out[b] = sum_k rw[b,k] * sv_o (.) Hadamard(sum of partials).
 //
 // Lane mapping of the GEMV (wave64): lane = 16 * t4 + 8 * ss + g decodes the record of lane (4 g + t4) of unit
 // (strip0 + ss, chunk); it holds 32 weights of row g and 32 of row g + 8, in columns 16 t + 2 t4 + {0,1,8,9}. An MFMA
 // 16x16x32 takes 8 fp16 per lane: lanes with equal (ss, g) and different t4 are the k-groups of one A row, so the decoded
 // pairs are A operands as they leave the decoder, with no cross-lane movement. The B operand (tokens) comes from LDS,
-// staged in the matching column order. Partial sums instead of atomics make the layer output bitwise repeatable and
-// need no zeroed workspace.
+// staged in the matching column order. Partial sums instead of float atomics make the layer output bitwise repeatable;
+// the arrival counters are zero on entry and are reset by the block that consumes them.
 #include "nq_decode.hpp"
 #include "nq_host.hpp"
 #include <utility>
@@ -154,13 +155,79 @@ __device__ __forceinline__ void gemv_chunks(const Planes& P, const LaneCtx& L, i
     }
 }
 
+// finisher of gate|up for (run, 128-column group grp): h[slot] = fp16(WHT(silu(g) * u * su_d)), g = WHT(sum_y part_g) * sv_g
+__device__ __forceinline__ void finish_gu(const MoeArgs& a, const RunInfo& R, int grp, int NY, int warp, int SB, int lane)
+{
+    const _Float16* signs = (const _Float16*)R.ent[9];
+    const _Float16 *sv_g = signs + a.H, *sv_u = sv_g + a.I, *su_d = sv_u + a.I;
+    const int S = a.B * a.topk, col = grp * 128 + 2 * lane;
+    for (int j = warp; j < R.ntok; j += SB)
+    {
+        const int s = R.slot[j];
+        float g0 = 0.f, g1 = 0.f, u0 = 0.f, u1 = 0.f;
+        for (int y = 0; y < NY; ++y)
+        {
+            const float* p = a.part_gu + ((size_t)y * S + s) * 2 * a.I + col;
+            const float2 pg = *(const float2*)p, pu = *(const float2*)(p + a.I);
+            g0 += pg.x; g1 += pg.y; u0 += pu.x; u1 += pu.y;
+        }
+        wht128(g0, g1, lane); wht128(u0, u1, lane);
+        const half2_t svg = *(const half2_t*)(sv_g + col), svu = *(const half2_t*)(sv_u + col), sud = *(const half2_t*)(su_d + col);
+        g0 *= (float)svg.x; g1 *= (float)svg.y; u0 *= (float)svu.x; u1 *= (float)svu.y;
+        float v0 = g0 / (1.f + __expf(-g0)) * u0 * (float)sud.x, v1 = g1 / (1.f + __expf(-g1)) * u1 * (float)sud.y;
+        wht128(v0, v1, lane);
+        half2_t hv; hv.x = (_Float16)v0; hv.y = (_Float16)v1;
+        *(half2_t*)(a.h + (size_t)s * a.I + col) = hv;
+    }
+}
+
+// combine of the down projection for output rows [grp * 128, +128): out[b] = sum_k rw[b,k] * sv_o[e] (.) WHT(sum_y part_d[slot])
+// picks of a token are spread over the block's wavefronts and reduced through LDS (red: SB * 128 floats)
+__device__ __forceinline__ void finish_dn(const MoeArgs& a, int grp, int NY, int warp, int SB, int lane, float* red)
+{
+    const int S = a.B * a.topk, col = grp * 128 + 2 * lane;
+    for (int b = 0; b < a.B; ++b)
+    {
+        float o0 = 0.f, o1 = 0.f;
+        for (int k = warp; k < a.topk; k += SB)
+        {
+            const int s = b * a.topk + k;
+            const long long ee = a.sel[s];
+            const float w = (float)a.rw[s];
+            if (ee < 0 || ee >= a.E || w == 0.f) continue;
+            const int64_t* ent = a.table + (size_t)ee * TBL_W;
+            if (ent[0] <= 0) continue;
+            float v0 = 0.f, v1 = 0.f;
+            for (int y = 0; y < NY; ++y)
+            {
+                const float2 p = *(const float2*)(a.part_d + ((size_t)y * S + s) * a.H + col);
+                v0 += p.x; v1 += p.y;
+            }
+            wht128(v0, v1, lane);
+            const half2_t sv = *(const half2_t*)((const _Float16*)ent[9] + a.H + 3 * a.I + col);
+            o0 += w * (v0 * (float)sv.x); o1 += w * (v1 * (float)sv.y);
+        }
+        red[warp * 128 + 2 * lane] = o0; red[warp * 128 + 2 * lane + 1] = o1;
+        __syncthreads();
+        if (warp == 0)
+        {
+            float r0 = 0.f, r1 = 0.f;
+            for (int w2 = 0; w2 < SB; ++w2) { r0 += red[w2 * 128 + 2 * lane]; r1 += red[w2 * 128 + 2 * lane + 1]; }
+            *(float2*)(a.out + (size_t)b * a.H + col) = make_float2(r0, r1);
+        }
+        __syncthreads();
+    }
+}
+
 // MODE 0: gate|up (N = 2I, K = H, input x rotated here). MODE 1: down (N = H, K = I, input h).
-// grid (N / 32 / SB, C / NC, S); block 64 * SB threads; dynamic LDS = ntokmax * (NC * 256 + 16) + 256 bytes
+// grid (N / 32 / SB, C / NC, S); block 64 * SB threads (SB = 1, 2 or 4: a block covers at most one 128-row group);
+// dynamic LDS = MAXTOK * (NC * 256 + 16) + 256 bytes (>= SB * 512 for the combine)
 template <int MODE>
-__global__ void __launch_bounds__(512) nq_gemv_k(MoeArgs a, int NC)
+__global__ void __launch_bounds__(256) nq_gemv_k(MoeArgs a, int NC)
 {
     extern __shared__ __align__(16) char smem[];
     __shared__ RunInfo R;
+    __shared__ int last;
     const int lane = threadIdx.x & 63, warp = threadIdx.x >> 6, SB = blockDim.x >> 6;
     if (warp == 0) route(a, blockIdx.z, &R, lane);
     if (MODE == 0 && a.hits && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x < a.B * a.topk)
@@ -170,11 +237,17 @@ __global__ void __launch_bounds__(512) nq_gemv_k(MoeArgs a, int NC)
             __hip_atomic_fetch_add(a.hits + ee, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     }
     __syncthreads();
-    if ((int)blockIdx.z >= R.nruns) return;                      // block-uniform
-    const int N = MODE == 0 ? 2 * a.I : a.H, K = MODE == 0 ? a.H : a.I, C = K / 128;
+    const int nruns = R.nruns;
+    const int N = MODE == 0 ? 2 * a.I : a.H, K = MODE == 0 ? a.H : a.I, C = K / 128, NY = C / NC;
+    if (MODE == 1 && nruns == 0 && blockIdx.z == 0 && blockIdx.y == 0)
+    {   // no active pick at all: nobody will arrive last, so the first plane of blocks writes the zero output
+        for (int i = threadIdx.x; i < a.B * SB * 32; i += blockDim.x)
+            a.out[(size_t)(i / (SB * 32)) * a.H + blockIdx.x * SB * 32 + i % (SB * 32)] = 0.f;
+    }
+    if ((int)blockIdx.z >= nruns) return;                        // block-uniform
     const int ntok = R.ntok, chunk0 = blockIdx.y * NC, k0 = chunk0 * 128;
     const int rowstride = NC * 256 + 16;                         // bytes per staged token (+16: spread tokens over banks)
-    char* zero = smem + ntok * rowstride;                      // 256 zero bytes after the token rows
+    char* zero = smem + ntok * rowstride;                        // 256 zero bytes after the token rows
     const _Float16* signs = (const _Float16*)R.ent[9];
 
     // ---- stage the run's tokens for this k-slice in B-operand order
@@ -228,63 +301,22 @@ __global__ void __launch_bounds__(512) nq_gemv_k(MoeArgs a, int NC)
         *(float4_t*)(part + row) = acc[0];
         *(float4_t*)(part + row + 8) = acc[1];
     }
-}
 
-// per (slot, 128-column group): h[slot] = fp16(WHT(silu(g) * u * su_d)), g = WHT(sum_ky part_g) * sv_g, u likewise
-// grid (I / 128 / 4, S), block 256 (wave = one column group)
-__global__ void __launch_bounds__(256) nq_fin_gu_k(MoeArgs a, int NY)
-{
-    const int lane = threadIdx.x & 63, grp = blockIdx.x * 4 + (threadIdx.x >> 6), s = blockIdx.y;
-    if (grp >= a.I / 128) return;
-    const long long ee = a.sel[s];
-    if (ee < 0 || ee >= a.E || (float)a.rw[s] == 0.f) return;
-    const int64_t* ent = a.table + (size_t)ee * TBL_W;
-    if (ent[0] <= 0) return;
-    const _Float16* signs = (const _Float16*)ent[9];
-    const _Float16 *sv_g = signs + a.H, *sv_u = sv_g + a.I, *su_d = sv_u + a.I;
-    const int S = a.B * a.topk, col = grp * 128 + 2 * lane;
-    float g0 = 0.f, g1 = 0.f, u0 = 0.f, u1 = 0.f;
-    for (int y = 0; y < NY; ++y)
-    {
-        const float* p = a.part_gu + ((size_t)y * S + s) * 2 * a.I + col;
-        const float2 pg = *(const float2*)p, pu = *(const float2*)(p + a.I);
-        g0 += pg.x; g1 += pg.y; u0 += pu.x; u1 += pu.y;
-    }
-    wht128(g0, g1, lane); wht128(u0, u1, lane);
-    const half2_t svg = *(const half2_t*)(sv_g + col), svu = *(const half2_t*)(sv_u + col), sud = *(const half2_t*)(su_d + col);
-    g0 *= (float)svg.x; g1 *= (float)svg.y; u0 *= (float)svu.x; u1 *= (float)svu.y;
-    float v0 = g0 / (1.f + __expf(-g0)) * u0 * (float)sud.x, v1 = g1 / (1.f + __expf(-g1)) * u1 * (float)sud.y;
-    wht128(v0, v1, lane);
-    half2_t hv; hv.x = (_Float16)v0; hv.y = (_Float16)v1;
-    *(half2_t*)(a.h + (size_t)s * a.I + col) = hv;
-}
-
-// per (token, 128-row group): out[b] = sum_k rw[b,k] * sv_o[e] (.) WHT(sum_ky part_d[slot]); grid (H / 128 / 4, B)
-__global__ void __launch_bounds__(256) nq_fin_dn_k(MoeArgs a, int NY)
-{
-    const int lane = threadIdx.x & 63, grp = blockIdx.x * 4 + (threadIdx.x >> 6), b = blockIdx.y;
-    if (grp >= a.H / 128) return;
-    const int S = a.B * a.topk, col = grp * 128 + 2 * lane;
-    float o0 = 0.f, o1 = 0.f;
-    for (int k = 0; k < a.topk; ++k)
-    {
-        const int s = b * a.topk + k;
-        const long long ee = a.sel[s];
-        const float w = (float)a.rw[s];
-        if (ee < 0 || ee >= a.E || w == 0.f) continue;
-        const int64_t* ent = a.table + (size_t)ee * TBL_W;
-        if (ent[0] <= 0) continue;
-        float v0 = 0.f, v1 = 0.f;
-        for (int y = 0; y < NY; ++y)
-        {
-            const float2 p = *(const float2*)(a.part_d + ((size_t)y * S + s) * a.H + col);
-            v0 += p.x; v1 += p.y;
-        }
-        wht128(v0, v1, lane);
-        const half2_t sv = *(const half2_t*)((const _Float16*)ent[9] + a.H + 3 * a.I + col);
-        o0 += w * (v0 * (float)sv.x); o1 += w * (v1 * (float)sv.y);
-    }
-    *(float2*)(a.out + (size_t)b * a.H + col) = make_float2(o0, o1);
+    // ---- arrival counter of the 128-row group this block belongs to; the last block to arrive finishes the group
+    const int rows0 = blockIdx.x * SB * 32;
+    const int grp = MODE == 0 ? (rows0 % a.I) / 128 : rows0 / 128;
+    int* cnt = MODE == 0 ? a.cnt_gu + blockIdx.z * (a.I / 128) + grp : a.cnt_d + grp;
+    const int expect = (MODE == 0 ? 2 : nruns) * NY * (128 / (SB * 32));
+    __threadfence();                                             // release: this block's partial sums are visible device-wide
+    __syncthreads();
+    if (threadIdx.x == 0)
+        last = __hip_atomic_fetch_add(cnt, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) == expect - 1;
+    __syncthreads();
+    if (!last) return;                                           // block-uniform
+    __threadfence();                                             // acquire: every other block's partial sums
+    if constexpr (MODE == 0) finish_gu(a, R, grp, NY, warp, SB, lane);
+    else finish_dn(a, grp, NY, warp, SB, lane, (float*)smem);
+    if (threadIdx.x == 0) __hip_atomic_store(cnt, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // table[e] <- stage[e] where seq[e] != applied[e]; publish applied (device copy and optional host-mapped mirror)
@@ -320,11 +352,7 @@ int launch_moe(const MoeArgs& a, const int* cfg_gu, const int* cfg_dn, int which
             if (e != hipSuccess) return set_error("moe_forward: LDS %d bytes: %s", shm, hipGetErrorString(e));
         }
         kern<<<dim3(NX, NY, S), 64 * SB, shm, st>>>(a, NC);
-        NQ_LAUNCH_CHECK("moe_forward gemv");
-        if (which & 4) continue;                                  // profiling: GEMV launches only
-        if (mode == 0) nq_fin_gu_k<<<dim3((a.I / 128 + 3) / 4, S), 256, 0, st>>>(a, NY);
-        else nq_fin_dn_k<<<dim3((a.H / 128 + 3) / 4, a.B), 256, 0, st>>>(a, NY);
-        NQ_LAUNCH_CHECK("moe_forward finisher");
+        NQ_LAUNCH_CHECK("moe_forward");
     }
     return 0;
 }

@@ -112,7 +112,8 @@ class MoELayer:
     Same constructor, attributes and call signature as the reference's MoELayer (sm120/moe.py:231-260). Differences that
     a caller can observe: acc_gu / acc_d hold per-k-slice partial sums ([NY, S, 2I] and [NY, S, H]) instead of
     atomically accumulated [S, 2I] / [S, H], so they are not zero between calls and outputs are bitwise repeatable;
-    cnt_gu, cnt_d, wq, zd, cnt_h exist for attribute compatibility and stay zero."""
+    cnt_gu / cnt_d are the arrival counters (zero on entry, zero on exit); wq, zd, cnt_h exist for attribute
+    compatibility and stay zero."""
 
     def __init__(s, E, H, I, nm_gu=0, nm_dn=0, Bmax=4, topk=8, G=4, dev="cuda", mod=None):
         if G != 4:
@@ -174,7 +175,9 @@ class MoELayer:
         a = _lib.NqMoeArgs()
         a.x, a.sel, a.rw, a.table, a.out = x.data_ptr(), sel.data_ptr(), rw.data_ptr(), tb.data_ptr(), out.data_ptr()
         a.acc_gu, a.h, a.acc_d, a.hits = s.acc_gu.data_ptr(), s.h.data_ptr(), s.acc_d.data_ptr(), s.hits_ptr or None
+        a.cnt_gu, a.cnt_d = s.cnt_gu.data_ptr(), s.cnt_d.data_ptr()
         a.acc_gu_elems, a.acc_d_elems, a.h_elems, a.out_elems = s.acc_gu.numel(), s.acc_d.numel(), s.h.numel(), out.numel()
+        a.cnt_gu_elems, a.cnt_d_elems = s.cnt_gu.numel(), s.cnt_d.numel()
         a.B, a.topk, a.E, a.H, a.I = B, topk, tb.shape[0], x.shape[1], s.I
         a.cfg_gu = (C.c_int32 * 4)(*(cg + [0] * (4 - len(cg)))); a.cfg_dn = (C.c_int32 * 4)(*(cd + [0] * (4 - len(cd))))
         a.force_level, a.which = force_level, which

@@ -62,7 +62,7 @@ def test_small_layer_all_levels_and_codes_vs_full_oracle():
             rw[1, 2] = 0
         x = (torch.randn(B, H, generator=g) * 0.05).half().to(DEV)
         want = oracle_layer(planes, levels, signs, x, sel, rw)
-        for cg, cd in (([1, 4, 2], [1, 4, 2]), ([1, 1, 1], [2, 2, 1]), ([2, 8, 2], [1, 8, 1])):
+        for cg, cd in (([1, 4, 2], [1, 4, 2]), ([1, 1, 1], [2, 2, 1]), ([2, 4, 2], [1, 2, 1])):
             y = L(x, sel, rw, cfg_gu=cg, cfg_dn=cd).clone()
             y2 = L(x, sel, rw, cfg_gu=cg, cfg_dn=cd).clone()
             torch.cuda.synchronize()
@@ -123,7 +123,7 @@ def test_full_shape_layer_like_reference_check():
             sel, rw = RT.routing_tensors(rows, seed=B)
             x = (torch.randn(B, H, device=DEV) * 0.05).half()
             want = O.moe_forward(dense, levels, lambda e: signs[e], x.cpu().numpy(), sel.cpu().numpy(), rw.cpu().numpy())
-            for cg, cd in (([1, 4, 6], [1, 4, 4]), ([2, 8, 4], [2, 8, 4]), ([1, 2, 12], [1, 8, 2])):
+            for cg, cd in (([1, 4, 6], [1, 4, 4]), ([2, 4, 4], [2, 4, 4]), ([1, 2, 12], [1, 1, 2])):
                 y = L(x, sel, rw, cfg_gu=cg, cfg_dn=cd)
                 torch.cuda.synchronize()
                 err = rel_err(y.cpu().numpy(), want)
@@ -171,6 +171,8 @@ def test_argument_errors():
     rw = torch.zeros(2, 4, dtype=torch.float16, device=DEV)
     with pytest.raises(RuntimeError, match="bad cfg"):
         L(x, sel, rw, cfg_gu=[1, 4, 3])
+    with pytest.raises(RuntimeError, match="sb must be"):
+        L(x, sel, rw, cfg_gu=[1, 8, 2])
     with pytest.raises(RuntimeError, match="persistent"):
         L(x, sel, rw, cfg_gu=[1, 4, 2, 1])
     with pytest.raises(RuntimeError, match="B="):
@@ -178,8 +180,11 @@ def test_argument_errors():
           torch.zeros(9, 4, dtype=torch.float16, device=DEV), out=torch.zeros(9, 256, device=DEV))
     with pytest.raises(AssertionError):
         L(x.float(), sel, rw)
+    L.out.fill_(7.0)
     y = L(x, sel, rw)                                            # all weights zero -> zeros, no fault
+    torch.cuda.synchronize()
     assert not y.any()
+    assert not L.cnt_gu.any() and not L.cnt_d.any()              # counters are zero again after every call
 
 
 def test_mailbox_kernel_matches_state_machine():
