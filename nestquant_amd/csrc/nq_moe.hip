@@ -22,6 +22,14 @@
 
 namespace nq {
 
+// Partial sums cross workgroups (and XCDs, whose L2s are not coherent with each other) inside one kernel. They are
+// written and read with device-scope relaxed atomics (sc1: write-through / read-through to the device coherence point)
+// and ordered by "all my stores are acknowledged (vmcnt 0) -> bump the group's arrival counter". A full device-scope
+// fence would also be correct but writes back and invalidates the whole L2 once per workgroup, which costs several times
+// the kernel's own run time.
+__device__ __forceinline__ void st_dev(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ float ld_dev(const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+
 constexpr int MAXTOK = 16;                     // MFMA N: tokens of one run (B <= 8 -> at most 8 with distinct top-k ids)
 struct RunInfo { int e, level, ntok, nruns; int slot[MAXTOK]; const int64_t* ent; };
 
@@ -168,8 +176,7 @@ __device__ __forceinline__ void finish_gu(const MoeArgs& a, const RunInfo& R, in
         for (int y = 0; y < NY; ++y)
         {
             const float* p = a.part_gu + ((size_t)y * S + s) * 2 * a.I + col;
-            const float2 pg = *(const float2*)p, pu = *(const float2*)(p + a.I);
-            g0 += pg.x; g1 += pg.y; u0 += pu.x; u1 += pu.y;
+            g0 += ld_dev(p); g1 += ld_dev(p + 1); u0 += ld_dev(p + a.I); u1 += ld_dev(p + a.I + 1);
         }
         wht128(g0, g1, lane); wht128(u0, u1, lane);
         const half2_t svg = *(const half2_t*)(sv_g + col), svu = *(const half2_t*)(sv_u + col), sud = *(const half2_t*)(su_d + col);
@@ -177,7 +184,7 @@ __device__ __forceinline__ void finish_gu(const MoeArgs& a, const RunInfo& R, in
         float v0 = g0 / (1.f + __expf(-g0)) * u0 * (float)sud.x, v1 = g1 / (1.f + __expf(-g1)) * u1 * (float)sud.y;
         wht128(v0, v1, lane);
         half2_t hv; hv.x = (_Float16)v0; hv.y = (_Float16)v1;
-        *(half2_t*)(a.h + (size_t)s * a.I + col) = hv;
+        *(half2_t*)(a.h + (size_t)s * a.I + col) = hv;           // read by the next kernel on the stream
     }
 }
 
@@ -200,8 +207,8 @@ __device__ __forceinline__ void finish_dn(const MoeArgs& a, int grp, int NY, int
             float v0 = 0.f, v1 = 0.f;
             for (int y = 0; y < NY; ++y)
             {
-                const float2 p = *(const float2*)(a.part_d + ((size_t)y * S + s) * a.H + col);
-                v0 += p.x; v1 += p.y;
+                const float* p = a.part_d + ((size_t)y * S + s) * a.H + col;
+                v0 += ld_dev(p); v1 += ld_dev(p + 1);
             }
             wht128(v0, v1, lane);
             const half2_t sv = *(const half2_t*)((const _Float16*)ent[9] + a.H + 3 * a.I + col);
@@ -298,8 +305,8 @@ __global__ void __launch_bounds__(256) nq_gemv_k(MoeArgs a, int NC)
         const int S = a.B * a.topk;
         float* part = (MODE == 0 ? a.part_gu : a.part_d) + ((size_t)blockIdx.y * S + R.slot[n]) * N;
         const int row = 16 * (2 * (blockIdx.x * SB + warp) + (t4 >> 1)) + 4 * (t4 & 1);
-        *(float4_t*)(part + row) = acc[0];
-        *(float4_t*)(part + row + 8) = acc[1];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { st_dev(part + row + i, acc[0][i]); st_dev(part + row + 8 + i, acc[1][i]); }
     }
 
     // ---- arrival counter of the 128-row group this block belongs to; the last block to arrive finishes the group
@@ -307,13 +314,12 @@ __global__ void __launch_bounds__(256) nq_gemv_k(MoeArgs a, int NC)
     const int grp = MODE == 0 ? (rows0 % a.I) / 128 : rows0 / 128;
     int* cnt = MODE == 0 ? a.cnt_gu + blockIdx.z * (a.I / 128) + grp : a.cnt_d + grp;
     const int expect = (MODE == 0 ? 2 : nruns) * NY * (128 / (SB * 32));
-    __threadfence();                                             // release: this block's partial sums are visible device-wide
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");             // this wavefront's partial sums are acknowledged
     __syncthreads();
     if (threadIdx.x == 0)
-        last = __hip_atomic_fetch_add(cnt, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) == expect - 1;
+        last = __hip_atomic_fetch_add(cnt, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == expect - 1;
     __syncthreads();
     if (!last) return;                                           // block-uniform
-    __threadfence();                                             // acquire: every other block's partial sums
     if constexpr (MODE == 0) finish_gu(a, R, grp, NY, warp, SB, lane);
     else finish_dn(a, grp, NY, warp, SB, lane, (float*)smem);
     if (threadIdx.x == 0) __hip_atomic_store(cnt, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
