@@ -27,8 +27,38 @@ namespace nq {
 // and ordered by "all my stores are acknowledged (vmcnt 0) -> bump the group's arrival counter". A full device-scope
 // fence would also be correct but writes back and invalidates the whole L2 once per workgroup, which costs several times
 // the kernel's own run time.
-__device__ __forceinline__ void st_dev(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-__device__ __forceinline__ float ld_dev(const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+// The compiler waits after every atomic load, which serialises the finisher's reads (one memory round trip per k-slice),
+// so the loads are issued as a batch of sc0 sc1 loads and waited for once; the wait names the destination registers so
+// that no use can move above it.
+__device__ __forceinline__ void st_dev4(float* p, float4_t v)
+{
+    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" :: "v"(p), "v"(v) : "memory");
+}
+__device__ __forceinline__ float2 ld_dev2_issue(const float* p)
+{
+    float2 v;
+    asm volatile("global_load_dwordx2 %0, %1, off sc0 sc1" : "=v"(v) : "v"(p) : "memory");
+    return v;
+}
+__device__ __forceinline__ void ld_wait(float2& a, float2& b, float2& c, float2& d)
+{
+    asm volatile("s_waitcnt vmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d) :: "memory");
+}
+// sum over k-slices y of the two floats at p + y * stride (device-coherent reads, four in flight at a time)
+__device__ __forceinline__ float2 sum_partials(const float* p, size_t stride, int NY)
+{
+    float2 acc = make_float2(0.f, 0.f);
+    for (int y = 0; y < NY; y += 4)
+    {
+        float2 v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = ld_dev2_issue(p + (size_t)(y + i < NY ? y + i : y) * stride);
+        ld_wait(v[0], v[1], v[2], v[3]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) if (y + i < NY) { acc.x += v[i].x; acc.y += v[i].y; }
+    }
+    return acc;
+}
 
 constexpr int MAXTOK = 16;                     // MFMA N: tokens of one run (B <= 8 -> at most 8 with distinct top-k ids)
 struct RunInfo { int e, level, ntok, nruns; int slot[MAXTOK]; const int64_t* ent; };
@@ -172,12 +202,9 @@ __device__ __forceinline__ void finish_gu(const MoeArgs& a, const RunInfo& R, in
     for (int j = warp; j < R.ntok; j += SB)
     {
         const int s = R.slot[j];
-        float g0 = 0.f, g1 = 0.f, u0 = 0.f, u1 = 0.f;
-        for (int y = 0; y < NY; ++y)
-        {
-            const float* p = a.part_gu + ((size_t)y * S + s) * 2 * a.I + col;
-            g0 += ld_dev(p); g1 += ld_dev(p + 1); u0 += ld_dev(p + a.I); u1 += ld_dev(p + a.I + 1);
-        }
+        const float* p = a.part_gu + (size_t)s * 2 * a.I + col;
+        const float2 pg = sum_partials(p, (size_t)S * 2 * a.I, NY), pu = sum_partials(p + a.I, (size_t)S * 2 * a.I, NY);
+        float g0 = pg.x, g1 = pg.y, u0 = pu.x, u1 = pu.y;
         wht128(g0, g1, lane); wht128(u0, u1, lane);
         const half2_t svg = *(const half2_t*)(sv_g + col), svu = *(const half2_t*)(sv_u + col), sud = *(const half2_t*)(su_d + col);
         g0 *= (float)svg.x; g1 *= (float)svg.y; u0 *= (float)svu.x; u1 *= (float)svu.y;
@@ -204,12 +231,8 @@ __device__ __forceinline__ void finish_dn(const MoeArgs& a, int grp, int NY, int
             if (ee < 0 || ee >= a.E || w == 0.f) continue;
             const int64_t* ent = a.table + (size_t)ee * TBL_W;
             if (ent[0] <= 0) continue;
-            float v0 = 0.f, v1 = 0.f;
-            for (int y = 0; y < NY; ++y)
-            {
-                const float* p = a.part_d + ((size_t)y * S + s) * a.H + col;
-                v0 += ld_dev(p); v1 += ld_dev(p + 1);
-            }
+            const float2 pv = sum_partials(a.part_d + (size_t)s * a.H + col, (size_t)S * a.H, NY);
+            float v0 = pv.x, v1 = pv.y;
             wht128(v0, v1, lane);
             const half2_t sv = *(const half2_t*)((const _Float16*)ent[9] + a.H + 3 * a.I + col);
             o0 += w * (v0 * (float)sv.x); o1 += w * (v1 * (float)sv.y);
@@ -305,8 +328,8 @@ __global__ void __launch_bounds__(256) nq_gemv_k(MoeArgs a, int NC)
         const int S = a.B * a.topk;
         float* part = (MODE == 0 ? a.part_gu : a.part_d) + ((size_t)blockIdx.y * S + R.slot[n]) * N;
         const int row = 16 * (2 * (blockIdx.x * SB + warp) + (t4 >> 1)) + 4 * (t4 & 1);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) { st_dev(part + row + i, acc[0][i]); st_dev(part + row + 8 + i, acc[1][i]); }
+        st_dev4(part + row, acc[0]);
+        st_dev4(part + row + 8, acc[1]);
     }
 
     // ---- arrival counter of the 128-row group this block belongs to; the last block to arrive finishes the group
