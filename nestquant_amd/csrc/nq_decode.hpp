@@ -28,6 +28,17 @@ constexpr uint32_t MUL1_B2 = 0xc931c931u;       // fp16 B twice
 constexpr int CODE_L3 = 10, CODE_L4N = 11;      // nested planes of this build: K=1 plane; P3 record || P4 record
 constexpr int NCODES = 12;
 
+// plane pointers come out of int64 table words; naming the global address space keeps their loads off the flat path
+// (flat loads also tick the LDS counter, so a prefetch in flight would stall every LDS read behind it)
+#define NQ_GLOBAL __attribute__((address_space(1)))
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));   // native vectors: loadable through any address space
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef const NQ_GLOBAL u32x4* gp_u4;
+typedef const NQ_GLOBAL u32x2* gp_u2;
+typedef const NQ_GLOBAL uint32_t* gp_u32;
+typedef const NQ_GLOBAL uint16_t* gp_u16;
+typedef const NQ_GLOBAL uint8_t* gp_u8;
+
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
@@ -73,12 +84,12 @@ __host__ inline int rec_bits(int code)
 // BITS % 16 bits per record bit-packed over records (reference sm120/moe.py:36-49, sm120/nqmoe.cu:17-20).
 // Code 11 stores its 128-bit record as uint2 (plane P3) | uint2 (plane P4).
 template <int CODE>
-__device__ __forceinline__ void load_record(uint32_t* w, const uint8_t* __restrict__ p, size_t rec, size_t nrec)
+__device__ __forceinline__ void load_record(uint32_t* w, gp_u8 p, size_t rec, size_t nrec)
 {
     constexpr int BITS = Rec<CODE>::BITS;
     if constexpr (Pat<CODE>::SPLIT)
     {
-        const uint2 a = ((const uint2*)p)[rec], b = ((const uint2*)(p + nrec * 8))[rec];
+        const u32x2 a = ((gp_u2)p)[rec], b = ((gp_u2)(p + nrec * 8))[rec];
         w[0] = a.x; w[1] = a.y; w[2] = b.x; w[3] = b.y;
     }
     else
@@ -89,17 +100,17 @@ __device__ __forceinline__ void load_record(uint32_t* w, const uint8_t* __restri
 #pragma unroll
         for (int i = 0; i < n4; ++i)
         {
-            const uint4 v = ((const uint4*)p)[rec * n4 + i];
+            const u32x4 v = ((gp_u4)p)[rec * n4 + i];
             w[k++] = v.x; w[k++] = v.y; w[k++] = v.z; w[k++] = v.w;
         }
         p += nrec * 16 * n4;
-        if constexpr (n2) { const uint2 v = ((const uint2*)p)[rec]; w[k++] = v.x; w[k++] = v.y; p += nrec * 8; }
-        if constexpr (n1) { w[k++] = ((const uint32_t*)p)[rec]; p += nrec * 4; }
-        if constexpr (nh) { w[k++] = ((const uint16_t*)p)[rec]; p += nrec * 2; }
+        if constexpr (n2) { const u32x2 v = ((gp_u2)p)[rec]; w[k++] = v.x; w[k++] = v.y; p += nrec * 8; }
+        if constexpr (n1) { w[k++] = ((gp_u32)p)[rec]; p += nrec * 4; }
+        if constexpr (nh) { w[k++] = ((gp_u16)p)[rec]; p += nrec * 2; }
         if constexpr (T)
         {
             const size_t b = rec * T;
-            const uint32_t* q = (const uint32_t*)p + (b >> 5);
+            gp_u32 q = (gp_u32)p + (b >> 5);
             const int sh = (int)(b & 31);
             uint32_t v;
             if constexpr (32 % T) v = __builtin_amdgcn_alignbit(q[1], q[0], sh);   // q[1] lies inside the 4-byte pad
@@ -216,13 +227,13 @@ __device__ __forceinline__ uint32_t weight_pair(const uint32_t* wb, const uint32
 //   [0] level 0/2/3/4  [1..4] gate|up base, residual plane, block words, flags  [5..8] down  [9] sign/scale vector
 //   [10],[11] residual window code of gate|up, down  [12],[13] sign-variant planes  [14..17] low-rank plane (unsupported)
 //   [18] in_had_down (unsupported unless 0/128)  [19] base codes (unsupported unless 0)
-struct Planes { const uint4* base; const uint8_t* res; const uint32_t* dw; const uint8_t* var; int code; };
+struct Planes { gp_u4 base; gp_u8 res; gp_u32 dw; gp_u8 var; int code; };
 __device__ __forceinline__ Planes planes_of(const int64_t* ent, int mode)
 {
     const int o = mode == 0 ? 1 : 5;
     Planes P;
-    P.base = (const uint4*)ent[o]; P.res = (const uint8_t*)ent[o + 1]; P.dw = (const uint32_t*)ent[o + 2];
-    P.var = (const uint8_t*)ent[mode == 0 ? 12 : 13]; P.code = (int)ent[10 + mode];
+    P.base = (gp_u4)ent[o]; P.res = (gp_u8)ent[o + 1]; P.dw = (gp_u32)ent[o + 2];
+    P.var = (gp_u8)ent[mode == 0 ? 12 : 13]; P.code = (int)ent[10 + mode];
     return P;
 }
 

@@ -41,7 +41,7 @@ __device__ __forceinline__ void decode_unit(const Planes& P, int lv, size_t unit
     const int src = (lane & ~3) | ((lane + 1) & 3);           // next lane of the ring
     uint32_t wb[6];
     {
-        const uint4 v = P.base[unit * 32 + lane32];
+        const u32x4 v = P.base[unit * 32 + lane32];
         wb[0] = v.x; wb[1] = v.y; wb[2] = v.z; wb[3] = v.w;
         ext_words<128, 4>(wb, __shfl(wb[0], src));
     }

@@ -139,7 +139,7 @@ __device__ __forceinline__ half8_t a_operand(const uint32_t* wb, const uint32_t*
     u[1] = weight_pair<RES, CODE, J + 1, J + 9>(wb, wr, k);
     u[2] = weight_pair<RES, CODE, J + 4, J + 12>(wb, wr, k);
     u[3] = weight_pair<RES, CODE, J + 5, J + 13>(wb, wr, k);
-    return __builtin_bit_cast(half8_t, *(uint4*)u);
+    return __builtin_bit_cast(half8_t, *(u32x4*)u);
 }
 
 struct LaneCtx
@@ -154,10 +154,9 @@ struct LaneCtx
 };
 
 template <bool RES, int CODE>
-__device__ __forceinline__ void gemv_chunks(const Planes& P, const LaneCtx& L, int NC, float4_t* acc)
+__device__ __forceinline__ void gemv_chunks(const Planes& P, const LaneCtx& L, int NC, float4_t* acc, u32x4 nb)
 {
     constexpr int NW = RES ? Rec<CODE>::NW : 1;
-    uint4 nb = P.base[L.rec0];
     uint32_t nr[NW + 2] = {0}, ndw = 0, nvar = 0;
     if constexpr (RES) { load_record<CODE>(nr, P.res, L.rec0, L.nrec); ndw = P.dw[L.unit0]; }
     if (P.var) nvar = P.var[L.unit0];
@@ -280,6 +279,17 @@ __global__ void __launch_bounds__(256) nq_gemv_k(MoeArgs a, int NC)
     char* zero = smem + ntok * rowstride;                        // 256 zero bytes after the token rows
     const _Float16* signs = (const _Float16*)R.ent[9];
 
+    // ---- lane context; the first base record is requested now so that its latency overlaps the staging below
+    const int t4 = lane >> 4, ss = (lane >> 3) & 1, g = lane & 7, n = lane & 15;
+    const int strip = 2 * (blockIdx.x * SB + warp) + ss;
+    const Planes P = planes_of(R.ent, MODE);
+    LaneCtx L;
+    L.unit0 = (size_t)strip * C + chunk0; L.rec0 = L.unit0 * 32 + 4 * g + t4;
+    L.nrec = (size_t)(N / 16) * C * 32;
+    L.src = (lane + 16) & 63; L.g = g;
+    L.xs = (n < ntok ? smem + n * rowstride : zero) + t4 * 16; L.xstep = n < ntok ? 256 : 0;
+    const u32x4 nb0 = P.base[L.rec0];
+
     // ---- stage the run's tokens for this k-slice in B-operand order
     if constexpr (MODE == 0)
     {
@@ -310,17 +320,9 @@ __global__ void __launch_bounds__(256) nq_gemv_k(MoeArgs a, int NC)
     __syncthreads();
 
     // ---- decode + MFMA over the k-slice
-    const int t4 = lane >> 4, ss = (lane >> 3) & 1, g = lane & 7, n = lane & 15;
-    const int strip = 2 * (blockIdx.x * SB + warp) + ss;
-    const Planes P = planes_of(R.ent, MODE);
-    LaneCtx L;
-    L.unit0 = (size_t)strip * C + chunk0; L.rec0 = L.unit0 * 32 + 4 * g + t4;
-    L.nrec = (size_t)(N / 16) * C * 32;
-    L.src = (lane + 16) & 63; L.g = g;
-    L.xs = (n < ntok ? smem + n * rowstride : zero) + t4 * 16; L.xstep = n < ntok ? 256 : 0;
     float4_t acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
-    if (R.level == 2) gemv_chunks<false, 0>(P, L, NC, acc);
-    else dispatch_code(P.code, [&](auto tag) { gemv_chunks<true, decltype(tag)::value>(P, L, NC, acc); });
+    if (R.level == 2) gemv_chunks<false, 0>(P, L, NC, acc, nb0);
+    else dispatch_code(P.code, [&](auto tag) { gemv_chunks<true, decltype(tag)::value>(P, L, NC, acc, nb0); });
 
     // ---- k-slice partial sums: lane (t4, n) holds rows 16 (strip0 + t4 / 2) + 4 (t4 & 1) + i (+ 8 for acc[1]) of token n
     if (n < ntok)
