@@ -319,10 +319,10 @@ def hadamard(n=128):
     return (H / np.sqrt(n)).astype(np.float32)
 
 
-def wht(v, n=128):
-    """Hadamard-n on each n-block of the last axis (fp32)"""
-    v = np.asarray(v, np.float32)
-    return (v.reshape(*v.shape[:-1], -1, n) @ hadamard(n)).reshape(v.shape)
+def wht(v, n=128, dtype=np.float32):
+    """Hadamard-n on each n-block of the last axis (fp32 unless dtype says otherwise)"""
+    v = np.asarray(v, dtype)
+    return (v.reshape(*v.shape[:-1], -1, n) @ hadamard(n).astype(dtype)).reshape(v.shape)
 
 
 def split_signs(signs, H, I):
@@ -333,26 +333,29 @@ def split_signs(signs, H, I):
     return {n: s[o[i]:o[i + 1]] for i, n in enumerate(names)}
 
 
-def expert_forward(x, Wgu, Wdn, signs, round_acts=True):
-    """x [T,H] fp32 through dense weights Wgu [2I,H], Wdn [H,I] (fp32 arrays holding fp16 values) -> [T,H] fp32.
-    round_acts: round the two rotated activations to fp16 as the kernels do (False = pure fp32 pipeline)."""
+def expert_forward(x, Wgu, Wdn, signs, round_acts=True, dtype=np.float32):
+    """x [T,H] through dense weights Wgu [2I,H], Wdn [H,I] (arrays holding fp16 values) -> [T,H].
+    round_acts: round the two rotated activations to fp16 as the kernels do (False = no activation rounding).
+    dtype: arithmetic type; float64 gives the exact-arithmetic arbiter used to separate rounding noise from errors."""
     H, I = Wdn.shape
-    sg = split_signs(signs, H, I)
-    rnd = (lambda a: a.astype(np.float16).astype(np.float32)) if round_acts else (lambda a: a)
-    x = np.asarray(x, np.float32)
-    xg = rnd(wht(x * sg["su_g"])); xu = rnd(wht(x * sg["su_u"]))
-    g = wht(xg @ Wgu[:I].T) * sg["sv_g"]
-    u = wht(xu @ Wgu[I:].T) * sg["sv_u"]
+    sg = {k: v.astype(dtype) for k, v in split_signs(signs, H, I).items()}
+    rnd = (lambda a: a.astype(np.float16).astype(dtype)) if round_acts else (lambda a: a)
+    x = np.asarray(x, dtype)
+    Wgu = np.asarray(Wgu, dtype); Wdn = np.asarray(Wdn, dtype)
+    wht_ = lambda v: wht(v, 128, dtype)
+    xg = rnd(wht_(x * sg["su_g"])); xu = rnd(wht_(x * sg["su_u"]))
+    g = wht_(xg @ Wgu[:I].T) * sg["sv_g"]
+    u = wht_(xu @ Wgu[I:].T) * sg["sv_u"]
     with np.errstate(over="ignore"):                       # exp overflow gives the correct limit silu(-inf) = -0
         sw = g / (1.0 + np.exp(-g)) * u
-    h = rnd(wht(sw * sg["su_d"]))
-    return wht(h @ Wdn.T) * sg["sv_o"]
+    h = rnd(wht_(sw * sg["su_d"]))
+    return wht_(h @ Wdn.T) * sg["sv_o"]
 
 
-def moe_forward(dense, levels, signs, x, sel, rw, round_acts=True):
+def moe_forward(dense, levels, signs, x, sel, rw, round_acts=True, dtype=np.float32):
     """dense: callable e -> (Wgu fp32 [2I,H], Wdn fp32 [H,I]) at the expert's level; levels [E]; signs: e -> vector.
     x [B,H] fp16/fp32, sel [B,topk] int, rw [B,topk] fp16 -> [B,H] fp32. Picks with rw == 0 or level <= 0 add 0."""
-    x = np.asarray(x, np.float32)
+    x = np.asarray(x, dtype)
     out = np.zeros_like(x)
     cache = {}
     for b in range(x.shape[0]):
@@ -363,7 +366,7 @@ def moe_forward(dense, levels, signs, x, sel, rw, round_acts=True):
             if e not in cache:
                 cache[e] = dense(e)
             Wgu, Wdn = cache[e]
-            out[b] += np.float32(w) * expert_forward(x[b:b + 1], Wgu, Wdn, signs(e), round_acts)[0]
+            out[b] += dtype(w) * expert_forward(x[b:b + 1], Wgu, Wdn, signs(e), round_acts, dtype)[0]
     return out
 
 

@@ -1,8 +1,11 @@
 """Decode-path MoE layer (nq_moe_forward through the C ABI) against the oracle's layer math.
 
-Tolerances: 1e-4 relative (L2) against the oracle pipeline with the same two fp16 activation roundings -- the band the
-reference's own kernel shows against its torch reference (1.4e-5 .. 9.8e-5, sm120/results/check_I512.txt) -- and 1e-3
-against an fp32 pipeline without those roundings (the north-star gate)."""
+Tolerances: 5e-5 relative (L2) against the oracle pipeline evaluated in float64 with the same two fp16 activation
+roundings. The reference's own kernel sits 1.4e-5 .. 9.8e-5 from its fp32 torch reference
+(sm120/results/check_I512.txt); most of that band is the fp32 reference's own summation error (measured here: the fp32
+numpy oracle is up to 3e-4 from the float64 one on these planes, whose 5% extreme block words give weights in the
+thousands), so the float64 oracle is the arbiter and the kernel is expected within ~1e-5 of it. The north-star gate --
+1e-3 against an fp32 matmul pipeline without the activation roundings -- is asserted separately."""
 import random
 
 import numpy as np
@@ -37,6 +40,7 @@ def oracle_layer(ex_cpu_planes, levels, signs, x, sel, rw, **kw):
     def dense(e):
         pg, pd, nested = ex_cpu_planes[e]
         return (O.dense_W(pg, levels[e], nested=nested).astype(np.float32), O.dense_W(pd, levels[e], nested=nested).astype(np.float32))
+    kw.setdefault("dtype", np.float64)
     return O.moe_forward(dense, levels, lambda e: signs[e], x.cpu().numpy(), sel.cpu().numpy(), rw.cpu().numpy(), **kw)
 
 
@@ -66,9 +70,9 @@ def test_small_layer_all_levels_and_codes_vs_full_oracle():
             y = L(x, sel, rw, cfg_gu=cg, cfg_dn=cd).clone()
             y2 = L(x, sel, rw, cfg_gu=cg, cfg_dn=cd).clone()
             torch.cuda.synchronize()
-            assert rel_err(y.cpu().numpy(), want) < 1e-4, (B, cg, cd)
+            assert rel_err(y.cpu().numpy(), want) < 5e-5, (B, cg, cd)
             assert torch.equal(y, y2)                              # partial sums, no atomics: bitwise repeatable
-        pure = oracle_layer(planes, levels, signs, x, sel, rw, round_acts=False)
+        pure = oracle_layer(planes, levels, signs, x, sel, rw, round_acts=False, dtype=np.float32)
         assert rel_err(y.cpu().numpy(), pure) < 1e-3
 
 
@@ -85,7 +89,7 @@ def test_golden_layer_fixture(golden_dir):
     sel = torch.from_numpy(z["sel"]).to(DEV); rw = torch.from_numpy(z["rw"].view(np.float16).copy()).to(DEV)
     y = L(x, sel, rw)
     torch.cuda.synchronize()
-    assert rel_err(y.cpu().numpy(), z["y"]) < 1e-4
+    assert rel_err(y.cpu().numpy(), z["y"]) < 1e-4               # the fixture is the reference's fp32 torch result
 
 
 def _dense_from_gpu(ex, levels):
@@ -111,6 +115,7 @@ def test_full_shape_layer_like_reference_check():
     dense = _dense_from_gpu(ex, levels)
     signs = [e.signs.cpu().numpy() for e in ex]
     rng = random.Random(0)
+    gx = torch.Generator().manual_seed(3)
     worst = 0.0
     for B in (1, 2, 3, 4):
         for mode in ("recency", "distinct", "same"):
@@ -121,15 +126,19 @@ def test_full_shape_layer_like_reference_check():
             else:
                 rows = RT.make_sel(B, range(NE), mode, p=0.5, rng=rng)
             sel, rw = RT.routing_tensors(rows, seed=B)
-            x = (torch.randn(B, H, device=DEV) * 0.05).half()
-            want = O.moe_forward(dense, levels, lambda e: signs[e], x.cpu().numpy(), sel.cpu().numpy(), rw.cpu().numpy())
+            x = (torch.randn(B, H, generator=gx) * 0.05).half().to(DEV)
+            a = (x.cpu().numpy(), sel.cpu().numpy(), rw.cpu().numpy())
+            want = O.moe_forward(dense, levels, lambda e: signs[e], *a, dtype=np.float64)
+            pure = O.moe_forward(dense, levels, lambda e: signs[e], *a, round_acts=False)
             for cg, cd in (([1, 4, 6], [1, 4, 4]), ([2, 4, 4], [2, 4, 4]), ([1, 2, 12], [1, 1, 2])):
                 y = L(x, sel, rw, cfg_gu=cg, cfg_dn=cd)
                 torch.cuda.synchronize()
                 err = rel_err(y.cpu().numpy(), want)
                 worst = max(worst, err)
-                assert err < 1e-4, (B, mode, cg, cd, err)
-    print("worst rel err", worst)
+                assert err < 5e-5, (B, mode, cg, cd, err)
+                assert rel_err(y.cpu().numpy(), pure) < 1e-3, (B, mode, cg, cd)
+    assert not L.cnt_gu.any() and not L.cnt_d.any()              # workspace counters are clean after the calls
+    print("worst rel err vs the float64 oracle", worst)
 
 
 def test_force_level_which_hits_and_out_of_range_ids():
@@ -143,10 +152,10 @@ def test_force_level_which_hits_and_out_of_range_ids():
     signs = [e.signs.cpu().numpy() for e in ex]
     for lv in (2, 4):                                            # rows are level 4; force_level = 2 must read the base only
         dense = _dense_from_gpu(ex, [lv] * NE)
-        want = O.moe_forward(dense, [lv] * NE, lambda e: signs[e], x.cpu().numpy(), sel.cpu().numpy(), rw.cpu().numpy())
+        want = O.moe_forward(dense, [lv] * NE, lambda e: signs[e], x.cpu().numpy(), sel.cpu().numpy(), rw.cpu().numpy(), dtype=np.float64)
         y = L(x, sel, rw, force_level=lv)
         torch.cuda.synchronize()
-        assert rel_err(y.cpu().numpy(), want) < 1e-4, lv
+        assert rel_err(y.cpu().numpy(), want) < 5e-5, lv
     # which = 1 then which = 2 equals which = 3
     y3 = L(x, sel, rw).clone()
     L(x, sel, rw, which=1); y12 = L(x, sel, rw, which=2).clone()
