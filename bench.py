@@ -121,12 +121,20 @@ def main():
     ap.add_argument("--warmup", type=int, default=32)
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calib", action="store_true", help="also run one 256 MiB device copy (reads 256 MiB, writes 256 MiB): "
+                    "the known-size kernel that scales rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py measures one GPU holding one full MoE layer; --gpus N > 1 is not part of this build")
     dev = "cuda"
     torch.cuda.set_device(0)
     B, K, W = a.batch, a.steps, a.warmup
+    if a.calib:
+        src = torch.ones(64 * 1024 * 1024, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     L, MB, ex, levels = build_layer(dev, Bmax=max(4, B))
     R = 64
     routes = make_routings(B, R, dev)
