@@ -26,6 +26,9 @@ from nestquant_amd import format as F, moe as M, routing as RT  # noqa: E402
 
 H, I, E, TOPK = 6144, 2048, 256, 8
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per gate|up launch / algorithmic bytes, from rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a 256 MiB copy kernel
+# (profiles/decode_gemv_hbm_traffic_pmc.txt)
+TRAFFIC_RATIO = 1.037
 
 
 def build_layer(dev, seed=0, Bmax=4):
@@ -207,7 +210,7 @@ def main():
     kbytes = sum(code_bytes(ex, levels, routes[i][2], "gu") for i in range(R)) / R
     achieved = kbytes / kdt / 1e9
     roofline = dict(bound="hbm", kernel="nq_gemv_k<0> (gate|up decode+GEMV)", achieved=round(achieved, 1), peak=HBM_PEAK_GBS, unit="GB/s",
-                    frac=round(achieved / HBM_PEAK_GBS, 4), traffic=None, us_per_launch=round(kdt * 1e6, 2),
+                    frac=round(achieved / HBM_PEAK_GBS, 4), traffic=int(kbytes * TRAFFIC_RATIO), us_per_launch=round(kdt * 1e6, 2),
                     algorithmic_bytes_per_launch=int(kbytes))
     cpu = None
     if not a.no_cpu:
