@@ -81,6 +81,37 @@ int nq_moe_forward(const NqMoeArgs* args, void* stream);
 int nq_mailbox(int64_t* table, const int64_t* stage, const int32_t* seq, int32_t* applied, int32_t* applied_host, int E,
                void* stream);
 
+/* ---- prefill (more tokens than a decode call takes): pairs (token, expert) sorted by expert ------------------------------
+ * pt / pe: int32[np] token and expert of each pair; prw: fp16[np] router weight. Pairs whose expert is at level <= 0,
+ * outside [0, E), or whose weight is 0 contribute nothing. Activation buffers xg, xu [np][H] and h [np][I] are fp16 with
+ * every 128-column chunk stored in the MFMA B-operand column order (an internal layout shared by these entry points). */
+
+/* xg / xu = fp16(Hadamard-128(x[pt] * su_g / su_u)). Replaces pf_pre (reference sm120/nqmoe.cu:1082-1117,1258-1267). */
+int nq_pf_pre(const void* x_f16, const int32_t* pt, const int32_t* pe, int np, const int64_t* table, void* xg_f16,
+              void* xu_f16, int E, int H, int I, void* stream);
+
+/* Grouped GEMM with the weights decoded from the trellis planes inside the kernel (level and planes from the live table
+ * row): for every tile t = tiles[t] = {expert, first pair row, rows, 0} (device int32[ntiles][4], rows <= bm,
+ * bm in {16, 32, 64, 128, 256}):  C[row][n] = sum_k A[row][k] * W_expert[n][k]  with fp32 accumulation and output.
+ * mode 0: gate|up, K = H, N = 2I, A0 = xg feeds weight rows [0, I), A1 = xu feeds rows [I, 2I), C = [np][2I];
+ * mode 1: down, K = I, N = H, A0 = h, A1 ignored, C = [np][H]. Replaces pf_decode + the Triton grouped GEMM / aten.mm
+ * (reference sm120/pf_gemm.py:7-34, sm120/moe.py:303-324); decoded weights never touch HBM. */
+int nq_pf_gemm(const int64_t* table, const int32_t* tiles, int ntiles, int bm, int mode, const void* A0_f16,
+               const void* A1_f16, float* C, int E, int H, int I, void* stream);
+
+/* h = fp16(Hadamard(silu(g) * u * su_d)), g = Hadamard(acc_gu[:, :I]) * sv_g, u = Hadamard(acc_gu[:, I:]) * sv_u.
+ * Replaces pf_mid (reference sm120/nqmoe.cu:1119-1203,1268-1277). */
+int nq_pf_mid(const float* acc_gu, const int32_t* pe, int np, const int64_t* table, void* h_f16, int E, int H, int I,
+              void* stream);
+
+/* out[pt[p]] += prw[p] * sv_o (.) Hadamard(y[p]) with float atomics; out fp32 [T][H] must be zeroed by the caller.
+ * Replaces pf_post (reference sm120/nqmoe.cu:1205-1240,1278-1287). */
+int nq_pf_post(const float* y, const int32_t* pt, const int32_t* pe, const void* prw_f16, int np, const int64_t* table,
+               float* out, int E, int H, int I, void* stream);
+
+/* hits[e] += counts[e] (hits may be host-mapped). Replaces pf_hits (reference sm120/nqmoe.cu:1241-1245,1288-1293). */
+int nq_pf_hits(const int32_t* counts, int32_t* hits, int E, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -111,3 +111,52 @@ extern "C" int nq_mailbox(int64_t* table, const int64_t* stage, const int32_t* s
     NQ_REQUIRE(E >= 1, "nq_mailbox: E=%d", E);
     return launch_mailbox(table, stage, seq, applied, applied_host, E, (hipStream_t)stream);
 }
+
+extern "C" int nq_pf_pre(const void* x, const int32_t* pt, const int32_t* pe, int np, const int64_t* table, void* xg, void* xu,
+                         int E, int H, int I, void* stream)
+{
+    NQ_REQUIRE(np >= 0, "nq_pf_pre: np=%d", np);
+    if (np == 0) return 0;
+    NQ_REQUIRE(x && pt && pe && table && xg && xu, "nq_pf_pre: null pointer");
+    NQ_REQUIRE(E >= 1 && shape_ok(H, I), "nq_pf_pre: E=%d H=%d I=%d (H, I positive multiples of 128)", E, H, I);
+    return launch_pf_pre(x, pt, pe, np, table, xg, xu, E, H, I, (hipStream_t)stream);
+}
+
+extern "C" int nq_pf_gemm(const int64_t* table, const int32_t* tiles, int ntiles, int bm, int mode, const void* A0, const void* A1,
+                          float* C, int E, int H, int I, void* stream)
+{
+    NQ_REQUIRE(ntiles >= 0, "nq_pf_gemm: ntiles=%d", ntiles);
+    if (ntiles == 0) return 0;
+    NQ_REQUIRE(table && tiles && A0 && C, "nq_pf_gemm: null pointer");
+    NQ_REQUIRE(mode == 0 || mode == 1, "nq_pf_gemm: mode %d not in {0,1}", mode);
+    NQ_REQUIRE(mode == 1 || A1, "nq_pf_gemm: gate|up needs both activation buffers");
+    NQ_REQUIRE(ntiles <= 65535, "nq_pf_gemm: %d tiles exceed one launch (65535)", ntiles);
+    NQ_REQUIRE(E >= 1 && shape_ok(H, I), "nq_pf_gemm: E=%d H=%d I=%d (H, I positive multiples of 128)", E, H, I);
+    return launch_pf_gemm(table, tiles, ntiles, bm, mode, A0, A1, C, E, H, I, (hipStream_t)stream);
+}
+
+extern "C" int nq_pf_mid(const float* acc_gu, const int32_t* pe, int np, const int64_t* table, void* h, int E, int H, int I, void* stream)
+{
+    NQ_REQUIRE(np >= 0, "nq_pf_mid: np=%d", np);
+    if (np == 0) return 0;
+    NQ_REQUIRE(acc_gu && pe && table && h, "nq_pf_mid: null pointer");
+    NQ_REQUIRE(E >= 1 && shape_ok(H, I), "nq_pf_mid: E=%d H=%d I=%d (H, I positive multiples of 128)", E, H, I);
+    return launch_pf_mid(acc_gu, pe, np, table, h, E, H, I, (hipStream_t)stream);
+}
+
+extern "C" int nq_pf_post(const float* y, const int32_t* pt, const int32_t* pe, const void* prw, int np, const int64_t* table,
+                          float* out, int E, int H, int I, void* stream)
+{
+    NQ_REQUIRE(np >= 0, "nq_pf_post: np=%d", np);
+    if (np == 0) return 0;
+    NQ_REQUIRE(y && pt && pe && prw && table && out, "nq_pf_post: null pointer");
+    NQ_REQUIRE(E >= 1 && shape_ok(H, I), "nq_pf_post: E=%d H=%d I=%d (H, I positive multiples of 128)", E, H, I);
+    return launch_pf_post(y, pt, pe, prw, np, table, out, E, H, I, (hipStream_t)stream);
+}
+
+extern "C" int nq_pf_hits(const int32_t* counts, int32_t* hits, int E, void* stream)
+{
+    NQ_REQUIRE(counts && E >= 1, "nq_pf_hits: null counts or E=%d", E);
+    if (!hits) return 0;
+    return launch_pf_hits(counts, hits, E, (hipStream_t)stream);
+}

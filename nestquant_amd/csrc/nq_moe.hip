@@ -16,9 +16,8 @@
 // pairs are A operands as they leave the decoder, with no cross-lane movement. The B operand (tokens) comes from LDS,
 // staged in the matching column order. Partial sums instead of float atomics make the layer output bitwise repeatable;
 // the arrival counters are zero on entry and are reset by the block that consumes them.
-#include "nq_decode.hpp"
+#include "nq_tile.hpp"
 #include "nq_host.hpp"
-#include <utility>
 
 namespace nq {
 
@@ -102,94 +101,6 @@ __device__ __forceinline__ void route(const MoeArgs& a, int z, RunInfo* R, int l
         rem &= ~m; ++r;
     }
     if (lane == 0) R->nruns = r;
-}
-
-// ---- Hadamard-128 on one wavefront: lane holds elements 2 lane, 2 lane + 1 --------------------------------------------
-__device__ __forceinline__ void wht128(float& a, float& b, int lane)
-{
-    const float s = a + b, d = a - b; a = s; b = d;
-#pragma unroll
-    for (int m = 1; m < 64; m <<= 1)
-    {
-        const float oa = __shfl_xor(a, m), ob = __shfl_xor(b, m);
-        a = (lane & m) ? oa - a : a + oa;
-        b = (lane & m) ? ob - b : b + ob;
-    }
-    a *= 0.08838834764f; b *= 0.08838834764f;
-}
-
-// LDS position (in halfs) of column c of a 128-column chunk in the B-operand order:
-// 16-byte block (mm, kg) holds, for i = 0..3, columns 32 mm + 2 kg + 8 (i >> 1) + (i & 1) and that + 16
-__device__ __forceinline__ int bop_index(int c)
-{
-    const int mm = c >> 5, hi = (c >> 4) & 1, kg = (c >> 1) & 3, i = 2 * ((c >> 3) & 1) + (c & 1);
-    return (mm * 4 + kg) * 8 + 2 * i + hi;
-}
-
-template <int... Is, class F> __device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, Is...>) { (f(CodeTag<Is>{}), ...); }
-template <int N, class F> __device__ __forceinline__ void static_for(F&& f) { static_for_impl(f, std::make_integer_sequence<int, N>{}); }
-
-// A operand of MFMA (MM, RHO): rows g + 8 RHO, columns of t = 2 MM and 2 MM + 1
-template <bool RES, int CODE, int MM, int RHO>
-__device__ __forceinline__ half8_t a_operand(const uint32_t* wb, const uint32_t* wr, const FoldK& k)
-{
-    constexpr int J = 16 * MM + 2 * RHO;
-    uint32_t u[4];
-    u[0] = weight_pair<RES, CODE, J + 0, J + 8>(wb, wr, k);
-    u[1] = weight_pair<RES, CODE, J + 1, J + 9>(wb, wr, k);
-    u[2] = weight_pair<RES, CODE, J + 4, J + 12>(wb, wr, k);
-    u[3] = weight_pair<RES, CODE, J + 5, J + 13>(wb, wr, k);
-    return __builtin_bit_cast(half8_t, *(u32x4*)u);
-}
-
-struct LaneCtx
-{
-    size_t rec0;          // record index of this lane in chunk 0 of its k-slice: (unit0) * 32 + 4 g + t4
-    size_t unit0;         // unit index (strip * C + chunk0)
-    size_t nrec;          // records of the whole projection (sub-array stride)
-    int src;              // lane holding the next record of the ring
-    int g;                // ring index (sign-variant bit)
-    const char* xs;       // this lane's B-operand base in LDS (bytes), kg folded in
-    int xstep;            // bytes per chunk (0 for lanes without a token)
-};
-
-template <bool RES, int CODE>
-__device__ __forceinline__ void gemv_chunks(const Planes& P, const LaneCtx& L, int NC, float4_t* acc, u32x4 nb)
-{
-    constexpr int NW = RES ? Rec<CODE>::NW : 1;
-    uint32_t nr[NW + 2] = {0}, ndw = 0, nvar = 0;
-    if constexpr (RES) { load_record<CODE>(nr, P.res, L.rec0, L.nrec); ndw = P.dw[L.unit0]; }
-    if (P.var) nvar = P.var[L.unit0];
-    for (int c = 0; c < NC; ++c)
-    {
-        uint32_t wb[6], wr[NW + 2];
-        wb[0] = nb.x; wb[1] = nb.y; wb[2] = nb.z; wb[3] = nb.w;
-#pragma unroll
-        for (int i = 0; i < NW; ++i) wr[i] = nr[i];
-        const uint32_t dw = ndw, var = nvar;
-        if (c + 1 < NC)                                         // prefetch the next chunk's records
-        {
-            nb = P.base[L.rec0 + (size_t)(c + 1) * 32];
-            if constexpr (RES) { load_record<CODE>(nr, P.res, L.rec0 + (size_t)(c + 1) * 32, L.nrec); ndw = P.dw[L.unit0 + c + 1]; }
-            if (P.var) nvar = P.var[L.unit0 + c + 1];
-        }
-        ext_words<128, 4>(wb, __shfl(wb[0], L.src));
-        const uint32_t sgm = ((var >> L.g) & 1u) * 0x80008000u;
-        FoldK k;
-        if constexpr (RES)
-        {
-            ext_words<Rec<CODE>::BITS, Rec<CODE>::NW>(wr, __shfl(wr[0], L.src));
-            k = consts_fold(dw, sgm);
-        }
-        else k = consts_l2(sgm);
-        const char* xp = L.xs + c * L.xstep;
-        static_for<4>([&](auto mm) {
-            constexpr int MM = decltype(mm)::value;
-            const half8_t b = *(const half8_t*)(xp + MM * 64);
-            acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_operand<RES, CODE, MM, 0>(wb, wr, k), b, acc[0], 0, 0, 0);
-            acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_operand<RES, CODE, MM, 1>(wb, wr, k), b, acc[1], 0, 0, 0);
-        });
-    }
 }
 
 // finisher of gate|up for (run, 128-column group grp): h[slot] = fp16(WHT(silu(g) * u * su_d)), g = WHT(sum_y part_g) * sv_g

@@ -1,0 +1,276 @@
+// Prefill path (T > 8 tokens): every routed expert's weights are decoded once per 16..256-row tile of its tokens, inside
+// the grouped GEMM itself, never written to HBM (reference: pf_decode to fp16 in HBM + Triton/cuBLAS grouped GEMM,
+// sm120/nqmoe.cu:942-1240, sm120/pf_gemm.py:7-34, sm120/moe.py:282-326).
+//
+//   nq_pf_pre_k   per (token, expert) pair, sorted by expert: xg / xu = fp16(Hadamard-128(x * su_g / su_u)), written in
+//                 B-operand column order so the GEMM stages them with straight 16-byte copies      (reference nq_pf_pre)
+//   nq_pf_gemm_k  C[rows of expert j][N] = A[rows][K] @ W_j[N][K]^T: grid (N / 128, tiles); a tile = (expert, row0, rows
+//                 <= 16 TG). Per 128-column chunk the block stages the tile's activations in LDS while each wavefront
+//                 decodes two strips of the expert's records into MFMA A operands, then runs TG x 8 MFMAs
+//                 (v_mfma_f32_16x16x32_f16, fp32 accumulate) over the staged tokens. Level from the live table row.
+//   nq_pf_mid_k   Hadamard * sv, SwiGLU, * su_d, Hadamard -> h fp16 (B-operand order)               (reference nq_pf_mid)
+//   nq_pf_post_k  out[token] += rw * sv_o (.) Hadamard(y)  (float atomics, as the reference)        (reference nq_pf_post)
+//   nq_pf_hits_k  hits[e] += counts[e]                                                            (reference nq_pf_hits)
+#include "nq_tile.hpp"
+#include "nq_host.hpp"
+
+namespace nq {
+
+constexpr int PF_ROW = 272;                    // LDS bytes per staged token: 256 + 16 (spreads tokens over banks)
+
+// grid (npairs), block 256: wave w handles 128-column groups w, w + 4, ... of gate then up
+__global__ void __launch_bounds__(256) nq_pf_pre_k(const _Float16* __restrict__ x, const int32_t* __restrict__ pt, const int32_t* __restrict__ pe,
+                                                    const int64_t* __restrict__ table, _Float16* xg, _Float16* xu, int E, int H, int I)
+{
+    const int p = blockIdx.x, lane = threadIdx.x & 63, warp = threadIdx.x >> 6;
+    const int e = pe[p];
+    const int ng = H / 128;
+    const bool live = e >= 0 && e < E && table[(size_t)e * TBL_W] > 0;
+    const _Float16* signs = live ? (const _Float16*)table[(size_t)e * TBL_W + 9] : nullptr;
+    const _Float16* xr = x + (size_t)pt[p] * H;
+    for (int task = warp; task < 2 * ng; task += 4)
+    {
+        const int up = task / ng, grp = task % ng, k = grp * 128 + 2 * lane;
+        _Float16* dst = (up ? xu : xg) + (size_t)p * H + grp * 128;
+        float v0 = 0.f, v1 = 0.f;
+        if (live)
+        {
+            const _Float16* su = up ? signs + 2 * H + 3 * I : signs;
+            const half2_t xv = *(const half2_t*)(xr + k), sv = *(const half2_t*)(su + k);
+            v0 = (float)xv.x * (float)sv.x; v1 = (float)xv.y * (float)sv.y;
+            wht128(v0, v1, lane);
+        }
+        dst[bop_index(2 * lane)] = (_Float16)v0; dst[bop_index(2 * lane + 1)] = (_Float16)v1;
+    }
+}
+
+// grid (npairs), block 256: acc_gu [P][2I] fp32 (gate | up) -> h [P][I] fp16 in B-operand order
+__global__ void __launch_bounds__(256) nq_pf_mid_k(const float* __restrict__ acc_gu, const int32_t* __restrict__ pe,
+                                                    const int64_t* __restrict__ table, _Float16* h, int E, int H, int I)
+{
+    const int p = blockIdx.x, lane = threadIdx.x & 63, warp = threadIdx.x >> 6;
+    const int e = pe[p];
+    const bool live = e >= 0 && e < E && table[(size_t)e * TBL_W] > 0;
+    const _Float16* signs = live ? (const _Float16*)table[(size_t)e * TBL_W + 9] : nullptr;
+    for (int grp = warp; grp < I / 128; grp += 4)
+    {
+        const int col = grp * 128 + 2 * lane;
+        _Float16* dst = h + (size_t)p * I + grp * 128;
+        float v0 = 0.f, v1 = 0.f;
+        if (live)
+        {
+            const _Float16 *sv_g = signs + H, *sv_u = sv_g + I, *su_d = sv_u + I;
+            const float2 pg = *(const float2*)(acc_gu + (size_t)p * 2 * I + col), pu = *(const float2*)(acc_gu + (size_t)p * 2 * I + I + col);
+            float g0 = pg.x, g1 = pg.y, u0 = pu.x, u1 = pu.y;
+            wht128(g0, g1, lane); wht128(u0, u1, lane);
+            const half2_t svg = *(const half2_t*)(sv_g + col), svu = *(const half2_t*)(sv_u + col), sud = *(const half2_t*)(su_d + col);
+            g0 *= (float)svg.x; g1 *= (float)svg.y; u0 *= (float)svu.x; u1 *= (float)svu.y;
+            v0 = g0 / (1.f + __expf(-g0)) * u0 * (float)sud.x; v1 = g1 / (1.f + __expf(-g1)) * u1 * (float)sud.y;
+            wht128(v0, v1, lane);
+        }
+        dst[bop_index(2 * lane)] = (_Float16)v0; dst[bop_index(2 * lane + 1)] = (_Float16)v1;
+    }
+}
+
+// grid (npairs), block 256: out[pt[p]] += rw[p] * sv_o (.) Hadamard(y[p])
+__global__ void __launch_bounds__(256) nq_pf_post_k(const float* __restrict__ y, const int32_t* __restrict__ pt, const int32_t* __restrict__ pe,
+                                                     const _Float16* __restrict__ prw, const int64_t* __restrict__ table, float* out, int E, int H, int I)
+{
+    const int p = blockIdx.x, lane = threadIdx.x & 63, warp = threadIdx.x >> 6;
+    const int e = pe[p];
+    const float w = (float)prw[p];
+    if (e < 0 || e >= E || w == 0.f || table[(size_t)e * TBL_W] <= 0) return;
+    const _Float16* sv_o = (const _Float16*)table[(size_t)e * TBL_W + 9] + H + 3 * I;
+    float* op = out + (size_t)pt[p] * H;
+    for (int grp = warp; grp < H / 128; grp += 4)
+    {
+        const int col = grp * 128 + 2 * lane;
+        const float2 v = *(const float2*)(y + (size_t)p * H + col);
+        float v0 = v.x, v1 = v.y;
+        wht128(v0, v1, lane);
+        const half2_t sv = *(const half2_t*)(sv_o + col);
+        atomicAdd(op + col, w * (v0 * (float)sv.x));
+        atomicAdd(op + col + 1, w * (v1 * (float)sv.y));
+    }
+}
+
+__global__ void nq_pf_hits_k(const int32_t* counts, int32_t* hits, int E)
+{
+    const int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e < E && counts[e]) __hip_atomic_fetch_add(hits + e, counts[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+struct PfGemm
+{
+    const int64_t* table; const int32_t* tiles;   // tiles [ntiles][4]: expert, first row, rows (<= 16 TG), unused
+    const _Float16* A0; const _Float16* A1;         // activations in B-operand order: A0 for weight rows < I (or all rows of down), A1 above
+    float* C; int mode, E, H, I;
+};
+
+// body for one (RES, CODE): all K / 128 chunks of this wave's two strips against the tile's tokens
+template <int TG, bool RES, int CODE>
+__device__ __forceinline__ void pf_chunks(const Planes& P, const LaneCtx& L, int C, const _Float16* A, int K, int row0, int nrows,
+                                          char* smem, float4_t (*acc)[2])
+{
+    constexpr int NW = RES ? Rec<CODE>::NW : 1;
+    u32x4 nb = P.base[L.rec0];
+    uint32_t nr[NW + 2] = {0}, ndw = 0, nvar = 0;
+    if constexpr (RES) { load_record<CODE>(nr, P.res, L.rec0, L.nrec); ndw = P.dw[L.unit0]; }
+    if (P.var) nvar = P.var[L.unit0];
+    const int t4 = threadIdx.x >> 4 & 3, n = threadIdx.x & 15;
+    for (int c = 0; c < C; ++c)
+    {
+        // ---- stage the tile's tokens for chunk c (rows beyond the tile read as zero)
+        __syncthreads();
+        for (int i = threadIdx.x; i < TG * 16 * 16; i += blockDim.x)
+        {
+            const int tok = i >> 4, q = i & 15;
+            uint4 v = make_uint4(0, 0, 0, 0);
+            if (tok < nrows) v = *(const uint4*)(A + (size_t)(row0 + tok) * K + c * 128 + q * 8);
+            *(uint4*)(smem + tok * PF_ROW + q * 16) = v;
+        }
+        // ---- decode this wave's unit pair of chunk c into A operands; prefetch chunk c + 1
+        uint32_t wb[6], wr[NW + 2];
+        wb[0] = nb.x; wb[1] = nb.y; wb[2] = nb.z; wb[3] = nb.w;
+#pragma unroll
+        for (int i = 0; i < NW; ++i) wr[i] = nr[i];
+        const uint32_t dw = ndw, var = nvar;
+        if (c + 1 < C)
+        {
+            nb = P.base[L.rec0 + (size_t)(c + 1) * 32];
+            if constexpr (RES) { load_record<CODE>(nr, P.res, L.rec0 + (size_t)(c + 1) * 32, L.nrec); ndw = P.dw[L.unit0 + c + 1]; }
+            if (P.var) nvar = P.var[L.unit0 + c + 1];
+        }
+        ext_words<128, 4>(wb, __shfl(wb[0], L.src));
+        const uint32_t sgm = ((var >> L.g) & 1u) * 0x80008000u;
+        FoldK k;
+        if constexpr (RES)
+        {
+            ext_words<Rec<CODE>::BITS, Rec<CODE>::NW>(wr, __shfl(wr[0], L.src));
+            k = consts_fold(dw, sgm);
+        }
+        else k = consts_l2(sgm);
+        half8_t aop[4][2];
+        static_for<4>([&](auto mm) {
+            constexpr int MM = decltype(mm)::value;
+            aop[MM][0] = a_operand<RES, CODE, MM, 0>(wb, wr, k);
+            aop[MM][1] = a_operand<RES, CODE, MM, 1>(wb, wr, k);
+        });
+        __syncthreads();
+        // ---- TG x 8 MFMAs: tokens 16 tg + n as the N dimension
+        const char* xp = smem + n * PF_ROW + t4 * 16;
+#pragma unroll
+        for (int tg = 0; tg < TG; ++tg)
+        {
+#pragma unroll
+            for (int mm = 0; mm < 4; ++mm)
+            {
+                const half8_t b = *(const half8_t*)(xp + tg * 16 * PF_ROW + mm * 64);
+                acc[tg][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aop[mm][0], b, acc[tg][0], 0, 0, 0);
+                acc[tg][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aop[mm][1], b, acc[tg][1], 0, 0, 0);
+            }
+        }
+    }
+}
+
+// grid (N / 128, ntiles), block 256 (4 wavefronts x 2 strips = 128 weight rows); dynamic LDS = 16 TG * PF_ROW bytes
+template <int TG>
+__global__ void __launch_bounds__(256) nq_pf_gemm_k(PfGemm a)
+{
+    extern __shared__ __align__(16) char smem[];
+    const int lane = threadIdx.x & 63, warp = threadIdx.x >> 6;
+    const int32_t* tile = a.tiles + 4 * blockIdx.y;
+    const int e = tile[0], row0 = tile[1], nrows = tile[2];
+    if (e < 0 || e >= a.E || nrows <= 0) return;
+    const int64_t* ent = a.table + (size_t)e * TBL_W;
+    const int lv = (int)ent[0];
+    if (lv <= 0) return;                                         // rows of a level-0 expert are skipped downstream
+    const int N = a.mode == 0 ? 2 * a.I : a.H, K = a.mode == 0 ? a.H : a.I, C = K / 128;
+    const int sp = blockIdx.x * 4 + warp;                        // strip pair of this wavefront
+    const _Float16* A = (a.mode == 0 && (int)(blockIdx.x * 128) >= a.I) ? a.A1 : a.A0;
+    const int t4 = lane >> 4, ss = (lane >> 3) & 1, g = lane & 7, n = lane & 15;
+    const Planes P = planes_of(ent, a.mode);
+    LaneCtx L;
+    L.unit0 = (size_t)(2 * sp + ss) * C; L.rec0 = L.unit0 * 32 + 4 * g + t4;
+    L.nrec = (size_t)(N / 16) * C * 32;
+    L.src = (lane + 16) & 63; L.g = g; L.xs = nullptr; L.xstep = 0;
+    float4_t acc[TG][2];
+#pragma unroll
+    for (int tg = 0; tg < TG; ++tg) { acc[tg][0] = float4_t{0.f, 0.f, 0.f, 0.f}; acc[tg][1] = float4_t{0.f, 0.f, 0.f, 0.f}; }
+    if (lv == 2) pf_chunks<TG, false, 0>(P, L, C, A, K, row0, nrows, smem, acc);
+    else dispatch_code(P.code, [&](auto tag) { pf_chunks<TG, true, decltype(tag)::value>(P, L, C, A, K, row0, nrows, smem, acc); });
+    // lane (t4, n) holds, for token 16 tg + n, weight rows 32 sp + 16 (t4 >> 1) + 4 (t4 & 1) + i (+ 8 for acc[..][1])
+    const int wrow = 32 * sp + 16 * (t4 >> 1) + 4 * (t4 & 1);
+#pragma unroll
+    for (int tg = 0; tg < TG; ++tg)
+    {
+        const int tok = 16 * tg + n;
+        if (tok < nrows)
+        {
+            float* c = a.C + (size_t)(row0 + tok) * N + wrow;
+            *(float4_t*)c = acc[tg][0];
+            *(float4_t*)(c + 8) = acc[tg][1];
+        }
+    }
+}
+
+int launch_pf_pre(const void* x, const int32_t* pt, const int32_t* pe, int np, const int64_t* table, void* xg, void* xu, int E, int H, int I, hipStream_t st)
+{
+    if (!np) return 0;
+    nq_pf_pre_k<<<np, 256, 0, st>>>((const _Float16*)x, pt, pe, table, (_Float16*)xg, (_Float16*)xu, E, H, I);
+    NQ_LAUNCH_CHECK("nq_pf_pre");
+    return 0;
+}
+int launch_pf_mid(const float* acc_gu, const int32_t* pe, int np, const int64_t* table, void* h, int E, int H, int I, hipStream_t st)
+{
+    if (!np) return 0;
+    nq_pf_mid_k<<<np, 256, 0, st>>>(acc_gu, pe, table, (_Float16*)h, E, H, I);
+    NQ_LAUNCH_CHECK("nq_pf_mid");
+    return 0;
+}
+int launch_pf_post(const float* y, const int32_t* pt, const int32_t* pe, const void* prw, int np, const int64_t* table, float* out, int E, int H, int I, hipStream_t st)
+{
+    if (!np) return 0;
+    nq_pf_post_k<<<np, 256, 0, st>>>(y, pt, pe, (const _Float16*)prw, table, out, E, H, I);
+    NQ_LAUNCH_CHECK("nq_pf_post");
+    return 0;
+}
+int launch_pf_hits(const int32_t* counts, int32_t* hits, int E, hipStream_t st)
+{
+    nq_pf_hits_k<<<(E + 255) / 256, 256, 0, st>>>(counts, hits, E);
+    NQ_LAUNCH_CHECK("nq_pf_hits");
+    return 0;
+}
+
+template <int TG>
+static int launch_gemm_tg(const PfGemm& a, int ntiles, int N, hipStream_t st)
+{
+    const int shm = 16 * TG * PF_ROW;
+    if (shm > 48 * 1024)
+    {
+        hipError_t e = hipFuncSetAttribute((const void*)nq_pf_gemm_k<TG>, hipFuncAttributeMaxDynamicSharedMemorySize, shm);
+        if (e != hipSuccess) return set_error("nq_pf_gemm: LDS %d bytes: %s", shm, hipGetErrorString(e));
+    }
+    nq_pf_gemm_k<TG><<<dim3(N / 128, ntiles), 256, shm, st>>>(a);
+    NQ_LAUNCH_CHECK("nq_pf_gemm");
+    return 0;
+}
+
+int launch_pf_gemm(const int64_t* table, const int32_t* tiles, int ntiles, int bm, int mode, const void* A0, const void* A1, float* C,
+                   int E, int H, int I, hipStream_t st)
+{
+    if (!ntiles) return 0;
+    PfGemm a{table, tiles, (const _Float16*)A0, (const _Float16*)A1, C, mode, E, H, I};
+    const int N = mode == 0 ? 2 * I : H;
+    switch (bm)
+    {
+        case 16: return launch_gemm_tg<1>(a, ntiles, N, st);
+        case 32: return launch_gemm_tg<2>(a, ntiles, N, st);
+        case 64: return launch_gemm_tg<4>(a, ntiles, N, st);
+        case 128: return launch_gemm_tg<8>(a, ntiles, N, st);
+        case 256: return launch_gemm_tg<16>(a, ntiles, N, st);
+    }
+    return set_error("nq_pf_gemm: tile height %d not in {16, 32, 64, 128, 256}", bm);
+}
+
+}  // namespace nq

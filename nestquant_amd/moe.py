@@ -185,6 +185,90 @@ class MoELayer:
         return out
 
 
+_PF = {}
+PF_TILES = (16, 32, 64, 128, 256)            # token-tile heights the grouped GEMM is compiled for
+
+
+def pf_bytes(H, I, R, G=0):
+    """bytes of prefill scratch for R pair rows (G is accepted for signature compatibility: no decoded-weight scratch exists)"""
+    return R * (2 * H * 2 + 2 * I * 4 + I * 2 + H * 4)
+
+
+def pf_scratch(dev, H, I, R, G=0):
+    """Prefill scratch shared by every layer on `dev`, allocated on first use: xg | xu fp16 [R, H], acc_gu fp32 [R, 2I],
+    h fp16 [R, I], y fp32 [R, H]. Unlike the reference (sm120/moe.py:263-274) there is no dense-weight scratch: the
+    grouped GEMM decodes weights in registers."""
+    k = (str(dev), H, I, R)
+    if k not in _PF:
+        f16, f32 = torch.float16, torch.float32
+        _PF[k] = dict(xg=torch.empty(R, H, dtype=f16, device=dev), xu=torch.empty(R, H, dtype=f16, device=dev),
+                      acc=torch.empty(R, 2 * I, dtype=f32, device=dev), h=torch.empty(R, I, dtype=f16, device=dev),
+                      y=torch.empty(R, H, dtype=f32, device=dev))
+    return _PF[k]
+
+
+def pf_tiles(segs):
+    """segs [(expert, first row, rows)] -> {tile height: int32 [n, 4] rows (expert, row0, rows, 0)}. Rows of an expert are
+    cut into 256-row tiles; the remainder takes the smallest compiled height that holds it."""
+    out = {bm: [] for bm in PF_TILES}
+    for e, r0, n in segs:
+        while n > 0:
+            take = min(n, PF_TILES[-1])
+            bm = next(b for b in PF_TILES if b >= take)
+            out[bm].append((e, r0, take, 0))
+            r0 += take; n -= take
+    return {bm: torch.tensor(v, dtype=torch.int32) for bm, v in out.items() if v}
+
+
+def prefill(s, x, sel, rw, out=None, R=None, G=None, table=None):
+    """T > Bmax tokens (reference sm120/moe.py:282-326): pairs sorted by expert, each routed expert decoded inside the
+    grouped GEMMs at the level of its live table row, same math as the decode path (fp32 accumulation order differs).
+    One host sync (expert counts). Not graph-capturable. Exports routing hits like the decode kernel."""
+    assert x.dtype == torch.float16 and rw.dtype == torch.float16 and sel.dtype == torch.int64, (x.dtype, rw.dtype, sel.dtype)
+    assert x.is_contiguous()
+    T, k = sel.shape
+    H, I, E, dev, Lb = s.H, s.I, s.E, x.device, s.M
+    tb = s.table if table is None else table
+    st = _lib.stream_ptr()
+    out = torch.zeros(T, H, dtype=torch.float32, device=dev) if out is None else out.zero_()
+    flat = sel.reshape(-1); rwf = rw.reshape(-1)
+    order = torch.argsort(flat, stable=True)
+    pe = flat[order].int(); pt = (order // k).int(); prw = rwf[order].contiguous()
+    one = torch.ones_like(flat, dtype=torch.int32)
+    cnt = torch.zeros(E, dtype=torch.int32, device=dev).scatter_add_(0, flat, one)
+    if s.hits_ptr:
+        hc = torch.zeros(E + 1, dtype=torch.int32, device=dev).scatter_add_(0, torch.where(rwf != 0, flat, E), one)[:E].contiguous()
+        _lib.check(Lb.nq_pf_hits(hc.data_ptr(), s.hits_ptr, E, st))
+    cnt = cnt.cpu().tolist()                                         # the one host sync
+    start, o = [0] * E, 0
+    for e in range(E):
+        start[e] = o; o += cnt[e]
+    P = T * k
+    R = min(P, R or int(__import__("os").environ.get("NQ_PF_ROWS", "32768")))
+    S = pf_scratch(dev, H, I, R)
+    for c in range(0, P, R):
+        d = min(P, c + R); n = d - c
+        segs = []
+        for e in range(E):
+            u, v = max(start[e], c), min(start[e] + cnt[e], d)
+            if v > u:
+                segs.append((e, u - c, v - u))
+        tiles = {bm: t.pin_memory().to(dev, non_blocking=True) for bm, t in pf_tiles(segs).items()}
+        pts, pes, prws = pt[c:d], pe[c:d], prw[c:d]
+        _lib.check(Lb.nq_pf_pre(x.data_ptr(), pts.data_ptr(), pes.data_ptr(), n, tb.data_ptr(), S["xg"].data_ptr(),
+                                S["xu"].data_ptr(), E, H, I, st))
+        for bm, t in tiles.items():
+            _lib.check(Lb.nq_pf_gemm(tb.data_ptr(), t.data_ptr(), t.shape[0], bm, 0, S["xg"].data_ptr(), S["xu"].data_ptr(),
+                                     S["acc"].data_ptr(), E, H, I, st))
+        _lib.check(Lb.nq_pf_mid(S["acc"].data_ptr(), pes.data_ptr(), n, tb.data_ptr(), S["h"].data_ptr(), E, H, I, st))
+        for bm, t in tiles.items():
+            _lib.check(Lb.nq_pf_gemm(tb.data_ptr(), t.data_ptr(), t.shape[0], bm, 1, S["h"].data_ptr(), None,
+                                     S["y"].data_ptr(), E, H, I, st))
+        _lib.check(Lb.nq_pf_post(S["y"].data_ptr(), pts.data_ptr(), pes.data_ptr(), prws.data_ptr(), n, tb.data_ptr(),
+                                 out.data_ptr(), E, H, I, st))
+    return out
+
+
 class Mailbox:
     """Graph-safe table updates (reference sm120/moe.py:329-342): call apply() on the compute stream before the layer;
     stage rows from a side stream with post(). One outstanding op per expert."""
@@ -218,3 +302,6 @@ class Mailbox:
 
     def done(s, e):
         return int(s.applied_host[e]) == s.hseq[e]
+
+
+MoELayer.prefill = prefill
