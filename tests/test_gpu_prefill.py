@@ -78,7 +78,8 @@ def test_full_shape_prefill_vs_decode_slices():
     ys = sliced_decode(L, x, sel, rw)
     torch.cuda.synchronize()
     cnt = torch.bincount(sel.flatten().cpu(), minlength=NE).tolist()
-    assert max(cnt) > 256 and min(c for c in cnt if c) < 64      # both a multi-tile expert and a small remainder tile
+    kinds = M.pf_tiles([(e, 0, c) for e, c in enumerate(cnt) if c])
+    assert max(cnt) > 256 and len(kinds) >= 3                    # multi-tile experts and remainder tiles of several heights
     assert rel_err(y.cpu().numpy(), ys.cpu().numpy()) < 2e-5
     # float64 oracle on a few tokens through HIP-decoded dense weights (the decoder is proved bit-exact elsewhere)
     from tests.test_gpu_moe import _dense_from_gpu
