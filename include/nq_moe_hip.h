@@ -82,7 +82,7 @@ int nq_mailbox(int64_t* table, const int64_t* stage, const int32_t* seq, int32_t
                void* stream);
 
 /* ---- prefill (more tokens than a decode call takes): pairs (token, expert) sorted by expert ------------------------------
- * pt / pe: int32[np] token and expert of each pair; prw: fp16[np] router weight. Pairs whose expert is at level <= 0,
+ * pt / pe: int32[np] token and expert of each pair. Pairs whose expert is at level <= 0,
  * outside [0, E), or whose weight is 0 contribute nothing. Activation buffers xg, xu [np][H] and h [np][I] are fp16 with
  * every 128-column chunk stored in the MFMA B-operand column order (an internal layout shared by these entry points). */
 
@@ -104,10 +104,13 @@ int nq_pf_gemm(const int64_t* table, const int32_t* tiles, int ntiles, int bm, i
 int nq_pf_mid(const float* acc_gu, const int32_t* pe, int np, const int64_t* table, void* h_f16, int E, int H, int I,
               void* stream);
 
-/* out[pt[p]] += prw[p] * sv_o (.) Hadamard(y[p]) with float atomics; out fp32 [T][H] must be zeroed by the caller.
- * Replaces pf_post (reference sm120/nqmoe.cu:1205-1240,1278-1287). */
-int nq_pf_post(const float* y, const int32_t* pt, const int32_t* pe, const void* prw_f16, int np, const int64_t* table,
-               float* out, int E, int H, int I, void* stream);
+/* For every token t < T: out[t] += sum over its picks k whose pair row pos[t][k] lies in [row_lo, row_lo + nrows) of
+ * rw[t][k] * sv_o (.) Hadamard(y[pos[t][k] - row_lo]). pos int32 [T][topk] = row of pair (t, k) in the expert-sorted
+ * order; sel int64 [T][topk]; rw fp16 [T][topk]; y fp32 [nrows][H]; out fp32 [T][H], zeroed by the caller before the
+ * first row chunk. Gathered per token: no atomics, fixed summation order. Replaces pf_post (reference
+ * sm120/nqmoe.cu:1205-1240,1278-1287, which adds with float atomics). */
+int nq_pf_post(const float* y, const int32_t* pos, const int64_t* sel, const void* rw_f16, int T, int topk, int row_lo,
+               int nrows, const int64_t* table, float* out, int E, int H, int I, void* stream);
 
 /* hits[e] += counts[e] (hits may be host-mapped). Replaces pf_hits (reference sm120/nqmoe.cu:1241-1245,1288-1293). */
 int nq_pf_hits(const int32_t* counts, int32_t* hits, int E, void* stream);

@@ -37,7 +37,8 @@ int launch_dequant(const int64_t* row, int proj, int level, int H, int I, void* 
 int launch_pf_decode(const int64_t* table, const int32_t* experts, int G, void* Wgu, void* Wdn, int H, int I, hipStream_t st);
 int launch_pf_pre(const void* x, const int32_t* pt, const int32_t* pe, int np, const int64_t* table, void* xg, void* xu, int E, int H, int I, hipStream_t st);
 int launch_pf_mid(const float* acc_gu, const int32_t* pe, int np, const int64_t* table, void* h, int E, int H, int I, hipStream_t st);
-int launch_pf_post(const float* y, const int32_t* pt, const int32_t* pe, const void* prw, int np, const int64_t* table, float* out, int E, int H, int I, hipStream_t st);
+int launch_pf_post(const float* y, const int32_t* pos, const int64_t* sel, const void* rw, int T, int topk, int row_lo, int nrows,
+                   const int64_t* table, float* out, int E, int H, int I, hipStream_t st);
 int launch_pf_hits(const int32_t* counts, int32_t* hits, int E, hipStream_t st);
 int launch_pf_gemm(const int64_t* table, const int32_t* tiles, int ntiles, int bm, int mode, const void* A0, const void* A1, float* C,
                    int E, int H, int I, hipStream_t st);

@@ -9,7 +9,7 @@
 //                 decodes two strips of the expert's records into MFMA A operands, then runs TG x 8 MFMAs
 //                 (v_mfma_f32_16x16x32_f16, fp32 accumulate) over the staged tokens. Level from the live table row.
 //   nq_pf_mid_k   Hadamard * sv, SwiGLU, * su_d, Hadamard -> h fp16 (B-operand order)               (reference nq_pf_mid)
-//   nq_pf_post_k  out[token] += rw * sv_o (.) Hadamard(y)  (float atomics, as the reference)        (reference nq_pf_post)
+//   nq_pf_post_k  out[token] += sum over its picks of rw * sv_o (.) Hadamard(y): gathered per token, no atomics  (reference nq_pf_post)
 //   nq_pf_hits_k  hits[e] += counts[e]                                                            (reference nq_pf_hits)
 #include "nq_tile.hpp"
 #include "nq_host.hpp"
@@ -17,6 +17,19 @@
 namespace nq {
 
 constexpr int PF_ROW = 272;                    // LDS bytes per staged token: 256 + 16 (spreads tokens over banks)
+
+// lane holds columns 2 lane, 2 lane + 1 of a 128-column chunk; columns c and c + 16 are neighbours in the B-operand order,
+// so lanes l and l ^ 8 swap one value each and every lane stores one aligned 4-byte pair
+__device__ __forceinline__ void store_bop(_Float16* dst, float v0, float v1, int lane)
+{
+    const bool hi = (lane >> 3) & 1;
+    const float mine = hi ? v1 : v0, give = hi ? v0 : v1;
+    const float got = __shfl_xor(give, 8);                        // low lanes get the partner's v0, high lanes the partner's v1
+    half2_t w;
+    w.x = (_Float16)(hi ? got : mine); w.y = (_Float16)(hi ? mine : got);
+    const int c = hi ? 2 * (lane ^ 8) + 1 : 2 * lane;           // the pair's low column: (c, c + 16)
+    *(half2_t*)(dst + bop_index(c)) = w;
+}
 
 // grid (npairs), block 256: wave w handles 128-column groups w, w + 4, ... of gate then up
 __global__ void __launch_bounds__(256) nq_pf_pre_k(const _Float16* __restrict__ x, const int32_t* __restrict__ pt, const int32_t* __restrict__ pe,
@@ -40,7 +53,7 @@ __global__ void __launch_bounds__(256) nq_pf_pre_k(const _Float16* __restrict__ 
             v0 = (float)xv.x * (float)sv.x; v1 = (float)xv.y * (float)sv.y;
             wht128(v0, v1, lane);
         }
-        dst[bop_index(2 * lane)] = (_Float16)v0; dst[bop_index(2 * lane + 1)] = (_Float16)v1;
+        store_bop(dst, v0, v1, lane);
     }
 }
 
@@ -68,29 +81,41 @@ __global__ void __launch_bounds__(256) nq_pf_mid_k(const float* __restrict__ acc
             v0 = g0 / (1.f + __expf(-g0)) * u0 * (float)sud.x; v1 = g1 / (1.f + __expf(-g1)) * u1 * (float)sud.y;
             wht128(v0, v1, lane);
         }
-        dst[bop_index(2 * lane)] = (_Float16)v0; dst[bop_index(2 * lane + 1)] = (_Float16)v1;
+        store_bop(dst, v0, v1, lane);
     }
 }
 
-// grid (npairs), block 256: out[pt[p]] += rw[p] * sv_o (.) Hadamard(y[p])
-__global__ void __launch_bounds__(256) nq_pf_post_k(const float* __restrict__ y, const int32_t* __restrict__ pt, const int32_t* __restrict__ pe,
-                                                     const _Float16* __restrict__ prw, const int64_t* __restrict__ table, float* out, int E, int H, int I)
+// grid (T), block 256: out[t] += sum over the token's picks whose pair row lies in [row_lo, row_lo + nrows) of
+// rw * sv_o (.) Hadamard(y[row]); pos[t][k] = row of pair (t, k) in the expert-sorted order. One block owns a token, so
+// the sum needs no atomics and its order is fixed (the reference's pf_post adds with float atomics in arrival order).
+__global__ void __launch_bounds__(256) nq_pf_post_k(const float* __restrict__ y, const int32_t* __restrict__ pos, const int64_t* __restrict__ sel,
+                                                     const _Float16* __restrict__ rw, int topk, int row_lo, int nrows,
+                                                     const int64_t* __restrict__ table, float* out, int E, int H, int I)
 {
-    const int p = blockIdx.x, lane = threadIdx.x & 63, warp = threadIdx.x >> 6;
-    const int e = pe[p];
-    const float w = (float)prw[p];
-    if (e < 0 || e >= E || w == 0.f || table[(size_t)e * TBL_W] <= 0) return;
-    const _Float16* sv_o = (const _Float16*)table[(size_t)e * TBL_W + 9] + H + 3 * I;
-    float* op = out + (size_t)pt[p] * H;
+    const int t = blockIdx.x, lane = threadIdx.x & 63, warp = threadIdx.x >> 6;
     for (int grp = warp; grp < H / 128; grp += 4)
     {
         const int col = grp * 128 + 2 * lane;
-        const float2 v = *(const float2*)(y + (size_t)p * H + col);
-        float v0 = v.x, v1 = v.y;
-        wht128(v0, v1, lane);
-        const half2_t sv = *(const half2_t*)(sv_o + col);
-        atomicAdd(op + col, w * (v0 * (float)sv.x));
-        atomicAdd(op + col + 1, w * (v1 * (float)sv.y));
+        float o0 = 0.f, o1 = 0.f;
+        bool any = false;
+        for (int k = 0; k < topk; ++k)
+        {
+            const int r = pos[(size_t)t * topk + k] - row_lo;
+            const long long e = sel[(size_t)t * topk + k];
+            const float w = (float)rw[(size_t)t * topk + k];
+            if (r < 0 || r >= nrows || e < 0 || e >= E || w == 0.f || table[(size_t)e * TBL_W] <= 0) continue;
+            const float2 v = *(const float2*)(y + (size_t)r * H + col);
+            float v0 = v.x, v1 = v.y;
+            wht128(v0, v1, lane);
+            const half2_t sv = *(const half2_t*)((const _Float16*)table[(size_t)e * TBL_W + 9] + H + 3 * I + col);
+            o0 += w * (v0 * (float)sv.x); o1 += w * (v1 * (float)sv.y);
+            any = true;
+        }
+        if (any)
+        {
+            float2* op = (float2*)(out + (size_t)t * H + col);
+            float2 cur = *op; cur.x += o0; cur.y += o1; *op = cur;
+        }
     }
 }
 
@@ -117,12 +142,12 @@ __device__ __forceinline__ void pf_chunks(const Planes& P, const LaneCtx& L, int
     uint32_t nr[NW + 2] = {0}, ndw = 0, nvar = 0;
     if constexpr (RES) { load_record<CODE>(nr, P.res, L.rec0, L.nrec); ndw = P.dw[L.unit0]; }
     if (P.var) nvar = P.var[L.unit0];
-    const int t4 = threadIdx.x >> 4 & 3, n = threadIdx.x & 15;
+    const int t4 = threadIdx.x >> 4 & 3, n = threadIdx.x & 15, ntg = (nrows + 15) >> 4;
     for (int c = 0; c < C; ++c)
     {
         // ---- stage the tile's tokens for chunk c (rows beyond the tile read as zero)
         __syncthreads();
-        for (int i = threadIdx.x; i < TG * 16 * 16; i += blockDim.x)
+        for (int i = threadIdx.x; i < ntg * 16 * 16; i += blockDim.x)
         {
             const int tok = i >> 4, q = i & 15;
             uint4 v = make_uint4(0, 0, 0, 0);
@@ -157,17 +182,21 @@ __device__ __forceinline__ void pf_chunks(const Planes& P, const LaneCtx& L, int
             aop[MM][1] = a_operand<RES, CODE, MM, 1>(wb, wr, k);
         });
         __syncthreads();
-        // ---- TG x 8 MFMAs: tokens 16 tg + n as the N dimension
+        // ---- up to TG x 8 MFMAs: tokens 16 tg + n as the N dimension. mm is the outer loop so that consecutive MFMAs
+        // write different accumulators (a dependent MFMA would wait for the previous one to drain).
         const char* xp = smem + n * PF_ROW + t4 * 16;
 #pragma unroll
-        for (int tg = 0; tg < TG; ++tg)
+        for (int mm = 0; mm < 4; ++mm)
         {
 #pragma unroll
-            for (int mm = 0; mm < 4; ++mm)
+            for (int tg = 0; tg < TG; ++tg)
             {
-                const half8_t b = *(const half8_t*)(xp + tg * 16 * PF_ROW + mm * 64);
-                acc[tg][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aop[mm][0], b, acc[tg][0], 0, 0, 0);
-                acc[tg][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aop[mm][1], b, acc[tg][1], 0, 0, 0);
+                if (tg < ntg)                                    // block-uniform: row groups beyond the tile are skipped
+                {
+                    const half8_t b = *(const half8_t*)(xp + tg * 16 * PF_ROW + mm * 64);
+                    acc[tg][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aop[mm][0], b, acc[tg][0], 0, 0, 0);
+                    acc[tg][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aop[mm][1], b, acc[tg][1], 0, 0, 0);
+                }
             }
         }
     }
@@ -228,10 +257,11 @@ int launch_pf_mid(const float* acc_gu, const int32_t* pe, int np, const int64_t*
     NQ_LAUNCH_CHECK("nq_pf_mid");
     return 0;
 }
-int launch_pf_post(const float* y, const int32_t* pt, const int32_t* pe, const void* prw, int np, const int64_t* table, float* out, int E, int H, int I, hipStream_t st)
+int launch_pf_post(const float* y, const int32_t* pos, const int64_t* sel, const void* rw, int T, int topk, int row_lo, int nrows,
+                   const int64_t* table, float* out, int E, int H, int I, hipStream_t st)
 {
-    if (!np) return 0;
-    nq_pf_post_k<<<np, 256, 0, st>>>(y, pt, pe, (const _Float16*)prw, table, out, E, H, I);
+    if (!T || !nrows) return 0;
+    nq_pf_post_k<<<T, 256, 0, st>>>(y, pos, sel, (const _Float16*)rw, topk, row_lo, nrows, table, out, E, H, I);
     NQ_LAUNCH_CHECK("nq_pf_post");
     return 0;
 }

@@ -233,7 +233,10 @@ def prefill(s, x, sel, rw, out=None, R=None, G=None, table=None):
     out = torch.zeros(T, H, dtype=torch.float32, device=dev) if out is None else out.zero_()
     flat = sel.reshape(-1); rwf = rw.reshape(-1)
     order = torch.argsort(flat, stable=True)
-    pe = flat[order].int(); pt = (order // k).int(); prw = rwf[order].contiguous()
+    pe = flat[order].int(); pt = (order // k).int()
+    pos = torch.empty_like(order, dtype=torch.int32)
+    pos[order] = torch.arange(order.numel(), dtype=torch.int32, device=dev)       # row of pair (t, k) in sorted order
+    selc, rwc = sel.contiguous(), rw.contiguous()
     one = torch.ones_like(flat, dtype=torch.int32)
     cnt = torch.zeros(E, dtype=torch.int32, device=dev).scatter_add_(0, flat, one)
     if s.hits_ptr:
@@ -254,7 +257,7 @@ def prefill(s, x, sel, rw, out=None, R=None, G=None, table=None):
             if v > u:
                 segs.append((e, u - c, v - u))
         tiles = {bm: t.pin_memory().to(dev, non_blocking=True) for bm, t in pf_tiles(segs).items()}
-        pts, pes, prws = pt[c:d], pe[c:d], prw[c:d]
+        pts, pes = pt[c:d], pe[c:d]
         _lib.check(Lb.nq_pf_pre(x.data_ptr(), pts.data_ptr(), pes.data_ptr(), n, tb.data_ptr(), S["xg"].data_ptr(),
                                 S["xu"].data_ptr(), E, H, I, st))
         for bm, t in tiles.items():
@@ -264,7 +267,7 @@ def prefill(s, x, sel, rw, out=None, R=None, G=None, table=None):
         for bm, t in tiles.items():
             _lib.check(Lb.nq_pf_gemm(tb.data_ptr(), t.data_ptr(), t.shape[0], bm, 1, S["h"].data_ptr(), None,
                                      S["y"].data_ptr(), E, H, I, st))
-        _lib.check(Lb.nq_pf_post(S["y"].data_ptr(), pts.data_ptr(), pes.data_ptr(), prws.data_ptr(), n, tb.data_ptr(),
+        _lib.check(Lb.nq_pf_post(S["y"].data_ptr(), pos.data_ptr(), selc.data_ptr(), rwc.data_ptr(), T, k, c, n, tb.data_ptr(),
                                  out.data_ptr(), E, H, I, st))
     return out
 

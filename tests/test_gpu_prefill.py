@@ -80,7 +80,7 @@ def test_full_shape_prefill_vs_decode_slices():
     cnt = torch.bincount(sel.flatten().cpu(), minlength=NE).tolist()
     kinds = M.pf_tiles([(e, 0, c) for e, c in enumerate(cnt) if c])
     assert max(cnt) > 256 and len(kinds) >= 3                    # multi-tile experts and remainder tiles of several heights
-    assert rel_err(y.cpu().numpy(), ys.cpu().numpy()) < 2e-5
+    assert rel_err(y.cpu().numpy(), ys.cpu().numpy()) < 5e-5     # two summation orders, each ~1e-5 from exact
     # float64 oracle on a few tokens through HIP-decoded dense weights (the decoder is proved bit-exact elsewhere)
     from tests.test_gpu_moe import _dense_from_gpu
     dense = _dense_from_gpu(ex, levels); signs = [e.signs.cpu().numpy() for e in ex]
