@@ -182,20 +182,23 @@ __device__ __forceinline__ void pf_chunks(const Planes& P, const LaneCtx& L, int
             aop[MM][1] = a_operand<RES, CODE, MM, 1>(wb, wr, k);
         });
         __syncthreads();
-        // ---- up to TG x 8 MFMAs: tokens 16 tg + n as the N dimension. mm is the outer loop so that consecutive MFMAs
-        // write different accumulators (a dependent MFMA would wait for the previous one to drain).
+        // ---- TG x 8 MFMAs: tokens 16 tg + n as the N dimension (row groups beyond the tile multiply stale LDS rows whose
+        // results are never stored). Two row groups are interleaved so that four different accumulators separate an MFMA
+        // from the next one that depends on it.
         const char* xp = smem + n * PF_ROW + t4 * 16;
+        constexpr int TS = TG >= 2 ? 2 : 1;
 #pragma unroll
-        for (int mm = 0; mm < 4; ++mm)
+        for (int tg = 0; tg < TG; tg += TS)
         {
 #pragma unroll
-            for (int tg = 0; tg < TG; ++tg)
+            for (int mm = 0; mm < 4; ++mm)
             {
-                if (tg < ntg)                                    // block-uniform: row groups beyond the tile are skipped
+#pragma unroll
+                for (int u = 0; u < TS; ++u)
                 {
-                    const half8_t b = *(const half8_t*)(xp + tg * 16 * PF_ROW + mm * 64);
-                    acc[tg][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aop[mm][0], b, acc[tg][0], 0, 0, 0);
-                    acc[tg][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aop[mm][1], b, acc[tg][1], 0, 0, 0);
+                    const half8_t b = *(const half8_t*)(xp + (tg + u) * 16 * PF_ROW + mm * 64);
+                    acc[tg + u][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aop[mm][0], b, acc[tg + u][0], 0, 0, 0);
+                    acc[tg + u][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aop[mm][1], b, acc[tg + u][1], 0, 0, 0);
                 }
             }
         }
