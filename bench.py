@@ -26,6 +26,7 @@ from nestquant_amd import format as F, moe as M, routing as RT  # noqa: E402
 
 H, I, E, TOPK = 6144, 2048, 256, 8
 HBM_PEAK_GBS = 8000.0
+MFMA_PEAK_TFLOPS = 2500.0            # dense fp16 / bf16 MFMA peak of MI355X
 # HBM bytes per gate|up launch / algorithmic bytes, from rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a 256 MiB copy kernel
 # (profiles/decode_gemv_hbm_traffic_pmc.txt)
 TRAFFIC_RATIO = 1.037
@@ -117,6 +118,110 @@ def cpu_baseline(ex, levels, e, x):
                 f"dense decode {1e3 * (t1 - t0):.1f} ms + fp32 layer math {1e3 * (t2 - t1):.1f} ms"), y
 
 
+def zipf_routing(T, dev, seed=11, skew=1.1):
+    """prefill routing: expert popularity ~ rank^-skew over a seeded permutation, 8 distinct experts per token (Gumbel top-k)"""
+    g = torch.Generator().manual_seed(seed)
+    p = torch.arange(1, E + 1, dtype=torch.float64) ** -skew
+    p = (p / p.sum())[torch.randperm(E, generator=g)]
+    u = torch.rand(T, E, generator=g, dtype=torch.float64).clamp_min(1e-300)
+    ids = torch.topk(p.log()[None] - torch.log(-torch.log(u)), TOPK, dim=-1).indices
+    w = torch.rand(T, TOPK, generator=g) + 0.1
+    return ids.to(dev), (w / w.sum(1, keepdim=True)).half().to(dev)
+
+
+def prefill_leg(L, ex, dev, T=4096, reps=3):
+    """config 4: 4096 tokens, Zipf(1.1) popularity, every expert at (nested) level 4; decode-fused grouped GEMMs"""
+    saved = L.table.clone()
+    for e in range(E):
+        L.set(e, ex[e], 4)
+    sel, rw = zipf_routing(T, dev)
+    g = torch.Generator().manual_seed(12)
+    x = (torch.randn(T, H, generator=g) * 0.05).half().to(dev)
+    L.prefill(x, sel, rw)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        L.prefill(x, sel, rw)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / reps
+    L.table.copy_(saved)
+    flops = T * TOPK * 6 * H * I
+    cnt = torch.bincount(sel.flatten().cpu(), minlength=E)
+    return dict(workload=f"prefill: T={T} tokens, top-8 over E=256 with Zipf(1.1) popularity, all experts at level 4, "
+                         f"rows per expert max {int(cnt.max())} / median {int(cnt.median())}",
+                ms=round(dt * 1e3, 3), tflops=round(flops / dt / 1e12, 1), flop=flops, mfma_peak_tflops=MFMA_PEAK_TFLOPS,
+                mfma_frac=round(flops / dt / 1e12 / MFMA_PEAK_TFLOPS, 4),
+                note="whole prefill() call: sort, pre, 2 decode-fused grouped GEMMs, mid, post; bound by the VALU trellis decode")
+
+
+def churn_leg(L, MB, ex, levels, routes, xs, dev, steps=64, ops_per_step=8):
+    """config 5: B=1 layer steps with 8 promote/demote ops per step issued on a side stream (pinned host -> slot copies)"""
+    from nestquant_amd import churn as CH
+    lv4 = [e for e in range(E) if levels[e] >= 3]
+    X = CH.ChurnExecutor(L, MB, {e: ex[e] for e in range(E)}, nslots=len(lv4) + 4 * ops_per_step)
+    saved = L.table.clone()
+    for e in range(E):
+        L.table[e].copy_(X.row(e, 2))
+    for e in lv4:                                                # bring the pool to the config-3 state (levels 3 become 4)
+        X.promote(e, 4)
+    MB.apply(); torch.cuda.synchronize(); X.poll()
+    X.bytes_copied = 0
+    s = torch.cuda.Stream()
+    graphs = []
+    for i in range(len(routes)):
+        with torch.cuda.stream(s):
+            MB.apply(); L(xs[i], routes[i][0], routes[i][1])
+        torch.cuda.synchronize()
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr, stream=s):
+            MB.apply(); L(xs[i], routes[i][0], routes[i][1])
+        graphs.append(gr)
+
+    def run(churn):
+        rng = __import__("random").Random(5)
+        lat, lags, issued = [], [], {}
+        t0 = time.perf_counter()
+        for st in range(steps):
+            if churn:
+                n = 0
+                cand = list(range(E)); rng.shuffle(cand)
+                for e in cand:
+                    if n == ops_per_step:
+                        break
+                    if not X.idle(e):
+                        continue
+                    ok = X.promote(e, 4) if X.level[e] == 2 else X.demote(e, 2)
+                    if ok:
+                        issued[e] = st; n += 1
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            with torch.cuda.stream(s):
+                e0.record(s); graphs[st % len(graphs)].replay(); e1.record(s)
+            e1.synchronize()
+            lat.append(e0.elapsed_time(e1) * 1e3)
+            for e in X.poll():
+                lags.append(st - issued.pop(e))
+        wall = time.perf_counter() - t0
+        return sorted(lat)[len(lat) // 2], lags, wall
+
+    idle_us, _, _ = run(False)
+    churn_us, lags, wall = run(True)
+    torch.cuda.synchronize()
+    for _ in range(64):                                          # drain outstanding ops, then check the books
+        MB.apply(); torch.cuda.synchronize()
+        X.poll()
+        if not X.pend:
+            break
+    X.check_invariants()
+    res = dict(workload=f"plane churn: {steps} B=1 layer steps, {ops_per_step} promote(2->4)/demote(4->2) ops per step on a side "
+                        f"stream, {X.lay.bytes} B per promotion from pinned host memory",
+               step_us_idle=round(idle_us, 2), step_us_churn=round(churn_us, 2), ops=X.n_ops - len(lv4), refused=X.n_refused,
+               h2d_GBps=round(X.bytes_copied / wall / 1e9, 2), h2d_MB=round(X.bytes_copied / 1e6, 1),
+               lag_steps_median=(sorted(lags)[len(lags) // 2] if lags else None), lag_steps_max=(max(lags) if lags else None),
+               invariants="B,T,O,K hold after the run")
+    L.table.copy_(saved)
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -124,6 +229,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=32)
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-prefill", action="store_true", help="skip the prefill (4096 tokens) leg")
+    ap.add_argument("--no-churn", action="store_true", help="skip the plane-churn leg")
     ap.add_argument("--calib", action="store_true", help="also run one 256 MiB device copy (reads 256 MiB, writes 256 MiB): "
                     "the known-size kernel that scales rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
     a = ap.parse_args()
@@ -216,6 +323,8 @@ def main():
     if not a.no_cpu:
         cpu, _ = cpu_baseline(ex, levels, routes[0][2][0], xs[0])
     lv_counts = {lv: levels.count(lv) for lv in (2, 3, 4)}
+    prefill = None if a.no_prefill else prefill_leg(L, ex, dev)
+    churn = None if a.no_churn else churn_leg(L, MB, ex, levels, routes[:16], xs, dev)
     print(json.dumps({
         "metric": "MoE layer us + HBM GB/s (decode bs1 top-8); prefill grouped-GEMM TFLOP/s",
         "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": W,
@@ -224,7 +333,7 @@ def main():
         "config": {"workload": f"decode MoE layer: E=256 top-8 B={B}, H=6144 I=2048, levels 2/3/4 = "
                                f"{lv_counts[2]}/{lv_counts[3]}/{lv_counts[4]} experts, seeded softmax routing avoiding the previous step",
                    "code_MB_per_step": round(nbytes / K / 1e6, 2), "hbm_frac_layer": round(gbs / HBM_PEAK_GBS, 4)},
-        "roofline": roofline, "cpu_baseline": cpu}))
+        "roofline": roofline, "cpu_baseline": cpu, "prefill": prefill, "churn": churn}))
 
 
 if __name__ == "__main__":
