@@ -164,7 +164,9 @@ def churn_leg(L, MB, ex, levels, routes, xs, dev, steps=64, ops_per_step=8):
         L.table[e].copy_(X.row(e, 2))
     for e in lv4:                                                # bring the pool to the config-3 state (levels 3 become 4)
         X.promote(e, 4)
+    torch.cuda.synchronize()                                     # the side-stream copies and rows have landed
     MB.apply(); torch.cuda.synchronize(); X.poll()
+    assert not X.pend
     X.bytes_copied = 0
     s = torch.cuda.Stream()
     graphs = []
@@ -199,7 +201,7 @@ def churn_leg(L, MB, ex, levels, routes, xs, dev, steps=64, ops_per_step=8):
             e1.synchronize()
             lat.append(e0.elapsed_time(e1) * 1e3)
             for e in X.poll():
-                lags.append(st - issued.pop(e))
+                lags.append(st - issued.pop(e, st))
         wall = time.perf_counter() - t0
         return sorted(lat)[len(lat) // 2], lags, wall
 
