@@ -308,3 +308,16 @@ class Mailbox:
 
 
 MoELayer.prefill = prefill
+
+
+def proj_gemv(layer, x, e=0, cfg=None):
+    """Raw fused decode+GEMV of the gate|up projection of expert e for every token of x [B, H] (B <= 8), without the
+    SwiGLU finisher: returns fp32 [B, 2I] = W_gu . fp16(Hadamard(x * su)) (rows < I rotated with su_g, the rest with su_u),
+    read back from the layer's k-slice partial sums after a gate|up-only launch whose finisher output is ignored."""
+    B = x.shape[0]
+    sel = torch.full((B, 1), e, dtype=torch.int64, device=x.device)
+    rw = torch.ones(B, 1, dtype=torch.float16, device=x.device)
+    cfg = list(cfg or layer.cfg_gu)
+    layer(x, sel, rw, which=1, cfg_gu=cfg)
+    ny = (layer.H // 128) // (cfg[0] * cfg[2])
+    return layer.acc_gu[:ny, :B].sum(0)
