@@ -320,4 +320,5 @@ def proj_gemv(layer, x, e=0, cfg=None):
     cfg = list(cfg or layer.cfg_gu)
     layer(x, sel, rw, which=1, cfg_gu=cfg)
     ny = (layer.H // 128) // (cfg[0] * cfg[2])
-    return layer.acc_gu[:ny, :B].sum(0)
+    n = 2 * layer.I                                               # partial sums are laid out [k-slice][B * topk of the call][2I]
+    return layer.acc_gu.view(-1)[: ny * B * n].view(ny, B, n).sum(0)
