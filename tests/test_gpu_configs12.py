@@ -73,4 +73,4 @@ def test_config2_single_projection(level):
         xg = O.wht(xf * signs["su_g"]).astype(np.float16).astype(np.float64)
         xu = O.wht(xf * signs["su_u"]).astype(np.float16).astype(np.float64)
         want = np.concatenate([xg @ Wq[:I].astype(np.float64).T, xu @ Wq[I:].astype(np.float64).T], 1)
-        assert rel_err(raw, want) < 2e-5, (level, B)
+        assert rel_err(raw, want) < 1e-4, (level, B)             # fp32 accumulation over K = 6144 with block-word extremes
