@@ -18,6 +18,7 @@
 // the arrival counters are zero on entry and are reset by the block that consumes them.
 #include "nq_tile.hpp"
 #include "nq_host.hpp"
+#include <algorithm>
 
 namespace nq {
 
@@ -59,12 +60,15 @@ __device__ __forceinline__ float2 sum_partials(const float* p, size_t stride, in
     return acc;
 }
 
+#ifndef NQ_OCC
+#define NQ_OCC
+#endif
 constexpr int MAXTOK = 16;                     // MFMA N: tokens of one run (B <= 8 -> at most 8 with distinct top-k ids)
 struct RunInfo { int e, level, ntok, nruns; int slot[MAXTOK]; const int64_t* ent; };
 
 // ---- routing dedup: picks -> runs, numbered by first occurrence; slots in pick order ---------------------------------
 // called by one full wavefront; lane s owns pick s (S <= 64). Fills run z.
-__device__ __forceinline__ void route(const MoeArgs& a, int z, RunInfo* R, int lane)
+__device__ __forceinline__ void route(const MoeArgs& a, int z, RunInfo* R, int lane, int rows)
 {
     const int S = a.B * a.topk;
     int e = -1; bool ok = false;
@@ -88,14 +92,14 @@ __device__ __forceinline__ void route(const MoeArgs& a, int z, RunInfo* R, int l
         if (r == z && ((m >> lane) & 1ull))
         {
             const int pos = __popcll(m & below);
-            if (pos < MAXTOK) R->slot[pos] = lane;
+            if (pos < rows) R->slot[pos] = lane;
             if (pos == 0)
             {
                 R->e = e; R->ent = a.table + (size_t)e * TBL_W;
                 const int lv = (int)R->ent[0];
                 R->level = a.force_level ? a.force_level : lv;
                 const int n = __popcll(m);
-                R->ntok = n < MAXTOK ? n : MAXTOK;
+                R->ntok = n < rows ? n : rows;
             }
         }
         rem &= ~m; ++r;
@@ -161,15 +165,15 @@ __device__ __forceinline__ void finish_dn(const MoeArgs& a, int grp, int NY, int
 
 // MODE 0: gate|up (N = 2I, K = H, input x rotated here). MODE 1: down (N = H, K = I, input h).
 // grid (N / 32 / SB, C / NC, S); block 64 * SB threads (SB = 1, 2 or 4: a block covers at most one 128-row group);
-// dynamic LDS = MAXTOK * (NC * 256 + 16) + 256 bytes (>= SB * 512 for the combine)
+// dynamic LDS = rows * (NC * 256 + 16) + 256 bytes (>= SB * 512 for the combine), rows = min(B * topk, MAXTOK) staged tokens
 template <int MODE>
-__global__ void __launch_bounds__(256) nq_gemv_k(MoeArgs a, int NC)
+__global__ void __launch_bounds__(256) NQ_OCC nq_gemv_k(MoeArgs a, int NC, int rows)
 {
     extern __shared__ __align__(16) char smem[];
     __shared__ RunInfo R;
     __shared__ int last;
     const int lane = threadIdx.x & 63, warp = threadIdx.x >> 6, SB = blockDim.x >> 6;
-    if (warp == 0) route(a, blockIdx.z, &R, lane);
+    if (warp == 0) route(a, blockIdx.z, &R, lane, rows);
     if (MODE == 0 && a.hits && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x < a.B * a.topk)
     {
         const long long ee = a.sel[threadIdx.x];
@@ -286,14 +290,15 @@ int launch_moe(const MoeArgs& a, const int* cfg_gu, const int* cfg_dn, int which
         const int NC = cf[0] * cf[2], SB = cf[1];
         const int N = mode == 0 ? 2 * a.I : a.H, K = mode == 0 ? a.H : a.I, C = K / 128;
         const int NX = N / 32 / SB, NY = C / NC;
-        const int shm = MAXTOK * (NC * 256 + 16) + 256;
+        const int rows = S < MAXTOK ? S : MAXTOK;
+        const int shm = std::max(rows * (NC * 256 + 16) + 256, SB * 512);
         auto kern = mode == 0 ? nq_gemv_k<0> : nq_gemv_k<1>;
         if (shm > 48 * 1024)
         {
             hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, shm);
             if (e != hipSuccess) return set_error("moe_forward: LDS %d bytes: %s", shm, hipGetErrorString(e));
         }
-        kern<<<dim3(NX, NY, S), 64 * SB, shm, st>>>(a, NC);
+        kern<<<dim3(NX, NY, S), 64 * SB, shm, st>>>(a, NC, rows);
         NQ_LAUNCH_CHECK("moe_forward");
     }
     return 0;
