@@ -44,83 +44,108 @@ __device__ __forceinline__ void ld_wait(float2& a, float2& b, float2& c, float2&
 {
     asm volatile("s_waitcnt vmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d) :: "memory");
 }
-// sum over k-slices y of the two floats at p + y * stride (device-coherent reads, four in flight at a time)
-__device__ __forceinline__ float2 sum_partials(const float* p, size_t stride, int NY)
+// sums over k-slices y of the two floats at p[q] + y * stride, for NR rows q at once: the reads of all rows are in flight
+// together, four slices per row at a time (device-coherent reads)
+template <int NR>
+__device__ __forceinline__ void sum_partials(const float* const* p, size_t stride, int NY, float2* out)
 {
-    float2 acc = make_float2(0.f, 0.f);
+#pragma unroll
+    for (int q = 0; q < NR; ++q) out[q] = make_float2(0.f, 0.f);
     for (int y = 0; y < NY; y += 4)
     {
-        float2 v[4];
+        float2 v[NR][4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) v[i] = ld_dev2_issue(p + (size_t)(y + i < NY ? y + i : y) * stride);
-        ld_wait(v[0], v[1], v[2], v[3]);
+        for (int q = 0; q < NR; ++q)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) if (y + i < NY) { acc.x += v[i].x; acc.y += v[i].y; }
+            for (int i = 0; i < 4; ++i) v[q][i] = ld_dev2_issue(p[q] + (size_t)(y + i < NY ? y + i : y) * stride);
+#pragma unroll
+        for (int q = 0; q < NR; ++q) ld_wait(v[q][0], v[q][1], v[q][2], v[q][3]);
+#pragma unroll
+        for (int q = 0; q < NR; ++q)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) if (y + i < NY) { out[q].x += v[q][i].x; out[q].y += v[q][i].y; }
     }
-    return acc;
 }
 
-#ifndef NQ_OCC
-#define NQ_OCC
-#endif
-constexpr int MAXTOK = 16;                     // MFMA N: tokens of one run (B <= 8 -> at most 8 with distinct top-k ids)
-struct RunInfo { int e, level, ntok, nruns; int slot[MAXTOK]; const int64_t* ent; };
+constexpr int MAXTOK = 8;                      // tokens of one run = tokens of one call (the MFMA N dimension holds 16)
+struct RunInfo
+{
+    Planes P;                     // this launch's projection of the run's expert
+    const _Float16* signs;        // su_g | sv_g | sv_u | su_d | sv_o | su_u
+    int level, ntok, nruns;
+    int slot[MAXTOK];
+    float pick_w[64];             // routing weight of every pick, 0 for picks that contribute nothing
+    const _Float16* pick_signs[64];
+};
 
 // ---- routing dedup: picks -> runs, numbered by first occurrence; slots in pick order ---------------------------------
-// called by one full wavefront; lane s owns pick s (S <= 64). Fills run z.
-__device__ __forceinline__ void route(const MoeArgs& a, int z, RunInfo* R, int lane, int rows)
+// called by one full wavefront; lane s owns pick s (S <= 64). Fills run z. A run takes at most one pick per token: a token
+// that names the same expert twice opens a second run of that expert, so a run never has more than B tokens. Every lane
+// requests the table-row fields of its own pick together with the level, so the leader's fields cost no second round trip.
+template <int MODE>
+__device__ __forceinline__ void route(const MoeArgs& a, int z, RunInfo* R, int lane)
 {
     const int S = a.B * a.topk;
-    int e = -1; bool ok = false;
+    int e = -1, lv = 0; bool ok = false;
+    int64_t f_base = 0, f_res = 0, f_dw = 0, f_var = 0, f_code = 0, f_signs = 0;
     if (lane < S)
     {
         const long long ee = a.sel[lane];
         if (ee >= 0 && ee < a.E)
         {
             e = (int)ee;
-            ok = (float)a.rw[lane] != 0.f && a.table[(size_t)e * TBL_W] > 0;
+            const int64_t* ent = a.table + (size_t)e * TBL_W;
+            constexpr int o = MODE == 0 ? 1 : 5;
+            lv = (int)ent[0];
+            f_base = ent[o]; f_res = ent[o + 1]; f_dw = ent[o + 2]; f_var = ent[MODE == 0 ? 12 : 13]; f_code = ent[10 + MODE]; f_signs = ent[9];
+            ok = (float)a.rw[lane] != 0.f && lv > 0;
         }
     }
     unsigned long long rem = __ballot(ok);
     const unsigned long long below = (1ull << lane) - 1ull;
+    const int tok = lane / a.topk, sh = tok * a.topk;
+    const unsigned long long mytok = sh < 64 ? (a.topk >= 64 ? ~0ull : ((1ull << a.topk) - 1ull)) << sh : 0ull;
     int r = 0;
     while (rem)
     {
         const int leader = __ffsll((long long)rem) - 1;
         const int ev = __shfl(e, leader);
-        const unsigned long long m = __ballot(ok && e == ev);
+        const unsigned long long same = __ballot(((rem >> lane) & 1ull) && e == ev);
+        const unsigned long long m = __ballot(((same >> lane) & 1ull) && (same & mytok & below) == 0ull);   // first pick per token
         if (r == z && ((m >> lane) & 1ull))
         {
             const int pos = __popcll(m & below);
-            if (pos < rows) R->slot[pos] = lane;
+            R->slot[pos] = lane;
             if (pos == 0)
             {
-                R->e = e; R->ent = a.table + (size_t)e * TBL_W;
-                const int lv = (int)R->ent[0];
+                Planes P;
+                P.base = (gp_u4)f_base; P.res = (gp_u8)f_res; P.dw = (gp_u32)f_dw; P.var = (gp_u8)f_var; P.code = (int)f_code;
+                R->P = P; R->signs = (const _Float16*)f_signs;
                 R->level = a.force_level ? a.force_level : lv;
-                const int n = __popcll(m);
-                R->ntok = n < rows ? n : rows;
+                R->ntok = __popcll(m);
             }
         }
         rem &= ~m; ++r;
     }
+    R->pick_w[lane] = ok ? (float)a.rw[lane] : 0.f; R->pick_signs[lane] = (const _Float16*)f_signs;
     if (lane == 0) R->nruns = r;
 }
 
 // finisher of gate|up for (run, 128-column group grp): h[slot] = fp16(WHT(silu(g) * u * su_d)), g = WHT(sum_y part_g) * sv_g
 __device__ __forceinline__ void finish_gu(const MoeArgs& a, const RunInfo& R, int grp, int NY, int warp, int SB, int lane)
 {
-    const _Float16* signs = (const _Float16*)R.ent[9];
-    const _Float16 *sv_g = signs + a.H, *sv_u = sv_g + a.I, *su_d = sv_u + a.I;
+    const _Float16 *sv_g = R.signs + a.H, *sv_u = sv_g + a.I, *su_d = sv_u + a.I;
     const int S = a.B * a.topk, col = grp * 128 + 2 * lane;
     for (int j = warp; j < R.ntok; j += SB)
     {
         const int s = R.slot[j];
         const float* p = a.part_gu + (size_t)s * 2 * a.I + col;
-        const float2 pg = sum_partials(p, (size_t)S * 2 * a.I, NY), pu = sum_partials(p + a.I, (size_t)S * 2 * a.I, NY);
-        float g0 = pg.x, g1 = pg.y, u0 = pu.x, u1 = pu.y;
-        wht128(g0, g1, lane); wht128(u0, u1, lane);
         const half2_t svg = *(const half2_t*)(sv_g + col), svu = *(const half2_t*)(sv_u + col), sud = *(const half2_t*)(su_d + col);
+        const float* const rows2[2] = {p, p + a.I};
+        float2 pq[2];
+        sum_partials<2>(rows2, (size_t)S * 2 * a.I, NY, pq);
+        float g0 = pq[0].x, g1 = pq[0].y, u0 = pq[1].x, u1 = pq[1].y;
+        wht128(g0, g1, lane); wht128(u0, u1, lane);
         g0 *= (float)svg.x; g1 *= (float)svg.y; u0 *= (float)svu.x; u1 *= (float)svu.y;
         float v0 = g0 / (1.f + __expf(-g0)) * u0 * (float)sud.x, v1 = g1 / (1.f + __expf(-g1)) * u1 * (float)sud.y;
         wht128(v0, v1, lane);
@@ -131,25 +156,35 @@ __device__ __forceinline__ void finish_gu(const MoeArgs& a, const RunInfo& R, in
 
 // combine of the down projection for output rows [grp * 128, +128): out[b] = sum_k rw[b,k] * sv_o[e] (.) WHT(sum_y part_d[slot])
 // picks of a token are spread over the block's wavefronts and reduced through LDS (red: SB * 128 floats)
-__device__ __forceinline__ void finish_dn(const MoeArgs& a, int grp, int NY, int warp, int SB, int lane, float* red)
+__device__ __forceinline__ void finish_dn(const MoeArgs& a, const RunInfo& R, int grp, int NY, int warp, int SB, int lane, float* red)
 {
     const int S = a.B * a.topk, col = grp * 128 + 2 * lane;
     for (int b = 0; b < a.B; ++b)
     {
         float o0 = 0.f, o1 = 0.f;
-        for (int k = warp; k < a.topk; k += SB)
+        for (int k = warp; k < a.topk; k += 2 * SB)              // two picks of this wavefront at a time, their reads in flight together
         {
-            const int s = b * a.topk + k;
-            const long long ee = a.sel[s];
-            const float w = (float)a.rw[s];
-            if (ee < 0 || ee >= a.E || w == 0.f) continue;
-            const int64_t* ent = a.table + (size_t)ee * TBL_W;
-            if (ent[0] <= 0) continue;
-            const float2 pv = sum_partials(a.part_d + (size_t)s * a.H + col, (size_t)S * a.H, NY);
-            float v0 = pv.x, v1 = pv.y;
-            wht128(v0, v1, lane);
-            const half2_t sv = *(const half2_t*)((const _Float16*)ent[9] + a.H + 3 * a.I + col);
-            o0 += w * (v0 * (float)sv.x); o1 += w * (v1 * (float)sv.y);
+            float2 pv[2] = {make_float2(0.f, 0.f), make_float2(0.f, 0.f)};
+            float w[2] = {0.f, 0.f};
+            half2_t sv[2] = {};
+            const float* rows2[2] = {a.part_d, a.part_d};
+#pragma unroll
+            for (int q = 0; q < 2; ++q)
+            {
+                const int kq = k + q * SB, s = b * a.topk + kq;
+                if (kq >= a.topk || R.pick_w[s] == 0.f) continue;     // what route() saw: no second look at the table
+                w[q] = R.pick_w[s]; rows2[q] = a.part_d + (size_t)s * a.H + col;
+                sv[q] = *(const half2_t*)(R.pick_signs[s] + a.H + 3 * a.I + col);
+            }
+            if (w[0] == 0.f && w[1] == 0.f) continue;
+            sum_partials<2>(rows2, (size_t)S * a.H, NY, pv);
+#pragma unroll
+            for (int q = 0; q < 2; ++q)
+            {
+                float v0 = pv[q].x, v1 = pv[q].y;
+                wht128(v0, v1, lane);
+                if (w[q] != 0.f) { o0 += w[q] * (v0 * (float)sv[q].x); o1 += w[q] * (v1 * (float)sv[q].y); }
+            }
         }
         red[warp * 128 + 2 * lane] = o0; red[warp * 128 + 2 * lane + 1] = o1;
         __syncthreads();
@@ -163,17 +198,23 @@ __device__ __forceinline__ void finish_dn(const MoeArgs& a, int grp, int NY, int
     }
 }
 
+__device__ __forceinline__ uint64_t uni(uint64_t v)
+{
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return (uint64_t)hi << 32 | lo;
+}
+
 // MODE 0: gate|up (N = 2I, K = H, input x rotated here). MODE 1: down (N = H, K = I, input h).
 // grid (N / 32 / SB, C / NC, S); block 64 * SB threads (SB = 1, 2 or 4: a block covers at most one 128-row group);
-// dynamic LDS = rows * (NC * 256 + 16) + 256 bytes (>= SB * 512 for the combine), rows = min(B * topk, MAXTOK) staged tokens
+// dynamic LDS = rows * (NC * 256 + 16) + 256 bytes (>= SB * 512 for the combine), one row per token of the call
 template <int MODE>
-__global__ void __launch_bounds__(256) NQ_OCC nq_gemv_k(MoeArgs a, int NC, int rows)
+__global__ void __launch_bounds__(256) nq_gemv_k(MoeArgs a, int NC)
 {
     extern __shared__ __align__(16) char smem[];
     __shared__ RunInfo R;
     __shared__ int last;
     const int lane = threadIdx.x & 63, warp = threadIdx.x >> 6, SB = blockDim.x >> 6;
-    if (warp == 0) route(a, blockIdx.z, &R, lane, rows);
+    if (warp == 0) route<MODE>(a, blockIdx.z, &R, lane);
     if (MODE == 0 && a.hits && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x < a.B * a.topk)
     {
         const long long ee = a.sel[threadIdx.x];
@@ -192,12 +233,14 @@ __global__ void __launch_bounds__(256) NQ_OCC nq_gemv_k(MoeArgs a, int NC, int r
     const int ntok = R.ntok, chunk0 = blockIdx.y * NC, k0 = chunk0 * 128;
     const int rowstride = NC * 256 + 16;                         // bytes per staged token (+16: spread tokens over banks)
     char* zero = smem + ntok * rowstride;                        // 256 zero bytes after the token rows
-    const _Float16* signs = (const _Float16*)R.ent[9];
+    const _Float16* signs = (const _Float16*)uni((uint64_t)R.signs);
 
     // ---- lane context; the first base record is requested now so that its latency overlaps the staging below
     const int t4 = lane >> 4, ss = (lane >> 3) & 1, g = lane & 7, n = lane & 15;
     const int strip = 2 * (blockIdx.x * SB + warp) + ss;
-    const Planes P = planes_of(R.ent, MODE);
+    Planes P;                                                    // block-uniform: keep the plane addresses in scalar registers
+    P.base = (gp_u4)uni((uint64_t)R.P.base); P.res = (gp_u8)uni((uint64_t)R.P.res); P.dw = (gp_u32)uni((uint64_t)R.P.dw);
+    P.var = (gp_u8)uni((uint64_t)R.P.var); P.code = __builtin_amdgcn_readfirstlane(R.P.code);
     LaneCtx L;
     L.unit0 = (size_t)strip * C + chunk0; L.rec0 = L.unit0 * 32 + 4 * g + t4;
     L.nrec = (size_t)(N / 16) * C * 32;
@@ -210,15 +253,31 @@ __global__ void __launch_bounds__(256) NQ_OCC nq_gemv_k(MoeArgs a, int NC, int r
     {
         const bool up = (int)(blockIdx.x * SB * 32) >= a.I;      // gate rows use su_g, up rows su_u
         const _Float16* su = up ? signs + 2 * a.H + 3 * a.I : signs;
-        for (int task = warp; task < ntok * NC; task += SB)
+        // task = (token j, chunk c); a wavefront takes tasks warp, warp + SB, .. four at a time so that their activation and
+        // scale reads are in flight together
+        const int ntask = ntok * NC;
+        for (int t0 = warp; t0 < ntask; t0 += 4 * SB)
         {
-            const int j = task / NC, c = task % NC, kk = k0 + c * 128 + 2 * lane;
-            const int tok = R.slot[j] / a.topk;
-            const half2_t xv = *(const half2_t*)(a.x + (size_t)tok * a.H + kk), sv = *(const half2_t*)(su + kk);
-            float v0 = (float)xv.x * (float)sv.x, v1 = (float)xv.y * (float)sv.y;
-            wht128(v0, v1, lane);
-            _Float16* dst = (_Float16*)(smem + j * rowstride + c * 256);
-            dst[bop_index(2 * lane)] = (_Float16)v0; dst[bop_index(2 * lane + 1)] = (_Float16)v1;
+            half2_t xv[4], sv[4];
+            int dsto[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+            {
+                const int task = t0 + u * SB < ntask ? t0 + u * SB : t0;
+                const int j = task / NC, c = task - j * NC, kk = k0 + c * 128 + 2 * lane;
+                const int tok = R.slot[j] / a.topk;
+                xv[u] = *(const half2_t*)(a.x + (size_t)tok * a.H + kk); sv[u] = *(const half2_t*)(su + kk);
+                dsto[u] = j * rowstride + c * 256;
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+            {
+                if (t0 + u * SB >= ntask) break;
+                float v0 = (float)xv[u].x * (float)sv[u].x, v1 = (float)xv[u].y * (float)sv[u].y;
+                wht128(v0, v1, lane);
+                _Float16* dst = (_Float16*)(smem + dsto[u]);
+                dst[bop_index(2 * lane)] = (_Float16)v0; dst[bop_index(2 * lane + 1)] = (_Float16)v1;
+            }
         }
     }
     else
@@ -261,7 +320,7 @@ __global__ void __launch_bounds__(256) NQ_OCC nq_gemv_k(MoeArgs a, int NC, int r
     __syncthreads();
     if (!last) return;                                           // block-uniform
     if constexpr (MODE == 0) finish_gu(a, R, grp, NY, warp, SB, lane);
-    else finish_dn(a, grp, NY, warp, SB, lane, (float*)smem);
+    else finish_dn(a, R, grp, NY, warp, SB, lane, (float*)smem);
     if (threadIdx.x == 0) __hip_atomic_store(cnt, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
@@ -290,15 +349,14 @@ int launch_moe(const MoeArgs& a, const int* cfg_gu, const int* cfg_dn, int which
         const int NC = cf[0] * cf[2], SB = cf[1];
         const int N = mode == 0 ? 2 * a.I : a.H, K = mode == 0 ? a.H : a.I, C = K / 128;
         const int NX = N / 32 / SB, NY = C / NC;
-        const int rows = S < MAXTOK ? S : MAXTOK;
-        const int shm = std::max(rows * (NC * 256 + 16) + 256, SB * 512);
+        const int shm = std::max(a.B * (NC * 256 + 16) + 256, SB * 512);
         auto kern = mode == 0 ? nq_gemv_k<0> : nq_gemv_k<1>;
         if (shm > 48 * 1024)
         {
             hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, shm);
             if (e != hipSuccess) return set_error("moe_forward: LDS %d bytes: %s", shm, hipGetErrorString(e));
         }
-        kern<<<dim3(NX, NY, S), 64 * SB, shm, st>>>(a, NC, rows);
+        kern<<<dim3(NX, NY, S), 64 * SB, shm, st>>>(a, NC);
         NQ_LAUNCH_CHECK("moe_forward");
     }
     return 0;

@@ -64,6 +64,8 @@ def test_small_layer_all_levels_and_codes_vs_full_oracle():
         sel, rw = RT.routing_tensors(rows, seed=B)
         if B == 3:
             rw[1, 2] = 0
+        if B == 2:
+            sel[0, 1] = sel[0, 0]; sel[1, 3] = sel[1, 0]             # a token naming one expert twice: both picks count
         x = (torch.randn(B, H, generator=g) * 0.05).half().to(DEV)
         want = oracle_layer(planes, levels, signs, x, sel, rw)
         for cg, cd in (([1, 4, 2], [1, 4, 2]), ([1, 1, 1], [2, 2, 1]), ([2, 4, 2], [1, 2, 1])):
