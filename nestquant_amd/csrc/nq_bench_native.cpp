@@ -4,7 +4,10 @@
 // (--pmc FETCH_SIZE / WRITE_SIZE) can wrap; `--calib` adds one 256 MiB device copy as the known-size kernel that scales
 // those counters.
 //
-//   nq_bench_native [--experts 64] [--batch 1] [--steps 32] [--calib]
+//   nq_bench_native [--experts 64] [--batch 1] [--steps 32] [--calib] [--level L] [--prefill ROWS]
+//
+// --prefill ROWS times the decode-fused grouped GEMMs of the prefill path instead (nq_pf_gemm, gate|up then down): every
+// expert gets ROWS pair rows (<= 256, one tile each); --level L puts every expert at level L.
 //
 // Planes are pseudo-random words (the decoder's cost does not depend on the values); levels cycle 2,2,2,3,4,2,2,4 so
 // every step mixes levels; each step routes to 8 experts not used by the step before.
@@ -40,15 +43,18 @@ __global__ void copy_words(const uint4* __restrict__ a, uint4* __restrict__ b, s
 
 int main(int argc, char** argv)
 {
-    int E = 64, B = 1, steps = 32, calib = 0;
+    int E = 64, B = 1, steps = 32, calib = 0, level = 0, pf_rows = 0;
     for (int i = 1; i < argc; ++i)
     {
         if (!strcmp(argv[i], "--experts") && i + 1 < argc) E = atoi(argv[++i]);
         else if (!strcmp(argv[i], "--batch") && i + 1 < argc) B = atoi(argv[++i]);
         else if (!strcmp(argv[i], "--steps") && i + 1 < argc) steps = atoi(argv[++i]);
         else if (!strcmp(argv[i], "--calib")) calib = 1;
-        else { fprintf(stderr, "usage: %s [--experts E>=16] [--batch B<=8] [--steps K] [--calib]\n", argv[0]); return 2; }
+        else if (!strcmp(argv[i], "--level") && i + 1 < argc) level = atoi(argv[++i]);
+        else if (!strcmp(argv[i], "--prefill") && i + 1 < argc) pf_rows = atoi(argv[++i]);
+        else { fprintf(stderr, "usage: %s [--experts E>=16] [--batch B<=8] [--steps K] [--calib] [--level 2|3|4] [--prefill ROWS<=256]\n", argv[0]); return 2; }
     }
+    if ((level && level != 2 && level != 3 && level != 4) || pf_rows < 0 || pf_rows > 256) { fprintf(stderr, "need level in {2,3,4} and 0 <= ROWS <= 256\n"); return 2; }
     if (E < 16 || B < 1 || B > 8) { fprintf(stderr, "need E >= 16 and 1 <= B <= 8\n"); return 2; }
     const int H = 6144, I = 2048, topk = 8, S = B * topk;
     const size_t rec_gu = (size_t)(2 * I / 16) * (H / 128) * 32, rec_dn = (size_t)(H / 16) * (I / 128) * 32;
@@ -60,7 +66,7 @@ int main(int argc, char** argv)
     size_t plane_bytes = 0;
     for (int e = 0; e < E; ++e)
     {
-        const int lv = LV[e % 8];
+        const int lv = level ? level : LV[e % 8];
         int64_t* r = &table[(size_t)e * NQ_TBL_W];
         r[0] = lv; r[9] = (int64_t)signs;
         const size_t recs[2] = {rec_gu, rec_dn}, units[2] = {units_gu, units_dn};
@@ -82,6 +88,34 @@ int main(int argc, char** argv)
     }
     int64_t* d_table; HIPCHK(hipMalloc(&d_table, table.size() * 8));
     HIPCHK(hipMemcpy(d_table, table.data(), table.size() * 8, hipMemcpyHostToDevice));
+
+    if (pf_rows)
+    {
+        const int np = E * pf_rows;
+        int bm = 16; while (bm < pf_rows) bm *= 2;
+        uint16_t *xg, *xu, *hh; float *cgu, *cdn; int32_t* tiles;
+        HIPCHK(hipMalloc(&xg, (size_t)np * H * 2)); HIPCHK(hipMalloc(&xu, (size_t)np * H * 2)); HIPCHK(hipMalloc(&hh, (size_t)np * I * 2));
+        HIPCHK(hipMalloc(&cgu, (size_t)np * 2 * I * 4)); HIPCHK(hipMalloc(&cdn, (size_t)np * H * 4));
+        fill_half<<<1024, 256>>>(xg, (size_t)np * H, 0x2A66); fill_half<<<1024, 256>>>(xu, (size_t)np * H, 0x2A66); fill_half<<<1024, 256>>>(hh, (size_t)np * I, 0x2A66);
+        std::vector<int32_t> ht((size_t)E * 4);
+        for (int e = 0; e < E; ++e) { ht[4 * e] = e; ht[4 * e + 1] = e * pf_rows; ht[4 * e + 2] = pf_rows; ht[4 * e + 3] = 0; }
+        HIPCHK(hipMalloc(&tiles, ht.size() * 4)); HIPCHK(hipMemcpy(tiles, ht.data(), ht.size() * 4, hipMemcpyHostToDevice));
+        hipEvent_t e0, e1; HIPCHK(hipEventCreate(&e0)); HIPCHK(hipEventCreate(&e1));
+        NQCHK(nq_pf_gemm(d_table, tiles, E, bm, 0, xg, xu, cgu, E, H, I, nullptr)); NQCHK(nq_pf_gemm(d_table, tiles, E, bm, 1, hh, nullptr, cdn, E, H, I, nullptr));
+        HIPCHK(hipDeviceSynchronize());
+        HIPCHK(hipEventRecord(e0, nullptr));
+        for (int st = 0; st < steps; ++st)
+        {
+            NQCHK(nq_pf_gemm(d_table, tiles, E, bm, 0, xg, xu, cgu, E, H, I, nullptr));
+            NQCHK(nq_pf_gemm(d_table, tiles, E, bm, 1, hh, nullptr, cdn, E, H, I, nullptr));
+        }
+        HIPCHK(hipEventRecord(e1, nullptr)); HIPCHK(hipEventSynchronize(e1));
+        float ms; HIPCHK(hipEventElapsedTime(&ms, e0, e1));
+        const double flop = 2.0 * np * 3.0 * H * I;
+        printf("nq_bench_native prefill: E=%d tiles of %d rows (height %d), level %d: %.3f ms per gate|up + down pair, %.1f TFLOP/s, %.2f us per tile\n",
+               E, pf_rows, bm, level, ms / steps, flop / (ms / steps * 1e-3) / 1e12, ms * 1e3 / steps / E);
+        return 0;
+    }
 
     const int cfg_gu[4] = {1, 4, 12, 0}, cfg_dn[4] = {1, 4, 4, 0};
     const int ny_gu = H / 128 / (cfg_gu[0] * cfg_gu[2]), ny_dn = I / 128 / (cfg_dn[0] * cfg_dn[2]);

@@ -147,7 +147,7 @@ extern "C" int nq_pf_mid(const float* acc_gu, const int32_t* pe, int np, const i
 extern "C" int nq_pf_post(const float* y, const int32_t* pos, const int64_t* sel, const void* rw, int T, int topk, int row_lo, int nrows,
                           const int64_t* table, float* out, int E, int H, int I, void* stream)
 {
-    NQ_REQUIRE(T >= 0 && nrows >= 0 && topk >= 1 && row_lo >= 0, "nq_pf_post: T=%d topk=%d row_lo=%d nrows=%d", T, topk, row_lo, nrows);
+    NQ_REQUIRE(T >= 0 && nrows >= 0 && topk >= 1 && topk <= 64 && row_lo >= 0, "nq_pf_post: T=%d topk=%d (<= 64) row_lo=%d nrows=%d", T, topk, row_lo, nrows);
     if (T == 0 || nrows == 0) return 0;
     NQ_REQUIRE(y && pos && sel && rw && table && out, "nq_pf_post: null pointer");
     NQ_REQUIRE(E >= 1 && shape_ok(H, I), "nq_pf_post: E=%d H=%d I=%d (H, I positive multiples of 128)", E, H, I);

@@ -16,7 +16,7 @@
 
 namespace nq {
 
-constexpr int PF_ROW = 272;                    // LDS bytes per staged token: 256 + 16 (spreads tokens over banks)
+constexpr int PF_ROW = 256;                    // LDS bytes per staged token and chunk; 16-byte column q of row r sits in slot q ^ (r & 15)
 
 // lane holds columns 2 lane, 2 lane + 1 of a 128-column chunk; columns c and c + 16 are neighbours in the B-operand order,
 // so lanes l and l ^ 8 swap one value each and every lane stores one aligned 4-byte pair
@@ -93,29 +93,54 @@ __global__ void __launch_bounds__(256) nq_pf_post_k(const float* __restrict__ y,
                                                      const int64_t* __restrict__ table, float* out, int E, int H, int I)
 {
     const int t = blockIdx.x, lane = threadIdx.x & 63, warp = threadIdx.x >> 6;
+    // the token's live picks, gathered once: row, weight and sign vector (picks keep their order, so does the sum)
+    __shared__ int p_row[64]; __shared__ float p_w[64]; __shared__ const _Float16* p_sv[64]; __shared__ int p_n;
+    if (warp == 0)
+    {
+        bool ok = false; int r = 0; float w = 0.f; const _Float16* sv = nullptr;
+        if (lane < topk)
+        {
+            r = pos[(size_t)t * topk + lane] - row_lo;
+            const long long e = sel[(size_t)t * topk + lane];
+            w = (float)rw[(size_t)t * topk + lane];
+            if (r >= 0 && r < nrows && e >= 0 && e < E && w != 0.f && table[(size_t)e * TBL_W] > 0)
+            {
+                ok = true; sv = (const _Float16*)table[(size_t)e * TBL_W + 9] + H + 3 * I;
+            }
+        }
+        const unsigned long long m = __ballot(ok);
+        if (ok) { const int i = __popcll(m & ((1ull << lane) - 1ull)); p_row[i] = r; p_w[i] = w; p_sv[i] = sv; }
+        if (lane == 0) p_n = __popcll(m);
+    }
+    __syncthreads();
+    const int np = p_n;
+    if (np == 0) return;
     for (int grp = warp; grp < H / 128; grp += 4)
     {
         const int col = grp * 128 + 2 * lane;
         float o0 = 0.f, o1 = 0.f;
-        bool any = false;
-        for (int k = 0; k < topk; ++k)
+        for (int k0 = 0; k0 < np; k0 += 4)                       // four picks at a time, reads first
         {
-            const int r = pos[(size_t)t * topk + k] - row_lo;
-            const long long e = sel[(size_t)t * topk + k];
-            const float w = (float)rw[(size_t)t * topk + k];
-            if (r < 0 || r >= nrows || e < 0 || e >= E || w == 0.f || table[(size_t)e * TBL_W] <= 0) continue;
-            const float2 v = *(const float2*)(y + (size_t)r * H + col);
-            float v0 = v.x, v1 = v.y;
-            wht128(v0, v1, lane);
-            const half2_t sv = *(const half2_t*)((const _Float16*)table[(size_t)e * TBL_W + 9] + H + 3 * I + col);
-            o0 += w * (v0 * (float)sv.x); o1 += w * (v1 * (float)sv.y);
-            any = true;
+            float2 v[4]; half2_t sv[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+            {
+                const int k = k0 + u < np ? k0 + u : k0;
+                v[u] = *(const float2*)(y + (size_t)p_row[k] * H + col);
+                sv[u] = *(const half2_t*)(p_sv[k] + col);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+            {
+                if (k0 + u >= np) break;
+                float v0 = v[u].x, v1 = v[u].y;
+                wht128(v0, v1, lane);
+                const float w = p_w[k0 + u];
+                o0 += w * (v0 * (float)sv[u].x); o1 += w * (v1 * (float)sv[u].y);
+            }
         }
-        if (any)
-        {
-            float2* op = (float2*)(out + (size_t)t * H + col);
-            float2 cur = *op; cur.x += o0; cur.y += o1; *op = cur;
-        }
+        float2* op = (float2*)(out + (size_t)t * H + col);
+        float2 cur = *op; cur.x += o0; cur.y += o1; *op = cur;
     }
 }
 
@@ -142,17 +167,29 @@ __device__ __forceinline__ void pf_chunks(const Planes& P, const LaneCtx& L, int
     uint32_t nr[NW + 2] = {0}, ndw = 0, nvar = 0;
     if constexpr (RES) { load_record<CODE>(nr, P.res, L.rec0, L.nrec); ndw = P.dw[L.unit0]; }
     if (P.var) nvar = P.var[L.unit0];
-    const int t4 = threadIdx.x >> 4 & 3, n = threadIdx.x & 15, ntg = (nrows + 15) >> 4;
+    const int lane = threadIdx.x & 63, warp = threadIdx.x >> 6, t4 = lane >> 4, n = lane & 15;
+    // Staging: wavefront w copies rows 16 u + 4 w + (lane >> 4), u = 0 .. TG - 1, of the tile, one 1 KB
+    // global -> LDS load per u (64 lanes x 16 bytes land in LDS in lane order, so a load fills 4 rows x 256 bytes). The
+    // lane picks which 16-byte column of its row it fetches: column (lane & 15) ^ (row & 15) goes to slot lane & 15, and
+    // the MFMA reads undo the XOR, which spreads the 16 tokens of an operand read over all banks without padding.
+    // Rows beyond the tile re-read its last row: their products are never stored.
+    const int srow = 4 * warp + t4;                              // row & 15 of every row this lane stages
+    const uint32_t scol = (uint32_t)((n ^ srow) * 16);           // byte offset of the fetched column inside the chunk
+    uint32_t boff[4];                                            // B-operand read offsets of this lane for mm = 0..3
+#pragma unroll
+    for (int mm = 0; mm < 4; ++mm) boff[mm] = (uint32_t)(n * PF_ROW + (((4 * mm + t4) ^ n) << 4));
+    typedef const __attribute__((address_space(1))) void* gvp;
+    typedef __attribute__((address_space(3))) void* lvp;
     for (int c = 0; c < C; ++c)
     {
-        // ---- stage the tile's tokens for chunk c (rows beyond the tile read as zero)
-        __syncthreads();
-        for (int i = threadIdx.x; i < ntg * 16 * 16; i += blockDim.x)
+        // ---- request the tile's tokens for chunk c (asynchronous: the decode below runs while they arrive)
+#pragma unroll
+        for (int u = 0; u < TG; ++u)
         {
-            const int tok = i >> 4, q = i & 15;
-            uint4 v = make_uint4(0, 0, 0, 0);
-            if (tok < nrows) v = *(const uint4*)(A + (size_t)(row0 + tok) * K + c * 128 + q * 8);
-            *(uint4*)(smem + tok * PF_ROW + q * 16) = v;
+            if (16 * u >= nrows) break;                          // block-uniform
+            const int row = 16 * u + srow, grow = row < nrows ? row : nrows - 1;
+            const char* src = (const char*)A + ((size_t)(row0 + grow) * K + c * 128) * 2 + scol;
+            __builtin_amdgcn_global_load_lds((gvp)src, (lvp)(smem + (16 * u + 4 * warp) * PF_ROW), 16, 0, 0);
         }
         // ---- decode this wave's unit pair of chunk c into A operands; prefetch chunk c + 1
         uint32_t wb[6], wr[NW + 2];
@@ -181,11 +218,11 @@ __device__ __forceinline__ void pf_chunks(const Planes& P, const LaneCtx& L, int
             aop[MM][0] = a_operand<RES, CODE, MM, 0>(wb, wr, k);
             aop[MM][1] = a_operand<RES, CODE, MM, 1>(wb, wr, k);
         });
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");         // this wavefront's share of the tile has landed
         __syncthreads();
         // ---- TG x 8 MFMAs: tokens 16 tg + n as the N dimension (row groups beyond the tile multiply stale LDS rows whose
         // results are never stored). Two row groups are interleaved so that four different accumulators separate an MFMA
         // from the next one that depends on it.
-        const char* xp = smem + n * PF_ROW + t4 * 16;
         constexpr int TS = TG >= 2 ? 2 : 1;
 #pragma unroll
         for (int tg = 0; tg < TG; tg += TS)
@@ -196,18 +233,21 @@ __device__ __forceinline__ void pf_chunks(const Planes& P, const LaneCtx& L, int
 #pragma unroll
                 for (int u = 0; u < TS; ++u)
                 {
-                    const half8_t b = *(const half8_t*)(xp + (tg + u) * 16 * PF_ROW + mm * 64);
+                    const half8_t b = *(const half8_t*)(smem + boff[mm] + (tg + u) * 16 * PF_ROW);
                     acc[tg + u][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aop[mm][0], b, acc[tg + u][0], 0, 0, 0);
                     acc[tg + u][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aop[mm][1], b, acc[tg + u][1], 0, 0, 0);
                 }
             }
         }
+        __syncthreads();                                         // every wavefront has read chunk c before chunk c + 1 overwrites it
     }
 }
 
 // grid (N / 128, ntiles), block 256 (4 wavefronts x 2 strips = 128 weight rows); dynamic LDS = 16 TG * PF_ROW bytes
+// two workgroups per CU at every tile height (the tallest would otherwise need one register too many): while one decodes on
+// the vector ALUs the other runs its MFMAs
 template <int TG>
-__global__ void __launch_bounds__(256) nq_pf_gemm_k(PfGemm a)
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) nq_pf_gemm_k(PfGemm a)
 {
     extern __shared__ __align__(16) char smem[];
     const int lane = threadIdx.x & 63, warp = threadIdx.x >> 6;
