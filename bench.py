@@ -29,7 +29,7 @@ HBM_PEAK_GBS = 8000.0
 MFMA_PEAK_TFLOPS = 2500.0            # dense fp16 / bf16 MFMA peak of MI355X
 # HBM bytes per gate|up launch / algorithmic bytes, from rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a 256 MiB copy kernel
 # (profiles/decode_gemv_hbm_traffic_pmc.txt)
-TRAFFIC_RATIO = 1.037
+TRAFFIC_RATIO = 1.029
 
 
 def build_layer(dev, seed=0, Bmax=4):
