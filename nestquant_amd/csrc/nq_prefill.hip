@@ -223,20 +223,50 @@ __device__ __forceinline__ void pf_chunks(const Planes& P, const LaneCtx& L, int
         // ---- TG x 8 MFMAs: tokens 16 tg + n as the N dimension (row groups beyond the tile multiply stale LDS rows whose
         // results are never stored). Two row groups are interleaved so that four different accumulators separate an MFMA
         // from the next one that depends on it.
-        constexpr int TS = TG >= 2 ? 2 : 1;
-#pragma unroll
-        for (int tg = 0; tg < TG; tg += TS)
+        constexpr int TS = TG >= 2 ? 2 : 1, NGRP = TG / TS * 4, PD = TG >= 16 ? 2 : 1;      // read-ahead depth in groups
+        if constexpr (PD == 0)
         {
 #pragma unroll
-            for (int mm = 0; mm < 4; ++mm)
+            for (int tg = 0; tg < TG; tg += TS)
             {
+#pragma unroll
+                for (int mm = 0; mm < 4; ++mm)
+                {
+#pragma unroll
+                    for (int u = 0; u < TS; ++u)
+                    {
+                        const half8_t b = *(const half8_t*)(smem + boff[mm] + (tg + u) * 16 * PF_ROW);
+                        acc[tg + u][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aop[mm][0], b, acc[tg + u][0], 0, 0, 0);
+                        acc[tg + u][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aop[mm][1], b, acc[tg + u][1], 0, 0, 0);
+                    }
+                }
+            }
+        }
+        else
+        {
+            // operand reads run PD groups ahead of the MFMAs that use them (a group = one mm of TS row groups)
+            half8_t bq[PD + 1][TS];
+            auto bread = [&](int grp, half8_t* dst) {
+                const int tg = grp / 4 * TS, mm = grp % 4;
+#pragma unroll
+                for (int u = 0; u < TS; ++u) dst[u] = *(const half8_t*)(smem + boff[mm] + (tg + u) * 16 * PF_ROW);
+            };
+#pragma unroll
+            for (int gq = 0; gq < PD; ++gq) bread(gq, bq[gq]);
+#pragma unroll
+            for (int gq = 0; gq < NGRP; ++gq)
+            {
+                if (gq + PD < NGRP) bread(gq + PD, bq[(gq + PD) % (PD + 1)]);
+                __builtin_amdgcn_sched_barrier(0);
+                const int tg = gq / 4 * TS, mm = gq % 4;
 #pragma unroll
                 for (int u = 0; u < TS; ++u)
                 {
-                    const half8_t b = *(const half8_t*)(smem + boff[mm] + (tg + u) * 16 * PF_ROW);
+                    const half8_t b = bq[gq % (PD + 1)][u];
                     acc[tg + u][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aop[mm][0], b, acc[tg + u][0], 0, 0, 0);
                     acc[tg + u][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aop[mm][1], b, acc[tg + u][1], 0, 0, 0);
                 }
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
         __syncthreads();                                         // every wavefront has read chunk c before chunk c + 1 overwrites it
