@@ -154,6 +154,48 @@ def prefill_leg(L, ex, dev, T=4096, reps=3):
                 note="whole prefill() call: sort, pre, 2 decode-fused grouped GEMMs, mid, post; bound by the VALU trellis decode")
 
 
+def caller_leg(L, MB, routes, xs, dev, reps=4):
+    """The serving caller's tensors (bf16 hidden states, fp32 routing weights, int32 ids, bf16 result; reference
+    sm120/serve/nq_vllm.py:520-574): the layer step with the casts as separate torch kernels around an fp16 call, as the
+    reference's caller runs it, against the same step with the kernels reading and writing the caller's types."""
+    R, B = len(routes), xs[0].shape[0]
+    xb = [x.bfloat16() for x in xs]
+    wf = [r[1].float() for r in routes]
+    idi = [r[0].int() for r in routes]
+    outb = torch.zeros(R, B, H, dtype=torch.bfloat16, device=dev)
+    s = torch.cuda.Stream()
+
+    def cast_step(i):
+        MB.apply()
+        outb[i].copy_(L(xb[i].half(), idi[i].long(), wf[i].half()))
+
+    def fused_step(i):
+        MB.apply()
+        L(xb[i], idi[i], wf[i], out=outb[i])
+
+    res = {}
+    for name, fn in (("casts_around_call", cast_step), ("fused_in_kernels", fused_step)):
+        with torch.cuda.stream(s):
+            for i in range(R):
+                fn(i)
+        torch.cuda.synchronize()
+        keep = outb.clone()
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr, stream=s):
+            for i in range(R):
+                fn(i)
+        gr.replay(); torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            gr.replay()
+        torch.cuda.synchronize()
+        res[name] = (round((time.perf_counter() - t0) / (reps * R) * 1e6, 2), keep)
+    assert torch.equal(res["casts_around_call"][1], res["fused_in_kernels"][1]), "fused dtype handling differs from explicit casts"
+    return {"workload": "decode layer step from bf16 activations, fp32 routing weights, int32 ids to a bf16 result (B=1)",
+            "us_casts_around_call": res["casts_around_call"][0], "us_fused_in_kernels": res["fused_in_kernels"][0],
+            "results": "bitwise equal"}
+
+
 def churn_leg(L, MB, ex, levels, routes, xs, dev, steps=64, ops_per_step=8):
     """config 5: B=1 layer steps with 8 promote/demote ops per step issued on a side stream (pinned host -> slot copies)"""
     from nestquant_amd import churn as CH
@@ -233,6 +275,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill (4096 tokens) leg")
     ap.add_argument("--no-churn", action="store_true", help="skip the plane-churn leg")
+    ap.add_argument("--no-caller", action="store_true", help="skip the caller-dtype leg (bf16 / fp32 / int32 tensors)")
     ap.add_argument("--calib", action="store_true", help="also run one 256 MiB device copy (reads 256 MiB, writes 256 MiB): "
                     "the known-size kernel that scales rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
     a = ap.parse_args()
@@ -326,6 +369,7 @@ def main():
         cpu, _ = cpu_baseline(ex, levels, routes[0][2][0], xs[0])
     lv_counts = {lv: levels.count(lv) for lv in (2, 3, 4)}
     prefill = None if a.no_prefill else prefill_leg(L, ex, dev)
+    caller = None if a.no_caller else caller_leg(L, MB, routes, xs, dev)
     churn = None if a.no_churn else churn_leg(L, MB, ex, levels, routes[:16], xs, dev)
     print(json.dumps({
         "metric": "MoE layer us + HBM GB/s (decode bs1 top-8); prefill grouped-GEMM TFLOP/s",
@@ -335,7 +379,7 @@ def main():
         "config": {"workload": f"decode MoE layer: E=256 top-8 B={B}, H=6144 I=2048, levels 2/3/4 = "
                                f"{lv_counts[2]}/{lv_counts[3]}/{lv_counts[4]} experts, seeded softmax routing avoiding the previous step",
                    "code_MB_per_step": round(nbytes / K / 1e6, 2), "hbm_frac_layer": round(gbs / HBM_PEAK_GBS, 4)},
-        "roofline": roofline, "cpu_baseline": cpu, "prefill": prefill, "churn": churn}))
+        "roofline": roofline, "cpu_baseline": cpu, "prefill": prefill, "caller_dtypes": caller, "churn": churn}))
 
 
 if __name__ == "__main__":

@@ -55,13 +55,19 @@ int nq_pf_decode(const int64_t* table, const int32_t* experts, int G, void* Wgu_
  * reference's workspace contract, sm120/nqmoe.cu:855-857). Picks with rw == 0, level <= 0 or an expert id outside
  * [0, E) contribute nothing. which: bit 0 = gate|up launch, bit 1 = down launch. hits: optional int32[E] pick counters
  * (device or host-mapped memory), incremented once per pick with rw != 0 (reference :784-787). */
+/* Element types of the caller's tensors. The casts the reference's caller launches around the call (x.half(), ids.long(),
+ * w.half(), out.to(x.dtype): sm120/serve/nq_vllm.py:522,560,573; fusing them is the open item of
+ * threads/13-moe-layer-kernel/INTEGRATION.md:191-192) happen inside the kernels with the same roundings: x and rw pass
+ * through fp16, the fp32 result is rounded once to the output type. */
+enum { NQ_DT_F16 = 0, NQ_DT_BF16 = 1, NQ_DT_F32 = 2, NQ_DT_I64 = 0, NQ_DT_I32 = 1, NQ_DT_OUT_F32 = 0, NQ_DT_OUT_F16 = 1, NQ_DT_OUT_BF16 = 2 };
+
 typedef struct NqMoeArgs
 {
-    const void* x;            /* fp16 [B][H] */
-    const int64_t* sel;       /* int64 [B][topk] */
-    const void* rw;           /* fp16 [B][topk] */
+    const void* x;            /* [B][H], x_dtype */
+    const void* sel;          /* [B][topk], sel_dtype */
+    const void* rw;           /* [B][topk], rw_dtype */
     const int64_t* table;     /* int64 [E][NQ_TBL_W] */
-    void* out;                /* fp32 [B][H] */
+    void* out;                /* [B][H], out_dtype */
     void* acc_gu;             /* fp32 workspace */
     void* h;                  /* fp16 workspace */
     void* acc_d;              /* fp32 workspace */
@@ -73,6 +79,10 @@ typedef struct NqMoeArgs
     int32_t cfg_gu[4], cfg_dn[4];
     int32_t force_level;      /* 0, or a level that overrides every active row's level (debug) */
     int32_t which;
+    int32_t x_dtype;          /* NQ_DT_F16 (0), NQ_DT_BF16, NQ_DT_F32: element type of x */
+    int32_t sel_dtype;        /* NQ_DT_I64 (0) or NQ_DT_I32 */
+    int32_t rw_dtype;         /* NQ_DT_F16 (0), NQ_DT_BF16, NQ_DT_F32 */
+    int32_t out_dtype;        /* NQ_DT_OUT_F32 (0), NQ_DT_OUT_F16, NQ_DT_OUT_BF16: element type of out */
 } NqMoeArgs;
 int nq_moe_forward(const NqMoeArgs* args, void* stream);
 

@@ -83,6 +83,8 @@ extern "C" int nq_moe_forward(const NqMoeArgs* p, void* stream)
     NQ_REQUIRE(shape_ok(p->H, p->I), "nq_moe_forward: H=%d I=%d must be positive multiples of 128", p->H, p->I);
     NQ_REQUIRE((p->which & ~3) == 0, "nq_moe_forward: which=%d", p->which);
     NQ_REQUIRE(p->force_level == 0 || p->force_level == 2 || p->force_level == 3 || p->force_level == 4, "nq_moe_forward: force_level=%d", p->force_level);
+    NQ_REQUIRE(p->x_dtype >= 0 && p->x_dtype <= 2 && p->rw_dtype >= 0 && p->rw_dtype <= 2 && p->sel_dtype >= 0 && p->sel_dtype <= 1 && p->out_dtype >= 0 && p->out_dtype <= 2,
+               "nq_moe_forward: dtype codes x=%d sel=%d rw=%d out=%d", p->x_dtype, p->sel_dtype, p->rw_dtype, p->out_dtype);
     const int64_t S = (int64_t)p->B * p->topk;
     for (int mode = 0; mode < 2; ++mode)
     {
@@ -98,9 +100,10 @@ extern "C" int nq_moe_forward(const NqMoeArgs* p, void* stream)
     NQ_REQUIRE(p->h_elems >= S * p->I && p->out_elems >= (int64_t)p->B * p->H, "workspace too small: h or out");
     NQ_REQUIRE(p->cnt_gu_elems >= S * (p->I / 128) && p->cnt_d_elems >= p->H / 128, "workspace too small: cnt_gu or cnt_d");
     MoeArgs a{};
-    a.x = (const _Float16*)p->x; a.sel = p->sel; a.rw = (const _Float16*)p->rw; a.B = p->B; a.topk = p->topk;
+    a.x = p->x; a.sel = p->sel; a.rw = p->rw; a.B = p->B; a.topk = p->topk;
+    a.x_dtype = p->x_dtype; a.sel_dtype = p->sel_dtype; a.rw_dtype = p->rw_dtype; a.out_dtype = p->out_dtype;
     a.table = p->table; a.E = p->E; a.H = p->H; a.I = p->I;
-    a.part_gu = (float*)p->acc_gu; a.h = (_Float16*)p->h; a.part_d = (float*)p->acc_d; a.out = (float*)p->out;
+    a.part_gu = (float*)p->acc_gu; a.h = (_Float16*)p->h; a.part_d = (float*)p->acc_d; a.out = p->out;
     a.force_level = p->force_level; a.hits = p->hits; a.cnt_gu = p->cnt_gu; a.cnt_d = p->cnt_d;
     return launch_moe(a, p->cfg_gu, p->cfg_dn, p->which, (hipStream_t)stream);
 }

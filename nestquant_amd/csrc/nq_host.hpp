@@ -23,9 +23,10 @@ inline int set_error(const char* fmt, ...)
 // arguments of one decode-path layer call (device pointers; see NqMoeArgs in include/nq_moe_hip.h)
 struct MoeArgs
 {
-    const _Float16* x; const int64_t* sel; const _Float16* rw; int B, topk;
+    const void* x; const void* sel; const void* rw; int B, topk;
+    int x_dtype, sel_dtype, rw_dtype, out_dtype;   // NQ_DT_*: x / rw f16, bf16 or f32; sel i64 or i32; out f32, f16 or bf16
     const int64_t* table; int E, H, I;
-    float* part_gu; _Float16* h; float* part_d; float* out;
+    float* part_gu; _Float16* h; float* part_d; void* out;
     int force_level; int* hits;
     int* cnt_gu; int* cnt_d;          // arrival counters [S * I/128] and [H/128]: zero on entry, zero on exit
 };

@@ -67,6 +67,45 @@ __device__ __forceinline__ void sum_partials(const float* const* p, size_t strid
     }
 }
 
+// ---- caller dtypes: the casts a caller would otherwise launch as separate kernels (x.half(), ids.long(), w.half(),
+// out.to(x.dtype); reference sm120/serve/nq_vllm.py:522,560,573) happen at the loads and the final store, with the same
+// roundings: activations and routing weights pass through fp16, the fp32 result is rounded once to the output type.
+constexpr int DT_DEFAULT = 0, DT_BF16 = 1, DT_F32 = 2, DT_I32 = 1, DT_OUT_F16 = 1, DT_OUT_BF16 = 2;
+__device__ __forceinline__ float bf16_to_f(uint16_t v) { return __builtin_bit_cast(float, (uint32_t)v << 16); }
+__device__ __forceinline__ uint16_t f_to_bf16(float f)           // round to nearest even; NaN stays NaN
+{
+    uint32_t u = __builtin_bit_cast(uint32_t, f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+__device__ __forceinline__ long long sel_at(const MoeArgs& a, int i)
+{
+    return a.sel_dtype == DT_I32 ? (long long)((const int32_t*)a.sel)[i] : (long long)((const int64_t*)a.sel)[i];
+}
+__device__ __forceinline__ float rw_at(const MoeArgs& a, int i)   // the weight as fp16 would hold it
+{
+    if (a.rw_dtype == DT_BF16) return (float)(_Float16)bf16_to_f(((const uint16_t*)a.rw)[i]);
+    if (a.rw_dtype == DT_F32) return (float)(_Float16)((const float*)a.rw)[i];
+    return (float)((const _Float16*)a.rw)[i];
+}
+__device__ __forceinline__ half2_t x2_at(const MoeArgs& a, size_t i)   // x[i], x[i + 1] (i even) as fp16
+{
+    if (a.x_dtype == DT_BF16)
+    {
+        const uint32_t v = *(const uint32_t*)((const uint16_t*)a.x + i);
+        return half2_t{(_Float16)bf16_to_f((uint16_t)v), (_Float16)bf16_to_f((uint16_t)(v >> 16))};
+    }
+    if (a.x_dtype == DT_F32) { const float2 v = *(const float2*)((const float*)a.x + i); return half2_t{(_Float16)v.x, (_Float16)v.y}; }
+    return *(const half2_t*)((const _Float16*)a.x + i);
+}
+__device__ __forceinline__ void out2_store(const MoeArgs& a, size_t i, float v0, float v1)   // out[i], out[i + 1] (i even)
+{
+    if (a.out_dtype == DT_OUT_F16) { half2_t h; h.x = (_Float16)v0; h.y = (_Float16)v1; *(half2_t*)((_Float16*)a.out + i) = h; }
+    else if (a.out_dtype == DT_OUT_BF16) *(uint32_t*)((uint16_t*)a.out + i) = (uint32_t)f_to_bf16(v0) | ((uint32_t)f_to_bf16(v1) << 16);
+    else *(float2*)((float*)a.out + i) = make_float2(v0, v1);
+}
+
 constexpr int MAXTOK = 8;                      // tokens of one run = tokens of one call (the MFMA N dimension holds 16)
 struct RunInfo
 {
@@ -90,7 +129,7 @@ __device__ __forceinline__ void route(const MoeArgs& a, int z, RunInfo* R, int l
     int64_t f_base = 0, f_res = 0, f_dw = 0, f_var = 0, f_code = 0, f_signs = 0;
     if (lane < S)
     {
-        const long long ee = a.sel[lane];
+        const long long ee = sel_at(a, lane);
         if (ee >= 0 && ee < a.E)
         {
             e = (int)ee;
@@ -98,7 +137,7 @@ __device__ __forceinline__ void route(const MoeArgs& a, int z, RunInfo* R, int l
             constexpr int o = MODE == 0 ? 1 : 5;
             lv = (int)ent[0];
             f_base = ent[o]; f_res = ent[o + 1]; f_dw = ent[o + 2]; f_var = ent[MODE == 0 ? 12 : 13]; f_code = ent[10 + MODE]; f_signs = ent[9];
-            ok = (float)a.rw[lane] != 0.f && lv > 0;
+            ok = rw_at(a, lane) != 0.f && lv > 0;
         }
     }
     unsigned long long rem = __ballot(ok);
@@ -127,7 +166,7 @@ __device__ __forceinline__ void route(const MoeArgs& a, int z, RunInfo* R, int l
         }
         rem &= ~m; ++r;
     }
-    R->pick_w[lane] = ok ? (float)a.rw[lane] : 0.f; R->pick_signs[lane] = (const _Float16*)f_signs;
+    R->pick_w[lane] = ok ? rw_at(a, lane) : 0.f; R->pick_signs[lane] = (const _Float16*)f_signs;
     if (lane == 0) R->nruns = r;
 }
 
@@ -192,7 +231,7 @@ __device__ __forceinline__ void finish_dn(const MoeArgs& a, const RunInfo& R, in
         {
             float r0 = 0.f, r1 = 0.f;
             for (int w2 = 0; w2 < SB; ++w2) { r0 += red[w2 * 128 + 2 * lane]; r1 += red[w2 * 128 + 2 * lane + 1]; }
-            *(float2*)(a.out + (size_t)b * a.H + col) = make_float2(r0, r1);
+            out2_store(a, (size_t)b * a.H + col, r0, r1);
         }
         __syncthreads();
     }
@@ -217,8 +256,8 @@ __global__ void __launch_bounds__(256) nq_gemv_k(MoeArgs a, int NC)
     if (warp == 0) route<MODE>(a, blockIdx.z, &R, lane);
     if (MODE == 0 && a.hits && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x < a.B * a.topk)
     {
-        const long long ee = a.sel[threadIdx.x];
-        if ((float)a.rw[threadIdx.x] != 0.f && ee >= 0 && ee < a.E)
+        const long long ee = sel_at(a, threadIdx.x);
+        if (rw_at(a, threadIdx.x) != 0.f && ee >= 0 && ee < a.E)
             __hip_atomic_fetch_add(a.hits + ee, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     }
     __syncthreads();
@@ -226,8 +265,8 @@ __global__ void __launch_bounds__(256) nq_gemv_k(MoeArgs a, int NC)
     const int N = MODE == 0 ? 2 * a.I : a.H, K = MODE == 0 ? a.H : a.I, C = K / 128, NY = C / NC;
     if (MODE == 1 && nruns == 0 && blockIdx.z == 0 && blockIdx.y == 0)
     {   // no active pick at all: nobody will arrive last, so the first plane of blocks writes the zero output
-        for (int i = threadIdx.x; i < a.B * SB * 32; i += blockDim.x)
-            a.out[(size_t)(i / (SB * 32)) * a.H + blockIdx.x * SB * 32 + i % (SB * 32)] = 0.f;
+        for (int i = threadIdx.x; i < a.B * SB * 16; i += blockDim.x)
+            out2_store(a, (size_t)(i / (SB * 16)) * a.H + blockIdx.x * SB * 32 + 2 * (i % (SB * 16)), 0.f, 0.f);
     }
     if ((int)blockIdx.z >= nruns) return;                        // block-uniform
     const int ntok = R.ntok, chunk0 = blockIdx.y * NC, k0 = chunk0 * 128;
@@ -266,7 +305,7 @@ __global__ void __launch_bounds__(256) nq_gemv_k(MoeArgs a, int NC)
                 const int task = t0 + u * SB < ntask ? t0 + u * SB : t0;
                 const int j = task / NC, c = task - j * NC, kk = k0 + c * 128 + 2 * lane;
                 const int tok = R.slot[j] / a.topk;
-                xv[u] = *(const half2_t*)(a.x + (size_t)tok * a.H + kk); sv[u] = *(const half2_t*)(su + kk);
+                xv[u] = x2_at(a, (size_t)tok * a.H + kk); sv[u] = *(const half2_t*)(su + kk);
                 dsto[u] = j * rowstride + c * 256;
             }
 #pragma unroll

@@ -106,6 +106,12 @@ def dense_W(ex, proj, level, dtype=torch.float16):
     return dequant(row, proj, ex.H, ex.I).to(dtype)
 
 
+# caller element types the decode kernels read / write directly (codes of include/nq_moe_hip.h)
+_DT_IN = {torch.float16: 0, torch.bfloat16: 1, torch.float32: 2}
+_DT_SEL = {torch.int64: 0, torch.int32: 1}
+_DT_OUT = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+
+
 class MoELayer:
     """Device table [E, TBL_W] + workspaces for up to Bmax tokens; table rows are flipped in place (graph-safe).
 
@@ -163,12 +169,16 @@ class MoELayer:
         s.table[e].copy_(row.to(s.table.device), non_blocking=False)
 
     def __call__(s, x, sel, rw, out=None, force_level=0, which=3, cfg_gu=None, cfg_dn=None, table=None):
-        """x fp16 [B, H], sel int64 [B, topk], rw fp16 [B, topk] -> fp32 [B, H] (s.out[:B] unless `out` is given).
+        """x [B, H], sel [B, topk], rw [B, topk] -> fp32 [B, H] (s.out[:B] unless `out` is given). As in the reference x
+        and rw are fp16 and sel int64; the kernels also take x / rw in bf16 or fp32, sel in int32 and `out` in fp16 or
+        bf16, with the roundings of x.half(), rw.half() and out.to(dtype) (the casts the reference's caller launches as
+        separate kernels, sm120/serve/nq_vllm.py:522,560).
         table: optional [E, TBL_W] override. Everything is enqueued on torch's current stream; nothing syncs."""
-        assert x.dtype == torch.float16 and rw.dtype == torch.float16 and sel.dtype == torch.int64, (x.dtype, rw.dtype, sel.dtype)
+        assert x.dtype in _DT_IN and rw.dtype in _DT_IN and sel.dtype in _DT_SEL, (x.dtype, rw.dtype, sel.dtype)
         assert x.is_contiguous() and sel.is_contiguous() and rw.is_contiguous()
         B, topk = sel.shape
         out = s.out[:B] if out is None else out
+        assert out.dtype in _DT_OUT and out.is_contiguous(), out.dtype
         tb = s.table if table is None else table
         cg, cd = list(cfg_gu or s.cfg_gu), list(cfg_dn or s.cfg_dn)
         s._alloc_partials(cg, cd)                    # grows only when a call brings a finer k-split than any before
@@ -181,6 +191,7 @@ class MoELayer:
         a.B, a.topk, a.E, a.H, a.I = B, topk, tb.shape[0], x.shape[1], s.I
         a.cfg_gu = (C.c_int32 * 4)(*(cg + [0] * (4 - len(cg)))); a.cfg_dn = (C.c_int32 * 4)(*(cd + [0] * (4 - len(cd))))
         a.force_level, a.which = force_level, which
+        a.x_dtype, a.sel_dtype, a.rw_dtype, a.out_dtype = _DT_IN[x.dtype], _DT_SEL[sel.dtype], _DT_IN[rw.dtype], _DT_OUT[out.dtype]
         _lib.check(s.M.nq_moe_forward(C.byref(a), _lib.stream_ptr()))
         return out
 
@@ -308,6 +319,30 @@ class Mailbox:
 
 
 MoELayer.prefill = prefill
+
+
+PF_MIN = 384         # tokens from which a step goes through prefill() (reference NQ_PF_MIN, sm120/serve/nq_vllm.py:187)
+
+
+def forward(layer, mailbox, x, topk_weights, topk_ids, pf_min=PF_MIN):
+    """One MoE layer step as the reference's serving caller runs it (sm120/serve/nq_vllm.py:520-574): apply the mailbox,
+    then up to Bmax tokens in one decode call, pf_min tokens or more through prefill() (never under graph capture), anything
+    between in slices of Bmax tokens. x [T, H] in fp16 / bf16 / fp32, weights [T, topk] likewise, ids int64 / int32;
+    returns [T, H] in x's dtype. The decode calls read the caller's dtypes and write the result dtype themselves."""
+    T = x.shape[0]
+    x, w, ids = x.contiguous(), topk_weights.contiguous(), topk_ids.contiguous()
+    if mailbox is not None:
+        mailbox.apply()
+    odt = x.dtype if x.dtype in _DT_OUT else torch.float32
+    if T <= layer.Bmax:
+        return layer(x, ids, w, out=torch.empty(T, layer.H, dtype=odt, device=x.device))
+    if T >= pf_min and not torch.cuda.is_current_stream_capturing():
+        return layer.prefill(x.half(), ids.long(), w.half()).to(x.dtype)
+    out = torch.empty(T, layer.H, dtype=odt, device=x.device)
+    for i in range(0, T, layer.Bmax):
+        j = min(T, i + layer.Bmax)
+        layer(x[i:j], ids[i:j], w[i:j], out=out[i:j])
+    return out
 
 
 def proj_gemv(layer, x, e=0, cfg=None):

@@ -190,7 +190,7 @@ def test_argument_errors():
         L(torch.zeros(9, 256, dtype=torch.float16, device=DEV), torch.zeros(9, 4, dtype=torch.int64, device=DEV),
           torch.zeros(9, 4, dtype=torch.float16, device=DEV), out=torch.zeros(9, 256, device=DEV))
     with pytest.raises(AssertionError):
-        L(x.float(), sel, rw)
+        L(x.double(), sel, rw)                                   # fp16 / bf16 / fp32 activations only
     L.out.fill_(7.0)
     y = L(x, sel, rw)                                            # all weights zero -> zeros, no fault
     torch.cuda.synchronize()
@@ -210,3 +210,46 @@ def test_mailbox_kernel_matches_state_machine():
     assert n == 2
     assert np.array_equal(L.table.cpu().numpy(), t) and np.array_equal(MB.applied.cpu().numpy(), a)
     assert MB.applied_host.numpy()[[1, 4]].tolist() == [1, 5]
+
+
+def test_caller_dtypes_and_forward_dispatch():
+    """bf16 / fp32 activations and weights, int32 ids, fp16 / bf16 results: bitwise what the reference's caller gets from
+    x.half(), w.half(), ids.long() and out.to(dtype) around an fp16 call; forward() slices 9..383 tokens by Bmax"""
+    H, I, NE = 512, 256, 12
+    ex = to_dev(experts_on_gpu(H, I, NE, 900, nested_ids=(1, 5)))
+    L = M.MoELayer(NE, H, I, Bmax=8, topk=4)
+    for e in range(NE):
+        L.set(e, ex[e], 4 if ex[e].nested else 2)
+    MB = M.Mailbox(L)
+    g = torch.Generator().manual_seed(5)
+    for T in (1, 5, 8):
+        sel = torch.stack([torch.randperm(NE, generator=g)[:4] for _ in range(T)]).to(DEV)
+        rw32 = (torch.rand(T, 4, generator=g) + 0.05).to(DEV)
+        x32 = (torch.randn(T, H, generator=g) * 0.3).to(DEV)
+        for xd in (torch.float16, torch.bfloat16, torch.float32):
+            for wd in (torch.float16, torch.bfloat16, torch.float32):
+                x, w = x32.to(xd), rw32.to(wd)
+                want32 = L(x.half(), sel, w.half()).clone()
+                for sd in (torch.int64, torch.int32):
+                    for od in (torch.float32, torch.float16, torch.bfloat16):
+                        out = torch.full((T, H), float("nan"), dtype=od, device=DEV)
+                        L(x, sel.to(sd), w, out=out)
+                        assert torch.equal(out, want32.to(od)), (T, xd, wd, sd, od)
+    # inactive call writes zeros in the output dtype
+    out = torch.full((2, H), 7.0, dtype=torch.bfloat16, device=DEV)
+    L(x32[:2].bfloat16(), sel[:2], torch.zeros(2, 4, dtype=torch.float16, device=DEV), out=out)
+    assert not out.any()
+    # dispatcher: 21 tokens = slices of 8, 8, 5; the same rows as three direct calls; result in x's dtype
+    T = 21
+    sel = torch.stack([torch.randperm(NE, generator=g)[:4] for _ in range(T)]).to(DEV).int()
+    w = (torch.rand(T, 4, generator=g) + 0.05).to(DEV)
+    x = (torch.randn(T, H, generator=g) * 0.3).to(DEV).bfloat16()
+    y = M.forward(L, MB, x, w, sel)
+    assert y.dtype == torch.bfloat16 and y.shape == (T, H)
+    for i in range(0, T, 8):
+        j = min(T, i + 8)
+        assert torch.equal(y[i:j], L(x[i:j].half(), sel[i:j].long(), w[i:j].half()).to(torch.bfloat16))
+    # at pf_min tokens or more the step goes through prefill(): same math, other summation order
+    yp = M.forward(L, MB, x, w, sel, pf_min=16)
+    assert yp.dtype == torch.bfloat16
+    assert rel_err(yp.float().cpu().numpy(), y.float().cpu().numpy()) < 2e-2     # two bf16 roundings of nearly equal fp32 results
