@@ -83,6 +83,9 @@ typedef struct NqMoeArgs
     int32_t sel_dtype;        /* NQ_DT_I64 (0) or NQ_DT_I32 */
     int32_t rw_dtype;         /* NQ_DT_F16 (0), NQ_DT_BF16, NQ_DT_F32 */
     int32_t out_dtype;        /* NQ_DT_OUT_F32 (0), NQ_DT_OUT_F16, NQ_DT_OUT_BF16: element type of out */
+    int32_t* cnt_h;           /* int32 [B*topk * I/128], zero on entry and on exit: arrival counters of the 512-column blocks
+                                 of experts with in_had_down = 512 (reference cnt_h, sm120/nqmoe.cu:860) */
+    int64_t cnt_h_elems;
 } NqMoeArgs;
 int nq_moe_forward(const NqMoeArgs* args, void* stream);
 

@@ -37,7 +37,7 @@ extern "C" int nq_validate_row(const int64_t* r, int H, int I)
     NQ_REQUIRE(r[1] && r[5] && r[9], "table row: null base plane or sign vector");
     NQ_REQUIRE(r[4] == 0 && r[8] == 0, "table row: mask mode (flags) is not implemented");
     NQ_REQUIRE(r[14] == 0 && r[15] == 0 && r[16] == 0 && r[17] == 0, "table row: low-rank plane is not implemented");
-    NQ_REQUIRE(r[18] == 0 || r[18] == 128, "table row: in_had_down %lld is not implemented (128 only)", (long long)r[18]);
+    NQ_REQUIRE(r[18] == 0 || r[18] == 128 || (r[18] == 512 && I % 512 == 0), "table row: in_had_down %lld must be 0, 128, or 512 dividing I = %d", (long long)r[18], I);
     NQ_REQUIRE(r[19] == 0, "table row: base code %lld is not implemented (K=2 ring base only)", (long long)r[19]);
     if (lv >= 3)
     {
@@ -105,6 +105,8 @@ extern "C" int nq_moe_forward(const NqMoeArgs* p, void* stream)
     a.table = p->table; a.E = p->E; a.H = p->H; a.I = p->I;
     a.part_gu = (float*)p->acc_gu; a.h = (_Float16*)p->h; a.part_d = (float*)p->acc_d; a.out = p->out;
     a.force_level = p->force_level; a.hits = p->hits; a.cnt_gu = p->cnt_gu; a.cnt_d = p->cnt_d;
+    NQ_REQUIRE(p->cnt_h && p->cnt_h_elems >= S * (p->I / 128), "workspace too small: cnt_h");
+    a.cnt_h = p->cnt_h;
     return launch_moe(a, p->cfg_gu, p->cfg_dn, p->which, (hipStream_t)stream);
 }
 

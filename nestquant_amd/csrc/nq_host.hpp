@@ -29,6 +29,7 @@ struct MoeArgs
     float* part_gu; _Float16* h; float* part_d; void* out;
     int force_level; int* hits;
     int* cnt_gu; int* cnt_d;          // arrival counters [S * I/128] and [H/128]: zero on entry, zero on exit
+    int* cnt_h;                       // arrival counters of the 512-column blocks (in_had_down = 512) [S * I/128]; may be null
 };
 
 // kernel launchers defined next to their kernels

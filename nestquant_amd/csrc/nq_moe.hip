@@ -34,6 +34,10 @@ __device__ __forceinline__ void st_dev4(float* p, float4_t v)
 {
     asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" :: "v"(p), "v"(v) : "memory");
 }
+__device__ __forceinline__ void st_dev2(float* p, float2 v)
+{
+    asm volatile("global_store_dwordx2 %0, %1, off sc0 sc1" :: "v"(p), "v"(v) : "memory");
+}
 __device__ __forceinline__ float2 ld_dev2_issue(const float* p)
 {
     float2 v;
@@ -112,6 +116,7 @@ struct RunInfo
     Planes P;                     // this launch's projection of the run's expert
     const _Float16* signs;        // su_g | sv_g | sv_u | su_d | sv_o | su_u
     int level, ntok, nruns;
+    int had;                      // width of the Hadamard on the down projection's input: 128 or 512
     int slot[MAXTOK];
     float pick_w[64];             // routing weight of every pick, 0 for picks that contribute nothing
     const _Float16* pick_signs[64];
@@ -126,7 +131,7 @@ __device__ __forceinline__ void route(const MoeArgs& a, int z, RunInfo* R, int l
 {
     const int S = a.B * a.topk;
     int e = -1, lv = 0; bool ok = false;
-    int64_t f_base = 0, f_res = 0, f_dw = 0, f_var = 0, f_code = 0, f_signs = 0;
+    int64_t f_base = 0, f_res = 0, f_dw = 0, f_var = 0, f_code = 0, f_signs = 0, f_had = 0;
     if (lane < S)
     {
         const long long ee = sel_at(a, lane);
@@ -136,7 +141,7 @@ __device__ __forceinline__ void route(const MoeArgs& a, int z, RunInfo* R, int l
             const int64_t* ent = a.table + (size_t)e * TBL_W;
             constexpr int o = MODE == 0 ? 1 : 5;
             lv = (int)ent[0];
-            f_base = ent[o]; f_res = ent[o + 1]; f_dw = ent[o + 2]; f_var = ent[MODE == 0 ? 12 : 13]; f_code = ent[10 + MODE]; f_signs = ent[9];
+            f_base = ent[o]; f_res = ent[o + 1]; f_dw = ent[o + 2]; f_var = ent[MODE == 0 ? 12 : 13]; f_code = ent[10 + MODE]; f_signs = ent[9]; f_had = ent[18];
             ok = rw_at(a, lane) != 0.f && lv > 0;
         }
     }
@@ -161,6 +166,7 @@ __device__ __forceinline__ void route(const MoeArgs& a, int z, RunInfo* R, int l
                 P.base = (gp_u4)f_base; P.res = (gp_u8)f_res; P.dw = (gp_u32)f_dw; P.var = (gp_u8)f_var; P.code = (int)f_code;
                 R->P = P; R->signs = (const _Float16*)f_signs;
                 R->level = a.force_level ? a.force_level : lv;
+                R->had = f_had == 512 ? 512 : 128;
                 R->ntok = __popcll(m);
             }
         }
@@ -170,11 +176,16 @@ __device__ __forceinline__ void route(const MoeArgs& a, int z, RunInfo* R, int l
     if (lane == 0) R->nruns = r;
 }
 
-// finisher of gate|up for (run, 128-column group grp): h[slot] = fp16(WHT(silu(g) * u * su_d)), g = WHT(sum_y part_g) * sv_g
-__device__ __forceinline__ void finish_gu(const MoeArgs& a, const RunInfo& R, int grp, int NY, int warp, int SB, int lane)
+// finisher of gate|up for (run z, 128-column group grp): h[slot] = fp16(WHT(silu(g) * u * su_d)), g = WHT(sum_y part_g) * sv_g.
+// With a 512-wide Hadamard on the down projection's input (in_had_down, reference sm120/nqmoe.cu:36-40,673-712;
+// WHT_512 = H_4 (x) WHT_128 / 2) the group's WHT_128 result goes, in fp32, into the gate columns of k-slice 0 that this
+// finisher has just consumed, and the last of the four groups of a 512-column block combines them with the Sylvester H_4
+// and rounds to fp16 once.
+__device__ __forceinline__ void finish_gu(const MoeArgs& a, const RunInfo& R, int z, int grp, int NY, int warp, int SB, int lane, int& last)
 {
     const _Float16 *sv_g = R.signs + a.H, *sv_u = sv_g + a.I, *su_d = sv_u + a.I;
     const int S = a.B * a.topk, col = grp * 128 + 2 * lane;
+    const bool wide = R.had == 512;
     for (int j = warp; j < R.ntok; j += SB)
     {
         const int s = R.slot[j];
@@ -188,9 +199,43 @@ __device__ __forceinline__ void finish_gu(const MoeArgs& a, const RunInfo& R, in
         g0 *= (float)svg.x; g1 *= (float)svg.y; u0 *= (float)svu.x; u1 *= (float)svu.y;
         float v0 = g0 / (1.f + __expf(-g0)) * u0 * (float)sud.x, v1 = g1 / (1.f + __expf(-g1)) * u1 * (float)sud.y;
         wht128(v0, v1, lane);
-        half2_t hv; hv.x = (_Float16)v0; hv.y = (_Float16)v1;
-        *(half2_t*)(a.h + (size_t)s * a.I + col) = hv;           // read by the next kernel on the stream
+        if (wide) st_dev2(a.part_gu + (size_t)s * 2 * a.I + col, make_float2(v0, v1));
+        else
+        {
+            half2_t hv; hv.x = (_Float16)v0; hv.y = (_Float16)v1;
+            *(half2_t*)(a.h + (size_t)s * a.I + col) = hv;       // read by the next kernel on the stream
+        }
     }
+    if (!wide) return;                                           // block-uniform
+    int* cnt = a.cnt_h + z * (a.I / 128) + grp / 4;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0) last = __hip_atomic_fetch_add(cnt, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 3;
+    __syncthreads();
+    if (!last) return;
+    const int c0 = (grp / 4) * 512 + 2 * lane;
+    for (int j = warp; j < R.ntok; j += SB)
+    {
+        const int s = R.slot[j];
+        float2 w[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) w[q] = ld_dev2_issue(a.part_gu + (size_t)s * 2 * a.I + c0 + q * 128);
+        ld_wait(w[0], w[1], w[2], w[3]);
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+        {
+            float h0 = 0.f, h1 = 0.f;
+#pragma unroll
+            for (int pp = 0; pp < 4; ++pp)
+            {
+                const float sg = (__builtin_popcount(q & pp) & 1) ? -0.5f : 0.5f;
+                h0 += sg * w[pp].x; h1 += sg * w[pp].y;
+            }
+            half2_t hv; hv.x = (_Float16)h0; hv.y = (_Float16)h1;
+            *(half2_t*)(a.h + (size_t)s * a.I + c0 + q * 128) = hv;
+        }
+    }
+    if (threadIdx.x == 0) __hip_atomic_store(cnt, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // combine of the down projection for output rows [grp * 128, +128): out[b] = sum_k rw[b,k] * sv_o[e] (.) WHT(sum_y part_d[slot])
@@ -358,7 +403,7 @@ __global__ void __launch_bounds__(256) nq_gemv_k(MoeArgs a, int NC)
         last = __hip_atomic_fetch_add(cnt, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == expect - 1;
     __syncthreads();
     if (!last) return;                                           // block-uniform
-    if constexpr (MODE == 0) finish_gu(a, R, grp, NY, warp, SB, lane);
+    if constexpr (MODE == 0) finish_gu(a, R, blockIdx.z, grp, NY, warp, SB, lane, last);
     else finish_dn(a, R, grp, NY, warp, SB, lane, (float*)smem);
     if (threadIdx.x == 0) __hip_atomic_store(cnt, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }

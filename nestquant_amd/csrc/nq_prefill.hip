@@ -57,14 +57,18 @@ __global__ void __launch_bounds__(256) nq_pf_pre_k(const _Float16* __restrict__ 
     }
 }
 
-// grid (npairs), block 256: acc_gu [P][2I] fp32 (gate | up) -> h [P][I] fp16 in B-operand order
+// grid (npairs), block 256: acc_gu [P][2I] fp32 (gate | up) -> h [P][I] fp16 in B-operand order. With in_had_down = 512
+// (table word 18) the four wavefronts hold the four 128-column groups of a 512-column block and combine their WHT_128
+// results through LDS with the Sylvester H_4 / 2 before the single rounding to fp16.
 __global__ void __launch_bounds__(256) nq_pf_mid_k(const float* __restrict__ acc_gu, const int32_t* __restrict__ pe,
                                                     const int64_t* __restrict__ table, _Float16* h, int E, int H, int I)
 {
+    __shared__ float wsh[4][128];
     const int p = blockIdx.x, lane = threadIdx.x & 63, warp = threadIdx.x >> 6;
     const int e = pe[p];
     const bool live = e >= 0 && e < E && table[(size_t)e * TBL_W] > 0;
     const _Float16* signs = live ? (const _Float16*)table[(size_t)e * TBL_W + 9] : nullptr;
+    const bool wide = live && table[(size_t)e * TBL_W + 18] == 512;      // block-uniform
     for (int grp = warp; grp < I / 128; grp += 4)
     {
         const int col = grp * 128 + 2 * lane;
@@ -80,6 +84,19 @@ __global__ void __launch_bounds__(256) nq_pf_mid_k(const float* __restrict__ acc
             g0 *= (float)svg.x; g1 *= (float)svg.y; u0 *= (float)svu.x; u1 *= (float)svu.y;
             v0 = g0 / (1.f + __expf(-g0)) * u0 * (float)sud.x; v1 = g1 / (1.f + __expf(-g1)) * u1 * (float)sud.y;
             wht128(v0, v1, lane);
+        }
+        if (wide)
+        {   // I % 512 == 0, so all four wavefronts are in this iteration: grp = 4 * block + warp
+            wsh[warp][2 * lane] = v0; wsh[warp][2 * lane + 1] = v1;
+            __syncthreads();
+            v0 = v1 = 0.f;
+#pragma unroll
+            for (int pp = 0; pp < 4; ++pp)
+            {
+                const float sg = (__builtin_popcount(warp & pp) & 1) ? -0.5f : 0.5f;
+                v0 += sg * wsh[pp][2 * lane]; v1 += sg * wsh[pp][2 * lane + 1];
+            }
+            __syncthreads();
         }
         store_bop(dst, v0, v1, lane);
     }

@@ -191,6 +191,7 @@ class MoELayer:
         a.B, a.topk, a.E, a.H, a.I = B, topk, tb.shape[0], x.shape[1], s.I
         a.cfg_gu = (C.c_int32 * 4)(*(cg + [0] * (4 - len(cg)))); a.cfg_dn = (C.c_int32 * 4)(*(cd + [0] * (4 - len(cd))))
         a.force_level, a.which = force_level, which
+        a.cnt_h, a.cnt_h_elems = s.cnt_h.data_ptr(), s.cnt_h.numel()
         a.x_dtype, a.sel_dtype, a.rw_dtype, a.out_dtype = _DT_IN[x.dtype], _DT_SEL[sel.dtype], _DT_IN[rw.dtype], _DT_OUT[out.dtype]
         _lib.check(s.M.nq_moe_forward(C.byref(a), _lib.stream_ptr()))
         return out

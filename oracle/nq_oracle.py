@@ -333,28 +333,42 @@ def split_signs(signs, H, I):
     return {n: s[o[i]:o[i + 1]] for i, n in enumerate(names)}
 
 
-def expert_forward(x, Wgu, Wdn, signs, round_acts=True, dtype=np.float32):
-    """x [T,H] through dense weights Wgu [2I,H], Wdn [H,I] (arrays holding fp16 values) -> [T,H].
+def expert_forward(x, Wgu, Wdn, signs, round_acts=True, dtype=np.float32, had_dn=128, lr=None, level=4):
+    """x [T,H] through dense weights Wgu [2I,H], Wdn [H,I] (arrays holding fp16 values) -> [T,H]
+    (reference sm120/moe.py:196-210).
     round_acts: round the two rotated activations to fp16 as the kernels do (False = no activation rounding).
-    dtype: arithmetic type; float64 gives the exact-arithmetic arbiter used to separate rounding noise from errors."""
+    dtype: arithmetic type; float64 gives the exact-arithmetic arbiter used to separate rounding noise from errors.
+    had_dn: width of the Hadamard on the down projection's input (128, or 512 = in_had_down).
+    lr: low-rank plane, dict of fp16-valued arrays Vg [rg,H], U2g/U2u/U4g/U4u [rg,I], Vd [rd,I], U2d/U4d [rd,H]; the U4
+    terms count at level 4 only."""
     H, I = Wdn.shape
     sg = {k: v.astype(dtype) for k, v in split_signs(signs, H, I).items()}
     rnd = (lambda a: a.astype(np.float16).astype(dtype)) if round_acts else (lambda a: a)
     x = np.asarray(x, dtype)
     Wgu = np.asarray(Wgu, dtype); Wdn = np.asarray(Wdn, dtype)
-    wht_ = lambda v: wht(v, 128, dtype)
+    wht_ = lambda v, n=128: wht(v, n, dtype)
     xg = rnd(wht_(x * sg["su_g"])); xu = rnd(wht_(x * sg["su_u"]))
     g = wht_(xg @ Wgu[:I].T) * sg["sv_g"]
     u = wht_(xu @ Wgu[I:].T) * sg["sv_u"]
+    if lr is not None:
+        L = {k: np.asarray(v, dtype) for k, v in lr.items()}
+        z = x @ L["Vg"].T
+        g = g + z @ L["U2g"] + (z @ L["U4g"] if level == 4 else 0)
+        u = u + z @ L["U2u"] + (z @ L["U4u"] if level == 4 else 0)
     with np.errstate(over="ignore"):                       # exp overflow gives the correct limit silu(-inf) = -0
         sw = g / (1.0 + np.exp(-g)) * u
-    h = rnd(wht_(sw * sg["su_d"]))
-    return wht_(h @ Wdn.T) * sg["sv_o"]
+    h = rnd(wht_(sw * sg["su_d"], had_dn))
+    y = wht_(h @ Wdn.T) * sg["sv_o"]
+    if lr is not None:
+        z = sw @ L["Vd"].T
+        y = y + z @ L["U2d"] + (z @ L["U4d"] if level == 4 else 0)
+    return y
 
 
-def moe_forward(dense, levels, signs, x, sel, rw, round_acts=True, dtype=np.float32):
+def moe_forward(dense, levels, signs, x, sel, rw, round_acts=True, dtype=np.float32, had_dn=128, lr=None):
     """dense: callable e -> (Wgu fp32 [2I,H], Wdn fp32 [H,I]) at the expert's level; levels [E]; signs: e -> vector.
-    x [B,H] fp16/fp32, sel [B,topk] int, rw [B,topk] fp16 -> [B,H] fp32. Picks with rw == 0 or level <= 0 add 0."""
+    x [B,H] fp16/fp32, sel [B,topk] int, rw [B,topk] fp16 -> [B,H] fp32. Picks with rw == 0 or level <= 0 add 0.
+    had_dn: down-input Hadamard width of every expert; lr: optional callable e -> low-rank dict (or None)."""
     x = np.asarray(x, dtype)
     out = np.zeros_like(x)
     cache = {}
@@ -366,7 +380,8 @@ def moe_forward(dense, levels, signs, x, sel, rw, round_acts=True, dtype=np.floa
             if e not in cache:
                 cache[e] = dense(e)
             Wgu, Wdn = cache[e]
-            out[b] += dtype(w) * expert_forward(x[b:b + 1], Wgu, Wdn, signs(e), round_acts, dtype)[0]
+            out[b] += dtype(w) * expert_forward(x[b:b + 1], Wgu, Wdn, signs(e), round_acts, dtype, had_dn,
+                                                None if lr is None else lr(e), levels[e])[0]
     return out
 
 

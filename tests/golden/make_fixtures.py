@@ -93,6 +93,34 @@ def main():
         packs[f"w{c}"] = w.numpy().astype(np.uint32)
         packs[f"p{c}"] = R.pack_words(w, b).numpy()
     np.savez_compressed(os.path.join(OUT, "pack_words.npz"), **packs)
+    # 5. optional layer features of the reference's Expert.ref: Hadamard-512 on the down projection's input (in_had_down)
+    #    and the low-rank plane (set_lr); H = 256, I = 512, 3 experts at levels 2 / 4 / 4
+    H, I = 256, 512
+    ex = [R.Expert(H, I, seed=700 + i, dev="cpu", rk_gu=(0, 7, 0)[i], rk_dn=(0, 0, 3)[i]) for i in range(3)]
+    levels = [2, 4, 4]
+    g = torch.Generator().manual_seed(11)
+    x = (torch.randn(2, H, generator=g) * 0.05).half()
+    sel = torch.tensor([[0, 1, 2], [2, 1, 0]])
+    rw = (torch.rand(2, 3, generator=g) + 0.1)
+    rw = (rw / rw.sum(1, keepdim=True)).half()
+    out = dict(H=H, I=I, seeds=np.arange(700, 703), levels=np.array(levels), rk_gu=np.array([0, 7, 0]), rk_dn=np.array([0, 0, 3]),
+               x=x.numpy().view(np.uint16), sel=sel.numpy(), rw=rw.numpy().view(np.uint16))
+    for e in ex:
+        e.had_dn = 512
+    out["y_had512"] = R.moe_ref(ex, levels, x, sel, rw).numpy()
+    rg, rd = 2, 3
+    names = ("Vg", "U2g", "U2u", "U4g", "U4u", "Vd", "U2d", "U4d")
+    shapes = ((rg, H), (rg, I), (rg, I), (rg, I), (rg, I), (rd, I), (rd, H), (rd, H))
+    for i, e in enumerate(ex):
+        t = [(torch.randn(*sh, generator=g) * (0.5 if n[0] == "V" else 0.02)).half() for n, sh in zip(names, shapes)]
+        e.set_lr(*t)
+        for n, v in zip(names, t):
+            out[f"lr{i}_{n}"] = v.numpy().view(np.uint16)
+    out["y_had512_lr"] = R.moe_ref(ex, levels, x, sel, rw).numpy()
+    for e in ex:
+        e.had_dn = 128
+    out["y_lr"] = R.moe_ref(ex, levels, x, sel, rw).numpy()
+    np.savez_compressed(os.path.join(OUT, "layer_had512_lr.npz"), **out)
     print("fixtures written to", OUT)
 
 

@@ -253,3 +253,39 @@ def test_caller_dtypes_and_forward_dispatch():
     yp = M.forward(L, MB, x, w, sel, pf_min=16)
     assert yp.dtype == torch.bfloat16
     assert rel_err(yp.float().cpu().numpy(), y.float().cpu().numpy()) < 2e-2     # two bf16 roundings of nearly equal fp32 results
+
+
+def _optional_feature_layer(golden_dir, had, with_lr):
+    """layer of the optional-feature fixture (H 256, I 512, 3 experts at levels 2 / 4 / 4) on the GPU"""
+    from tests.test_oracle_golden import LR_NAMES
+    z = np.load(f"{golden_dir}/layer_had512_lr.npz")
+    H, I = int(z["H"]), int(z["I"])
+    ex = to_dev([F.Expert(H, I, seed=int(z["seeds"][i]), dev="cpu", rk_gu=int(z["rk_gu"][i]), rk_dn=int(z["rk_dn"][i])) for i in range(3)])
+    for i, e in enumerate(ex):
+        e.had_dn = had
+        if with_lr:
+            e.set_lr(*[torch.from_numpy(z[f"lr{i}_{n}"].view(np.float16).copy()) for n in LR_NAMES])
+    L = M.MoELayer(3, H, I, Bmax=2, topk=3)
+    for e in range(3):
+        L.set(e, ex[e], int(z["levels"][e]))
+    x = torch.from_numpy(z["x"].view(np.float16).copy()).to(DEV)
+    sel = torch.from_numpy(z["sel"]).to(DEV); rw = torch.from_numpy(z["rw"].view(np.float16).copy()).to(DEV)
+    return z, L, ex, x, sel, rw
+
+
+def test_in_had_down_512_decode_and_prefill(golden_dir):
+    """Hadamard-512 on the down projection's input against the reference's own moe_ref output; every k-split; counters clean"""
+    z, L, ex, x, sel, rw = _optional_feature_layer(golden_dir, 512, False)
+    want = z["y_had512"]
+    for cg, cd in (([1, 4, 2], [1, 4, 4]), ([1, 4, 1], [1, 4, 1]), ([1, 2, 2], [1, 1, 2])):
+        y = L(x, sel, rw, cfg_gu=cg, cfg_dn=cd).clone()
+        torch.cuda.synchronize()
+        assert rel_err(y.cpu().numpy(), want) < 1e-4, (cg, cd)
+        assert torch.equal(y, L(x, sel, rw, cfg_gu=cg, cfg_dn=cd))
+        assert not L.cnt_h.any() and not L.cnt_gu.any() and not L.cnt_d.any()
+    assert rel_err(L.prefill(x, sel, rw).cpu().numpy(), want) < 1e-4
+    assert rel_err(want, z["y_lr"]) > 1e-2                        # a 128-wide rotation would be far off
+    # 512 must divide I
+    bad = F.Expert(256, 384, seed=1, dev="cpu"); bad.had_dn = 512
+    with pytest.raises(RuntimeError, match="in_had_down"):
+        M.validate_row(M.entry(to_dev([bad])[0], 2), 256, 384)

@@ -109,3 +109,43 @@ def test_expert_and_layer_math_match_reference():
     # distance to the pipeline without the two fp16 activation roundings stays inside the 1e-3 budget
     y_pure = O.moe_forward(dense, levels, lambda e: ex[e].signs.numpy(), x, sel, rw, round_acts=False)
     assert 0 < rel_err(y, y_pure) < 1e-3
+
+
+LR_NAMES = ("Vg", "U2g", "U2u", "U4g", "U4u", "Vd", "U2d", "U4d")
+
+
+def had512_lr_layer():
+    """the optional-feature fixture: experts rebuilt from their seeds, low-rank tensors and expected outputs as stored"""
+    z = np.load(os.path.join(GOLD, "layer_had512_lr.npz"))
+    H, I = int(z["H"]), int(z["I"])
+    ex = [F.Expert(H, I, seed=int(z["seeds"][i]), dev="cpu", rk_gu=int(z["rk_gu"][i]), rk_dn=int(z["rk_dn"][i])) for i in range(3)]
+    lr = [{n: z[f"lr{i}_{n}"].view(np.float16) for n in LR_NAMES} for i in range(3)]
+    return z, H, I, ex, lr
+
+
+def test_had512_and_low_rank_plane_match_reference():
+    """in_had_down = 512 and the low-rank plane (reference Expert.ref, sm120/moe.py:196-210), alone and together"""
+    z, H, I, ex, lr = had512_lr_layer()
+    levels = z["levels"].tolist()
+    x = z["x"].view(np.float16); rw = z["rw"].view(np.float16); sel = z["sel"]
+
+    def dense(e):
+        return (O.dense_W(oracle_plane(ex[e].gu), levels[e]).astype(np.float32),
+                O.dense_W(oracle_plane(ex[e].dn), levels[e]).astype(np.float32))
+
+    sg = lambda e: ex[e].signs.numpy()
+    y_h = O.moe_forward(dense, levels, sg, x, sel, rw, had_dn=512)
+    y_hl = O.moe_forward(dense, levels, sg, x, sel, rw, had_dn=512, lr=lambda e: lr[e])
+    y_l = O.moe_forward(dense, levels, sg, x, sel, rw, lr=lambda e: lr[e])
+    assert rel_err(y_h, z["y_had512"]) < 1e-4
+    assert rel_err(y_hl, z["y_had512_lr"]) < 1e-4
+    assert rel_err(y_l, z["y_lr"]) < 1e-4
+    # the three variants and the plain layer are far apart, so a dropped term or a wrong width fails the bars above
+    y_0 = O.moe_forward(dense, levels, sg, x, sel, rw)
+    for a, b in ((y_h, y_0), (y_l, y_0), (y_hl, y_h), (y_hl, y_l)):
+        assert rel_err(a, b) > 1e-2
+    # U4 terms count at level 4 only: expert 0 is at level 2
+    lr_no4 = [dict(d) for d in lr]
+    for n in ("U4g", "U4u", "U4d"):
+        lr_no4[0][n] = np.zeros_like(lr[0][n])
+    assert np.array_equal(O.moe_forward(dense, levels, sg, x, sel, rw, lr=lambda e: lr_no4[e]), y_l)
