@@ -86,6 +86,9 @@ typedef struct NqMoeArgs
     int32_t* cnt_h;           /* int32 [B*topk * I/128], zero on entry and on exit: arrival counters of the 512-column blocks
                                  of experts with in_had_down = 512 (reference cnt_h, sm120/nqmoe.cu:860) */
     int64_t cnt_h_elems;
+    void* zd;                 /* fp32 [B*topk * I/128 * 4]: low-rank plane, z_d partials written by the gate|up launch and read by the
+                                 down launch (reference zd, sm120/nqmoe.cu:860); needs no zeroing */
+    int64_t zd_elems;
 } NqMoeArgs;
 int nq_moe_forward(const NqMoeArgs* args, void* stream);
 
@@ -99,9 +102,10 @@ int nq_mailbox(int64_t* table, const int64_t* stage, const int32_t* seq, int32_t
  * outside [0, E), or whose weight is 0 contribute nothing. Activation buffers xg, xu [np][H] and h [np][I] are fp16 with
  * every 128-column chunk stored in the MFMA B-operand column order (an internal layout shared by these entry points). */
 
-/* xg / xu = fp16(Hadamard-128(x[pt] * su_g / su_u)). Replaces pf_pre (reference sm120/nqmoe.cu:1082-1117,1258-1267). */
+/* xg / xu = fp16(Hadamard-128(x[pt] * su_g / su_u)); zg fp32 [np][4] (may be NULL when no expert has a low-rank plane):
+ * zg[p] = x[pt[p]] V_gu^T of pair p's expert. Replaces pf_pre (reference sm120/nqmoe.cu:1082-1117,1258-1267). */
 int nq_pf_pre(const void* x_f16, const int32_t* pt, const int32_t* pe, int np, const int64_t* table, void* xg_f16,
-              void* xu_f16, int E, int H, int I, void* stream);
+              void* xu_f16, float* zg, int E, int H, int I, void* stream);
 
 /* Grouped GEMM with the weights decoded from the trellis planes inside the kernel (level and planes from the live table
  * row): for every tile t = tiles[t] = {expert, first pair row, rows, 0} (device int32[ntiles][4], rows <= bm,
@@ -112,18 +116,20 @@ int nq_pf_pre(const void* x_f16, const int32_t* pt, const int32_t* pe, int np, c
 int nq_pf_gemm(const int64_t* table, const int32_t* tiles, int ntiles, int bm, int mode, const void* A0_f16,
                const void* A1_f16, float* C, int E, int H, int I, void* stream);
 
-/* h = fp16(Hadamard(silu(g) * u * su_d)), g = Hadamard(acc_gu[:, :I]) * sv_g, u = Hadamard(acc_gu[:, I:]) * sv_u.
- * Replaces pf_mid (reference sm120/nqmoe.cu:1119-1203,1268-1277). */
-int nq_pf_mid(const float* acc_gu, const int32_t* pe, int np, const int64_t* table, void* h_f16, int E, int H, int I,
-              void* stream);
+/* h = fp16(Hadamard(silu(g) * u * su_d)), g = Hadamard(acc_gu[:, :I]) * sv_g, u = Hadamard(acc_gu[:, I:]) * sv_u; the last
+ * Hadamard is 128 or 512 wide (table word 18). Low-rank plane: g / u += zg (U2 [+ U4 at level 4]) and zd[p] = (silu(g) * u)
+ * V_dn^T, fp32 [np][4] (zg, zd may be NULL). Replaces pf_mid (reference sm120/nqmoe.cu:1119-1203,1268-1277). */
+int nq_pf_mid(const float* acc_gu, const int32_t* pe, int np, const int64_t* table, void* h_f16, const float* zg, float* zd,
+              int E, int H, int I, void* stream);
 
 /* For every token t < T: out[t] += sum over its picks k whose pair row pos[t][k] lies in [row_lo, row_lo + nrows) of
  * rw[t][k] * sv_o (.) Hadamard(y[pos[t][k] - row_lo]). pos int32 [T][topk] = row of pair (t, k) in the expert-sorted
  * order; sel int64 [T][topk]; rw fp16 [T][topk]; y fp32 [nrows][H]; out fp32 [T][H], zeroed by the caller before the
- * first row chunk. Gathered per token: no atomics, fixed summation order. Replaces pf_post (reference
- * sm120/nqmoe.cu:1205-1240,1278-1287, which adds with float atomics). */
+ * first row chunk; zd fp32 [nrows][4] from nq_pf_mid adds the low-rank term zd (U2_d [+ U4_d]) per pick (may be NULL).
+ * Gathered per token: no atomics, fixed summation order. Replaces pf_post (reference sm120/nqmoe.cu:1205-1240,1278-1287,
+ * which adds with float atomics). */
 int nq_pf_post(const float* y, const int32_t* pos, const int64_t* sel, const void* rw_f16, int T, int topk, int row_lo,
-               int nrows, const int64_t* table, float* out, int E, int H, int I, void* stream);
+               int nrows, const int64_t* table, float* out, const float* zd, int E, int H, int I, void* stream);
 
 /* hits[e] += counts[e] (hits may be host-mapped). Replaces pf_hits (reference sm120/nqmoe.cu:1241-1245,1288-1293). */
 int nq_pf_hits(const int32_t* counts, int32_t* hits, int E, void* stream);

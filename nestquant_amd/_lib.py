@@ -21,7 +21,7 @@ class NqMoeArgs(C.Structure):
                 ("B", C.c_int32), ("topk", C.c_int32), ("E", C.c_int32), ("H", C.c_int32), ("I", C.c_int32),
                 ("cfg_gu", C.c_int32 * 4), ("cfg_dn", C.c_int32 * 4), ("force_level", C.c_int32), ("which", C.c_int32),
                 ("x_dtype", C.c_int32), ("sel_dtype", C.c_int32), ("rw_dtype", C.c_int32), ("out_dtype", C.c_int32),
-                ("cnt_h", C.c_void_p), ("cnt_h_elems", C.c_int64)]
+                ("cnt_h", C.c_void_p), ("cnt_h_elems", C.c_int64), ("zd", C.c_void_p), ("zd_elems", C.c_int64)]
 
 
 # name -> (restype, argtypes); every symbol declared in include/nq_moe_hip.h
@@ -34,10 +34,10 @@ SIGNATURES = {
     "nq_pf_decode": (C.c_int, [_i64p, _i32p, _i, _vp, _vp, _i, _i, _vp]),
     "nq_moe_forward": (C.c_int, [C.POINTER(NqMoeArgs), _vp]),
     "nq_mailbox": (C.c_int, [_i64p, _i64p, _i32p, _i32p, _i32p, _i, _vp]),
-    "nq_pf_pre": (C.c_int, [_vp, _i32p, _i32p, _i, _i64p, _vp, _vp, _i, _i, _i, _vp]),
+    "nq_pf_pre": (C.c_int, [_vp, _i32p, _i32p, _i, _i64p, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "nq_pf_gemm": (C.c_int, [_i64p, _i32p, _i, _i, _i, _vp, _vp, _vp, _i, _i, _i, _vp]),
-    "nq_pf_mid": (C.c_int, [_vp, _i32p, _i, _i64p, _vp, _i, _i, _i, _vp]),
-    "nq_pf_post": (C.c_int, [_vp, _i32p, _i64p, _vp, _i, _i, _i, _i, _i64p, _vp, _i, _i, _i, _vp]),
+    "nq_pf_mid": (C.c_int, [_vp, _i32p, _i, _i64p, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "nq_pf_post": (C.c_int, [_vp, _i32p, _i64p, _vp, _i, _i, _i, _i, _i64p, _vp, _vp, _i, _i, _i, _vp]),
     "nq_pf_hits": (C.c_int, [_i32p, _i32p, _i, _vp]),
 }
 

@@ -36,7 +36,8 @@ extern "C" int nq_validate_row(const int64_t* r, int H, int I)
     if (lv == 0) return 0;
     NQ_REQUIRE(r[1] && r[5] && r[9], "table row: null base plane or sign vector");
     NQ_REQUIRE(r[4] == 0 && r[8] == 0, "table row: mask mode (flags) is not implemented");
-    NQ_REQUIRE(r[14] == 0 && r[15] == 0 && r[16] == 0 && r[17] == 0, "table row: low-rank plane is not implemented");
+    NQ_REQUIRE(r[14] ? (r[15] != 0 && r[16] >= 0 && r[16] <= 4 && r[17] >= 0 && r[17] <= 4 && r[16] + r[17] > 0) : (r[15] == 0 && r[16] == 0 && r[17] == 0),
+               "table row: low-rank plane needs both buffers and ranks r_gu, r_dn in [0, 4] (got %lld, %lld)", (long long)r[16], (long long)r[17]);
     NQ_REQUIRE(r[18] == 0 || r[18] == 128 || (r[18] == 512 && I % 512 == 0), "table row: in_had_down %lld must be 0, 128, or 512 dividing I = %d", (long long)r[18], I);
     NQ_REQUIRE(r[19] == 0, "table row: base code %lld is not implemented (K=2 ring base only)", (long long)r[19]);
     if (lv >= 3)
@@ -107,6 +108,8 @@ extern "C" int nq_moe_forward(const NqMoeArgs* p, void* stream)
     a.force_level = p->force_level; a.hits = p->hits; a.cnt_gu = p->cnt_gu; a.cnt_d = p->cnt_d;
     NQ_REQUIRE(p->cnt_h && p->cnt_h_elems >= S * (p->I / 128), "workspace too small: cnt_h");
     a.cnt_h = p->cnt_h;
+    NQ_REQUIRE(p->zd && p->zd_elems >= S * (p->I / 128) * 4, "workspace too small: zd");
+    a.zd = (float*)p->zd;
     return launch_moe(a, p->cfg_gu, p->cfg_dn, p->which, (hipStream_t)stream);
 }
 
@@ -118,13 +121,13 @@ extern "C" int nq_mailbox(int64_t* table, const int64_t* stage, const int32_t* s
 }
 
 extern "C" int nq_pf_pre(const void* x, const int32_t* pt, const int32_t* pe, int np, const int64_t* table, void* xg, void* xu,
-                         int E, int H, int I, void* stream)
+                         float* zg, int E, int H, int I, void* stream)
 {
     NQ_REQUIRE(np >= 0, "nq_pf_pre: np=%d", np);
     if (np == 0) return 0;
     NQ_REQUIRE(x && pt && pe && table && xg && xu, "nq_pf_pre: null pointer");
     NQ_REQUIRE(E >= 1 && shape_ok(H, I), "nq_pf_pre: E=%d H=%d I=%d (H, I positive multiples of 128)", E, H, I);
-    return launch_pf_pre(x, pt, pe, np, table, xg, xu, E, H, I, (hipStream_t)stream);
+    return launch_pf_pre(x, pt, pe, np, table, xg, xu, zg, E, H, I, (hipStream_t)stream);
 }
 
 extern "C" int nq_pf_gemm(const int64_t* table, const int32_t* tiles, int ntiles, int bm, int mode, const void* A0, const void* A1,
@@ -140,23 +143,24 @@ extern "C" int nq_pf_gemm(const int64_t* table, const int32_t* tiles, int ntiles
     return launch_pf_gemm(table, tiles, ntiles, bm, mode, A0, A1, C, E, H, I, (hipStream_t)stream);
 }
 
-extern "C" int nq_pf_mid(const float* acc_gu, const int32_t* pe, int np, const int64_t* table, void* h, int E, int H, int I, void* stream)
+extern "C" int nq_pf_mid(const float* acc_gu, const int32_t* pe, int np, const int64_t* table, void* h, const float* zg, float* zd,
+                         int E, int H, int I, void* stream)
 {
     NQ_REQUIRE(np >= 0, "nq_pf_mid: np=%d", np);
     if (np == 0) return 0;
     NQ_REQUIRE(acc_gu && pe && table && h, "nq_pf_mid: null pointer");
     NQ_REQUIRE(E >= 1 && shape_ok(H, I), "nq_pf_mid: E=%d H=%d I=%d (H, I positive multiples of 128)", E, H, I);
-    return launch_pf_mid(acc_gu, pe, np, table, h, E, H, I, (hipStream_t)stream);
+    return launch_pf_mid(acc_gu, pe, np, table, h, zg, zd, E, H, I, (hipStream_t)stream);
 }
 
 extern "C" int nq_pf_post(const float* y, const int32_t* pos, const int64_t* sel, const void* rw, int T, int topk, int row_lo, int nrows,
-                          const int64_t* table, float* out, int E, int H, int I, void* stream)
+                          const int64_t* table, float* out, const float* zd, int E, int H, int I, void* stream)
 {
     NQ_REQUIRE(T >= 0 && nrows >= 0 && topk >= 1 && topk <= 64 && row_lo >= 0, "nq_pf_post: T=%d topk=%d (<= 64) row_lo=%d nrows=%d", T, topk, row_lo, nrows);
     if (T == 0 || nrows == 0) return 0;
     NQ_REQUIRE(y && pos && sel && rw && table && out, "nq_pf_post: null pointer");
     NQ_REQUIRE(E >= 1 && shape_ok(H, I), "nq_pf_post: E=%d H=%d I=%d (H, I positive multiples of 128)", E, H, I);
-    return launch_pf_post(y, pos, sel, rw, T, topk, row_lo, nrows, table, out, E, H, I, (hipStream_t)stream);
+    return launch_pf_post(y, pos, sel, rw, T, topk, row_lo, nrows, table, out, zd, E, H, I, (hipStream_t)stream);
 }
 
 extern "C" int nq_pf_hits(const int32_t* counts, int32_t* hits, int E, void* stream)

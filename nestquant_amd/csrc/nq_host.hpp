@@ -29,6 +29,7 @@ struct MoeArgs
     float* part_gu; _Float16* h; float* part_d; void* out;
     int force_level; int* hits;
     int* cnt_gu; int* cnt_d;          // arrival counters [S * I/128] and [H/128]: zero on entry, zero on exit
+    float* zd;                        // low-rank plane: z_d partials [S][I/128][4], written by gate|up, read by down; may be null
     int* cnt_h;                       // arrival counters of the 512-column blocks (in_had_down = 512) [S * I/128]; may be null
 };
 
@@ -37,10 +38,10 @@ int launch_moe(const MoeArgs& a, const int* cfg_gu, const int* cfg_dn, int which
 int launch_mailbox(int64_t* table, const int64_t* stage, const int32_t* seq, int32_t* applied, int32_t* applied_host, int E, hipStream_t st);
 int launch_dequant(const int64_t* row, int proj, int level, int H, int I, void* out, hipStream_t st);
 int launch_pf_decode(const int64_t* table, const int32_t* experts, int G, void* Wgu, void* Wdn, int H, int I, hipStream_t st);
-int launch_pf_pre(const void* x, const int32_t* pt, const int32_t* pe, int np, const int64_t* table, void* xg, void* xu, int E, int H, int I, hipStream_t st);
-int launch_pf_mid(const float* acc_gu, const int32_t* pe, int np, const int64_t* table, void* h, int E, int H, int I, hipStream_t st);
+int launch_pf_pre(const void* x, const int32_t* pt, const int32_t* pe, int np, const int64_t* table, void* xg, void* xu, float* zg, int E, int H, int I, hipStream_t st);
+int launch_pf_mid(const float* acc_gu, const int32_t* pe, int np, const int64_t* table, void* h, const float* zg, float* zd, int E, int H, int I, hipStream_t st);
 int launch_pf_post(const float* y, const int32_t* pos, const int64_t* sel, const void* rw, int T, int topk, int row_lo, int nrows,
-                   const int64_t* table, float* out, int E, int H, int I, hipStream_t st);
+                   const int64_t* table, float* out, const float* zd, int E, int H, int I, hipStream_t st);
 int launch_pf_hits(const int32_t* counts, int32_t* hits, int E, hipStream_t st);
 int launch_pf_gemm(const int64_t* table, const int32_t* tiles, int ntiles, int bm, int mode, const void* A0, const void* A1, float* C,
                    int E, int H, int I, hipStream_t st);

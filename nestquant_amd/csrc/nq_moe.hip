@@ -117,9 +117,12 @@ struct RunInfo
     const _Float16* signs;        // su_g | sv_g | sv_u | su_d | sv_o | su_u
     int level, ntok, nruns;
     int had;                      // width of the Hadamard on the down projection's input: 128 or 512
+    const _Float16* lr; const _Float16* lr4; int rg, rd;      // low-rank plane of the run's expert (lr == nullptr: none)
+    float z[MAXTOK][4];           // gate|up finisher: x V_gu^T of the run's tokens
     int slot[MAXTOK];
     float pick_w[64];             // routing weight of every pick, 0 for picks that contribute nothing
     const _Float16* pick_signs[64];
+    const _Float16* pick_lr[64]; const _Float16* pick_lr4[64]; unsigned char pick_rg[64], pick_rd[64], pick_lv[64];
 };
 
 // ---- routing dedup: picks -> runs, numbered by first occurrence; slots in pick order ---------------------------------
@@ -131,7 +134,7 @@ __device__ __forceinline__ void route(const MoeArgs& a, int z, RunInfo* R, int l
 {
     const int S = a.B * a.topk;
     int e = -1, lv = 0; bool ok = false;
-    int64_t f_base = 0, f_res = 0, f_dw = 0, f_var = 0, f_code = 0, f_signs = 0, f_had = 0;
+    int64_t f_base = 0, f_res = 0, f_dw = 0, f_var = 0, f_code = 0, f_signs = 0, f_had = 0, f_lr = 0, f_lr4 = 0, f_rg = 0, f_rd = 0;
     if (lane < S)
     {
         const long long ee = sel_at(a, lane);
@@ -142,6 +145,7 @@ __device__ __forceinline__ void route(const MoeArgs& a, int z, RunInfo* R, int l
             constexpr int o = MODE == 0 ? 1 : 5;
             lv = (int)ent[0];
             f_base = ent[o]; f_res = ent[o + 1]; f_dw = ent[o + 2]; f_var = ent[MODE == 0 ? 12 : 13]; f_code = ent[10 + MODE]; f_signs = ent[9]; f_had = ent[18];
+            f_lr = ent[14]; f_lr4 = ent[15]; f_rg = ent[16]; f_rd = ent[17];
             ok = rw_at(a, lane) != 0.f && lv > 0;
         }
     }
@@ -167,12 +171,15 @@ __device__ __forceinline__ void route(const MoeArgs& a, int z, RunInfo* R, int l
                 R->P = P; R->signs = (const _Float16*)f_signs;
                 R->level = a.force_level ? a.force_level : lv;
                 R->had = f_had == 512 ? 512 : 128;
+                R->lr = (const _Float16*)f_lr; R->lr4 = (const _Float16*)f_lr4; R->rg = (int)f_rg; R->rd = (int)f_rd;
                 R->ntok = __popcll(m);
             }
         }
         rem &= ~m; ++r;
     }
     R->pick_w[lane] = ok ? rw_at(a, lane) : 0.f; R->pick_signs[lane] = (const _Float16*)f_signs;
+    R->pick_lr[lane] = (const _Float16*)f_lr; R->pick_lr4[lane] = (const _Float16*)f_lr4;
+    R->pick_rg[lane] = (unsigned char)f_rg; R->pick_rd[lane] = (unsigned char)f_rd; R->pick_lv[lane] = (unsigned char)(a.force_level ? a.force_level : lv);
     if (lane == 0) R->nruns = r;
 }
 
@@ -181,11 +188,40 @@ __device__ __forceinline__ void route(const MoeArgs& a, int z, RunInfo* R, int l
 // WHT_512 = H_4 (x) WHT_128 / 2) the group's WHT_128 result goes, in fp32, into the gate columns of k-slice 0 that this
 // finisher has just consumed, and the last of the four groups of a 512-column block combines them with the Sylvester H_4
 // and rounds to fp16 once.
-__device__ __forceinline__ void finish_gu(const MoeArgs& a, const RunInfo& R, int z, int grp, int NY, int warp, int SB, int lane, int& last)
+__device__ __forceinline__ void finish_gu(const MoeArgs& a, RunInfo& R, int z, int grp, int NY, int warp, int SB, int lane, int& last)
 {
     const _Float16 *sv_g = R.signs + a.H, *sv_u = sv_g + a.I, *su_d = sv_u + a.I;
     const int S = a.B * a.topk, col = grp * 128 + 2 * lane;
     const bool wide = R.had == 512;
+    // low-rank plane (reference sm120/nqmoe.cu:41-45,611-645): lr = V_gu [rg][H] | U2_g [rg][I] | U2_u [rg][I] | V_dn [rd][I] |
+    // U2_d [rd][H], lr4 = U4_g | U4_u | U4_d (level 4 only). z = x V_gu^T over the raw activations, one wavefront per token
+    const bool lowrank = R.lr != nullptr;                        // block-uniform
+    const int rg = lowrank ? R.rg : 0, rd = lowrank ? R.rd : 0;
+    if (rg)
+    {
+        for (int j = warp; j < R.ntok; j += SB)
+        {
+            const int tok = R.slot[j] / a.topk;
+            float zz[4] = {0.f, 0.f, 0.f, 0.f};
+            for (int k = 2 * lane; k < a.H; k += 128)
+            {
+                const half2_t xv = x2_at(a, (size_t)tok * a.H + k);
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (r < rg) { const half2_t vv = *(const half2_t*)(R.lr + (size_t)r * a.H + k); zz[r] += (float)xv.x * (float)vv.x + (float)xv.y * (float)vv.y; }
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+            {
+#pragma unroll
+                for (int m = 32; m >= 1; m >>= 1) zz[r] += __shfl_xor(zz[r], m);
+                if (lane == 0) R.z[j][r] = zz[r];
+            }
+        }
+        __syncthreads();
+    }
+    const _Float16* U2g = R.lr + (size_t)rg * a.H, *U2u = U2g + (size_t)rg * a.I, *Vd = U2u + (size_t)rg * a.I;
+    const _Float16* U4g = R.lr4, *U4u = U4g + (size_t)rg * a.I;
     for (int j = warp; j < R.ntok; j += SB)
     {
         const int s = R.slot[j];
@@ -197,7 +233,33 @@ __device__ __forceinline__ void finish_gu(const MoeArgs& a, const RunInfo& R, in
         float g0 = pq[0].x, g1 = pq[0].y, u0 = pq[1].x, u1 = pq[1].y;
         wht128(g0, g1, lane); wht128(u0, u1, lane);
         g0 *= (float)svg.x; g1 *= (float)svg.y; u0 *= (float)svu.x; u1 *= (float)svu.y;
-        float v0 = g0 / (1.f + __expf(-g0)) * u0 * (float)sud.x, v1 = g1 / (1.f + __expf(-g1)) * u1 * (float)sud.y;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            if (r < rg)
+            {
+                const float zr = R.z[j][r];
+                half2_t ug = *(const half2_t*)(U2g + (size_t)r * a.I + col), uu = *(const half2_t*)(U2u + (size_t)r * a.I + col);
+                g0 += zr * (float)ug.x; g1 += zr * (float)ug.y; u0 += zr * (float)uu.x; u1 += zr * (float)uu.y;
+                if (R.level == 4)
+                {
+                    ug = *(const half2_t*)(U4g + (size_t)r * a.I + col); uu = *(const half2_t*)(U4u + (size_t)r * a.I + col);
+                    g0 += zr * (float)ug.x; g1 += zr * (float)ug.y; u0 += zr * (float)uu.x; u1 += zr * (float)uu.y;
+                }
+            }
+        const float sw0 = g0 / (1.f + __expf(-g0)) * u0, sw1 = g1 / (1.f + __expf(-g1)) * u1;
+        if (rd)
+        {   // this group's share of z_d = sw V_dn^T, summed over the groups by the down combine
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+            {
+                float t = 0.f;
+                if (r < rd) { const half2_t vv = *(const half2_t*)(Vd + (size_t)r * a.I + col); t = sw0 * (float)vv.x + sw1 * (float)vv.y; }
+#pragma unroll
+                for (int m = 32; m >= 1; m >>= 1) t += __shfl_xor(t, m);
+                if (lane == 0) a.zd[((size_t)s * (a.I / 128) + grp) * 4 + r] = t;
+            }
+        }
+        float v0 = sw0 * (float)sud.x, v1 = sw1 * (float)sud.y;
         wht128(v0, v1, lane);
         if (wide) st_dev2(a.part_gu + (size_t)s * 2 * a.I + col, make_float2(v0, v1));
         else
@@ -267,7 +329,26 @@ __device__ __forceinline__ void finish_dn(const MoeArgs& a, const RunInfo& R, in
             {
                 float v0 = pv[q].x, v1 = pv[q].y;
                 wht128(v0, v1, lane);
-                if (w[q] != 0.f) { o0 += w[q] * (v0 * (float)sv[q].x); o1 += w[q] * (v1 * (float)sv[q].y); }
+                if (w[q] == 0.f) continue;
+                v0 *= (float)sv[q].x; v1 *= (float)sv[q].y;
+                const int s = b * a.topk + k + q * SB, prd = R.pick_lr[s] ? R.pick_rd[s] : 0;
+                if (prd)
+                {   // y += (sw V_dn^T) (U2_d [+ U4_d]): z_d summed over the I / 128 groups written by the gate|up finishers
+                    const int prg = R.pick_rg[s];
+                    const _Float16* U2d = R.pick_lr[s] + (size_t)prg * (a.H + 2 * a.I) + (size_t)prd * a.I;
+                    const _Float16* U4d = R.pick_lr4[s] + (size_t)prg * 2 * a.I;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        if (r < prd)
+                        {
+                            float zr = 0.f;
+                            for (int gq = 0; gq < a.I / 128; ++gq) zr += a.zd[((size_t)s * (a.I / 128) + gq) * 4 + r];
+                            half2_t ud = *(const half2_t*)(U2d + (size_t)r * a.H + col);
+                            v0 += zr * (float)ud.x; v1 += zr * (float)ud.y;
+                            if (R.pick_lv[s] == 4) { ud = *(const half2_t*)(U4d + (size_t)r * a.H + col); v0 += zr * (float)ud.x; v1 += zr * (float)ud.y; }
+                        }
+                }
+                o0 += w[q] * v0; o1 += w[q] * v1;
             }
         }
         red[warp * 128 + 2 * lane] = o0; red[warp * 128 + 2 * lane + 1] = o1;

@@ -33,14 +33,38 @@ __device__ __forceinline__ void store_bop(_Float16* dst, float v0, float v1, int
 
 // grid (npairs), block 256: wave w handles 128-column groups w, w + 4, ... of gate then up
 __global__ void __launch_bounds__(256) nq_pf_pre_k(const _Float16* __restrict__ x, const int32_t* __restrict__ pt, const int32_t* __restrict__ pe,
-                                                    const int64_t* __restrict__ table, _Float16* xg, _Float16* xu, int E, int H, int I)
+                                                    const int64_t* __restrict__ table, _Float16* xg, _Float16* xu, float* zg, int E, int H, int I)
 {
+    __shared__ float zsh[4][4];
     const int p = blockIdx.x, lane = threadIdx.x & 63, warp = threadIdx.x >> 6;
     const int e = pe[p];
     const int ng = H / 128;
     const bool live = e >= 0 && e < E && table[(size_t)e * TBL_W] > 0;
     const _Float16* signs = live ? (const _Float16*)table[(size_t)e * TBL_W + 9] : nullptr;
     const _Float16* xr = x + (size_t)pt[p] * H;
+    // low-rank plane (table words 14, 16): zg[p] = x V_gu^T over the raw activations, for the mid kernel
+    const _Float16* lr = live ? (const _Float16*)table[(size_t)e * TBL_W + 14] : nullptr;
+    const int rg = lr ? (int)table[(size_t)e * TBL_W + 16] : 0;
+    if (zg && rg)                                                // block-uniform
+    {
+        float zz[4] = {0.f, 0.f, 0.f, 0.f};
+        for (int k = 2 * threadIdx.x; k < H; k += 512)
+        {
+            const half2_t xv = *(const half2_t*)(xr + k);
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (r < rg) { const half2_t vv = *(const half2_t*)(lr + (size_t)r * H + k); zz[r] += (float)xv.x * (float)vv.x + (float)xv.y * (float)vv.y; }
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+        {
+#pragma unroll
+            for (int m = 32; m >= 1; m >>= 1) zz[r] += __shfl_xor(zz[r], m);
+            if (lane == 0) zsh[warp][r] = zz[r];
+        }
+        __syncthreads();
+        if (threadIdx.x < 4) zg[(size_t)p * 4 + threadIdx.x] = zsh[0][threadIdx.x] + zsh[1][threadIdx.x] + zsh[2][threadIdx.x] + zsh[3][threadIdx.x];
+    }
     for (int task = warp; task < 2 * ng; task += 4)
     {
         const int up = task / ng, grp = task % ng, k = grp * 128 + 2 * lane;
@@ -61,14 +85,23 @@ __global__ void __launch_bounds__(256) nq_pf_pre_k(const _Float16* __restrict__ 
 // (table word 18) the four wavefronts hold the four 128-column groups of a 512-column block and combine their WHT_128
 // results through LDS with the Sylvester H_4 / 2 before the single rounding to fp16.
 __global__ void __launch_bounds__(256) nq_pf_mid_k(const float* __restrict__ acc_gu, const int32_t* __restrict__ pe,
-                                                    const int64_t* __restrict__ table, _Float16* h, int E, int H, int I)
+                                                    const int64_t* __restrict__ table, _Float16* h, const float* zg, float* zd, int E, int H, int I)
 {
     __shared__ float wsh[4][128];
+    __shared__ float zsh[4][4];
     const int p = blockIdx.x, lane = threadIdx.x & 63, warp = threadIdx.x >> 6;
     const int e = pe[p];
     const bool live = e >= 0 && e < E && table[(size_t)e * TBL_W] > 0;
     const _Float16* signs = live ? (const _Float16*)table[(size_t)e * TBL_W + 9] : nullptr;
     const bool wide = live && table[(size_t)e * TBL_W + 18] == 512;      // block-uniform
+    // low-rank plane: g / u += zg (U2 [+ U4 at level 4]); zd[p] = sw V_dn^T for the post kernel
+    const _Float16* lr = live ? (const _Float16*)table[(size_t)e * TBL_W + 14] : nullptr;
+    const _Float16* lr4 = live ? (const _Float16*)table[(size_t)e * TBL_W + 15] : nullptr;
+    const int rg = lr && zg ? (int)table[(size_t)e * TBL_W + 16] : 0, rd = lr && zd ? (int)table[(size_t)e * TBL_W + 17] : 0;
+    const bool l4 = live && table[(size_t)e * TBL_W] == 4;
+    const _Float16* U2g = lr + (size_t)rg * H, *U2u = U2g + (size_t)rg * I, *Vd = U2u + (size_t)rg * I, *U4g = lr4, *U4u = lr4 + (size_t)rg * I;
+    float zr[4] = {0.f, 0.f, 0.f, 0.f}, zacc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int r = 0; r < rg; ++r) zr[r] = zg[(size_t)p * 4 + r];
     for (int grp = warp; grp < I / 128; grp += 4)
     {
         const int col = grp * 128 + 2 * lane;
@@ -82,7 +115,23 @@ __global__ void __launch_bounds__(256) nq_pf_mid_k(const float* __restrict__ acc
             wht128(g0, g1, lane); wht128(u0, u1, lane);
             const half2_t svg = *(const half2_t*)(sv_g + col), svu = *(const half2_t*)(sv_u + col), sud = *(const half2_t*)(su_d + col);
             g0 *= (float)svg.x; g1 *= (float)svg.y; u0 *= (float)svu.x; u1 *= (float)svu.y;
-            v0 = g0 / (1.f + __expf(-g0)) * u0 * (float)sud.x; v1 = g1 / (1.f + __expf(-g1)) * u1 * (float)sud.y;
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (r < rg)
+                {
+                    half2_t ug = *(const half2_t*)(U2g + (size_t)r * I + col), uu = *(const half2_t*)(U2u + (size_t)r * I + col);
+                    g0 += zr[r] * (float)ug.x; g1 += zr[r] * (float)ug.y; u0 += zr[r] * (float)uu.x; u1 += zr[r] * (float)uu.y;
+                    if (l4)
+                    {
+                        ug = *(const half2_t*)(U4g + (size_t)r * I + col); uu = *(const half2_t*)(U4u + (size_t)r * I + col);
+                        g0 += zr[r] * (float)ug.x; g1 += zr[r] * (float)ug.y; u0 += zr[r] * (float)uu.x; u1 += zr[r] * (float)uu.y;
+                    }
+                }
+            const float sw0 = g0 / (1.f + __expf(-g0)) * u0, sw1 = g1 / (1.f + __expf(-g1)) * u1;
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (r < rd) { const half2_t vv = *(const half2_t*)(Vd + (size_t)r * I + col); zacc[r] += sw0 * (float)vv.x + sw1 * (float)vv.y; }
+            v0 = sw0 * (float)sud.x; v1 = sw1 * (float)sud.y;
             wht128(v0, v1, lane);
         }
         if (wide)
@@ -100,6 +149,18 @@ __global__ void __launch_bounds__(256) nq_pf_mid_k(const float* __restrict__ acc
         }
         store_bop(dst, v0, v1, lane);
     }
+    if (rd)                                                      // block-uniform
+    {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+        {
+#pragma unroll
+            for (int m = 32; m >= 1; m >>= 1) zacc[r] += __shfl_xor(zacc[r], m);
+            if (lane == 0) zsh[warp][r] = zacc[r];
+        }
+        __syncthreads();
+        if (threadIdx.x < 4) zd[(size_t)p * 4 + threadIdx.x] = zsh[0][threadIdx.x] + zsh[1][threadIdx.x] + zsh[2][threadIdx.x] + zsh[3][threadIdx.x];
+    }
 }
 
 // grid (T), block 256: out[t] += sum over the token's picks whose pair row lies in [row_lo, row_lo + nrows) of
@@ -107,14 +168,15 @@ __global__ void __launch_bounds__(256) nq_pf_mid_k(const float* __restrict__ acc
 // the sum needs no atomics and its order is fixed (the reference's pf_post adds with float atomics in arrival order).
 __global__ void __launch_bounds__(256) nq_pf_post_k(const float* __restrict__ y, const int32_t* __restrict__ pos, const int64_t* __restrict__ sel,
                                                      const _Float16* __restrict__ rw, int topk, int row_lo, int nrows,
-                                                     const int64_t* __restrict__ table, float* out, int E, int H, int I)
+                                                     const int64_t* __restrict__ table, float* out, const float* zd, int E, int H, int I)
 {
     const int t = blockIdx.x, lane = threadIdx.x & 63, warp = threadIdx.x >> 6;
     // the token's live picks, gathered once: row, weight and sign vector (picks keep their order, so does the sum)
     __shared__ int p_row[64]; __shared__ float p_w[64]; __shared__ const _Float16* p_sv[64]; __shared__ int p_n;
+    __shared__ const _Float16* p_u2[64]; __shared__ const _Float16* p_u4[64]; __shared__ int p_rd[64];   // low-rank plane: U2_d, U4_d (level 4) and r_dn
     if (warp == 0)
     {
-        bool ok = false; int r = 0; float w = 0.f; const _Float16* sv = nullptr;
+        bool ok = false; int r = 0, rdn = 0; float w = 0.f; const _Float16* sv = nullptr; const _Float16* u2 = nullptr; const _Float16* u4 = nullptr;
         if (lane < topk)
         {
             r = pos[(size_t)t * topk + lane] - row_lo;
@@ -123,10 +185,18 @@ __global__ void __launch_bounds__(256) nq_pf_post_k(const float* __restrict__ y,
             if (r >= 0 && r < nrows && e >= 0 && e < E && w != 0.f && table[(size_t)e * TBL_W] > 0)
             {
                 ok = true; sv = (const _Float16*)table[(size_t)e * TBL_W + 9] + H + 3 * I;
+                const _Float16* lr = (const _Float16*)table[(size_t)e * TBL_W + 14];
+                if (lr && zd)
+                {
+                    const int rg = (int)table[(size_t)e * TBL_W + 16];
+                    rdn = (int)table[(size_t)e * TBL_W + 17];
+                    u2 = lr + (size_t)rg * (H + 2 * I) + (size_t)rdn * I;
+                    if (table[(size_t)e * TBL_W] == 4) u4 = (const _Float16*)table[(size_t)e * TBL_W + 15] + (size_t)rg * 2 * I;
+                }
             }
         }
         const unsigned long long m = __ballot(ok);
-        if (ok) { const int i = __popcll(m & ((1ull << lane) - 1ull)); p_row[i] = r; p_w[i] = w; p_sv[i] = sv; }
+        if (ok) { const int i = __popcll(m & ((1ull << lane) - 1ull)); p_row[i] = r; p_w[i] = w; p_sv[i] = sv; p_u2[i] = u2; p_u4[i] = u4; p_rd[i] = rdn; }
         if (lane == 0) p_n = __popcll(m);
     }
     __syncthreads();
@@ -153,7 +223,15 @@ __global__ void __launch_bounds__(256) nq_pf_post_k(const float* __restrict__ y,
                 float v0 = v[u].x, v1 = v[u].y;
                 wht128(v0, v1, lane);
                 const float w = p_w[k0 + u];
-                o0 += w * (v0 * (float)sv[u].x); o1 += w * (v1 * (float)sv[u].y);
+                v0 *= (float)sv[u].x; v1 *= (float)sv[u].y;
+                for (int r = 0; r < p_rd[k0 + u]; ++r)           // y += (sw V_dn^T) (U2_d [+ U4_d])
+                {
+                    const float zr = zd[(size_t)p_row[k0 + u] * 4 + r];
+                    half2_t ud = *(const half2_t*)(p_u2[k0 + u] + (size_t)r * H + col);
+                    v0 += zr * (float)ud.x; v1 += zr * (float)ud.y;
+                    if (p_u4[k0 + u]) { ud = *(const half2_t*)(p_u4[k0 + u] + (size_t)r * H + col); v0 += zr * (float)ud.x; v1 += zr * (float)ud.y; }
+                }
+                o0 += w * v0; o1 += w * v1;
             }
         }
         float2* op = (float2*)(out + (size_t)t * H + col);
@@ -333,25 +411,25 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) n
     }
 }
 
-int launch_pf_pre(const void* x, const int32_t* pt, const int32_t* pe, int np, const int64_t* table, void* xg, void* xu, int E, int H, int I, hipStream_t st)
+int launch_pf_pre(const void* x, const int32_t* pt, const int32_t* pe, int np, const int64_t* table, void* xg, void* xu, float* zg, int E, int H, int I, hipStream_t st)
 {
     if (!np) return 0;
-    nq_pf_pre_k<<<np, 256, 0, st>>>((const _Float16*)x, pt, pe, table, (_Float16*)xg, (_Float16*)xu, E, H, I);
+    nq_pf_pre_k<<<np, 256, 0, st>>>((const _Float16*)x, pt, pe, table, (_Float16*)xg, (_Float16*)xu, zg, E, H, I);
     NQ_LAUNCH_CHECK("nq_pf_pre");
     return 0;
 }
-int launch_pf_mid(const float* acc_gu, const int32_t* pe, int np, const int64_t* table, void* h, int E, int H, int I, hipStream_t st)
+int launch_pf_mid(const float* acc_gu, const int32_t* pe, int np, const int64_t* table, void* h, const float* zg, float* zd, int E, int H, int I, hipStream_t st)
 {
     if (!np) return 0;
-    nq_pf_mid_k<<<np, 256, 0, st>>>(acc_gu, pe, table, (_Float16*)h, E, H, I);
+    nq_pf_mid_k<<<np, 256, 0, st>>>(acc_gu, pe, table, (_Float16*)h, zg, zd, E, H, I);
     NQ_LAUNCH_CHECK("nq_pf_mid");
     return 0;
 }
 int launch_pf_post(const float* y, const int32_t* pos, const int64_t* sel, const void* rw, int T, int topk, int row_lo, int nrows,
-                   const int64_t* table, float* out, int E, int H, int I, hipStream_t st)
+                   const int64_t* table, float* out, const float* zd, int E, int H, int I, hipStream_t st)
 {
     if (!T || !nrows) return 0;
-    nq_pf_post_k<<<T, 256, 0, st>>>(y, pos, sel, (const _Float16*)rw, topk, row_lo, nrows, table, out, E, H, I);
+    nq_pf_post_k<<<T, 256, 0, st>>>(y, pos, sel, (const _Float16*)rw, topk, row_lo, nrows, table, out, zd, E, H, I);
     NQ_LAUNCH_CHECK("nq_pf_post");
     return 0;
 }

@@ -211,6 +211,18 @@ class Expert:
         if nested:                                       # slot image: [P3 | P4] per projection, contiguous
             s.gu.slot = s.gu.nested_plane(); s.dn.slot = s.dn.nested_plane()
 
+    def set_lr(s, Vg, U2g, U2u, U4g, U4u, Vd, U2d, U4d):
+        """low-rank plane (fp16; reference sm120/moe.py:184-189): Vg [rg, H], U2g / U2u / U4g / U4u [rg, I], Vd [rd, I],
+        U2d / U4d [rd, H] -> the two buffers of table words 14 / 15: lr = Vg | U2g | U2u | Vd | U2d, lr4 = U4g | U4u | U4d"""
+        f = lambda *t: torch.cat([x.reshape(-1) for x in t]).half().contiguous()
+        s.rg, s.rd = Vg.shape[0], Vd.shape[0]
+        s.lrT = (Vg, U2g, U2u, U4g, U4u, Vd, U2d, U4d)
+        if s.rg + s.rd == 0:
+            s.lr = s.lr4 = None
+            return s
+        s.lr = f(Vg, U2g, U2u, Vd, U2d).to(s.signs.device); s.lr4 = f(U4g, U4u, U4d).to(s.signs.device)
+        return s
+
     def compact(s):
         """drop everything a layer call does not read (unpacked words; for nested experts the wide plane and the separate
         P3 / P4 tensors, whose bytes live on in `slot`)"""

@@ -192,6 +192,7 @@ class MoELayer:
         a.cfg_gu = (C.c_int32 * 4)(*(cg + [0] * (4 - len(cg)))); a.cfg_dn = (C.c_int32 * 4)(*(cd + [0] * (4 - len(cd))))
         a.force_level, a.which = force_level, which
         a.cnt_h, a.cnt_h_elems = s.cnt_h.data_ptr(), s.cnt_h.numel()
+        a.zd, a.zd_elems = s.zd.data_ptr(), s.zd.numel()
         a.x_dtype, a.sel_dtype, a.rw_dtype, a.out_dtype = _DT_IN[x.dtype], _DT_SEL[sel.dtype], _DT_IN[rw.dtype], _DT_OUT[out.dtype]
         _lib.check(s.M.nq_moe_forward(C.byref(a), _lib.stream_ptr()))
         return out
@@ -203,7 +204,7 @@ PF_TILES = (16, 32, 64, 128, 256)            # token-tile heights the grouped GE
 
 def pf_bytes(H, I, R, G=0):
     """bytes of prefill scratch for R pair rows (G is accepted for signature compatibility: no decoded-weight scratch exists)"""
-    return R * (2 * H * 2 + 2 * I * 4 + I * 2 + H * 4)
+    return R * (2 * H * 2 + 2 * I * 4 + I * 2 + H * 4 + 32)
 
 
 def pf_scratch(dev, H, I, R, G=0):
@@ -215,7 +216,8 @@ def pf_scratch(dev, H, I, R, G=0):
         f16, f32 = torch.float16, torch.float32
         _PF[k] = dict(xg=torch.empty(R, H, dtype=f16, device=dev), xu=torch.empty(R, H, dtype=f16, device=dev),
                       acc=torch.empty(R, 2 * I, dtype=f32, device=dev), h=torch.empty(R, I, dtype=f16, device=dev),
-                      y=torch.empty(R, H, dtype=f32, device=dev))
+                      y=torch.empty(R, H, dtype=f32, device=dev),
+                      zg=torch.zeros(R, 4, dtype=f32, device=dev), zd=torch.zeros(R, 4, dtype=f32, device=dev))
     return _PF[k]
 
 
@@ -271,16 +273,17 @@ def prefill(s, x, sel, rw, out=None, R=None, G=None, table=None):
         tiles = {bm: t.pin_memory().to(dev, non_blocking=True) for bm, t in pf_tiles(segs).items()}
         pts, pes = pt[c:d], pe[c:d]
         _lib.check(Lb.nq_pf_pre(x.data_ptr(), pts.data_ptr(), pes.data_ptr(), n, tb.data_ptr(), S["xg"].data_ptr(),
-                                S["xu"].data_ptr(), E, H, I, st))
+                                S["xu"].data_ptr(), S["zg"].data_ptr(), E, H, I, st))
         for bm, t in tiles.items():
             _lib.check(Lb.nq_pf_gemm(tb.data_ptr(), t.data_ptr(), t.shape[0], bm, 0, S["xg"].data_ptr(), S["xu"].data_ptr(),
                                      S["acc"].data_ptr(), E, H, I, st))
-        _lib.check(Lb.nq_pf_mid(S["acc"].data_ptr(), pes.data_ptr(), n, tb.data_ptr(), S["h"].data_ptr(), E, H, I, st))
+        _lib.check(Lb.nq_pf_mid(S["acc"].data_ptr(), pes.data_ptr(), n, tb.data_ptr(), S["h"].data_ptr(), S["zg"].data_ptr(),
+                                S["zd"].data_ptr(), E, H, I, st))
         for bm, t in tiles.items():
             _lib.check(Lb.nq_pf_gemm(tb.data_ptr(), t.data_ptr(), t.shape[0], bm, 1, S["h"].data_ptr(), None,
                                      S["y"].data_ptr(), E, H, I, st))
         _lib.check(Lb.nq_pf_post(S["y"].data_ptr(), pos.data_ptr(), selc.data_ptr(), rwc.data_ptr(), T, k, c, n, tb.data_ptr(),
-                                 out.data_ptr(), E, H, I, st))
+                                 out.data_ptr(), S["zd"].data_ptr(), E, H, I, st))
     return out
 
 

@@ -289,3 +289,22 @@ def test_in_had_down_512_decode_and_prefill(golden_dir):
     bad = F.Expert(256, 384, seed=1, dev="cpu"); bad.had_dn = 512
     with pytest.raises(RuntimeError, match="in_had_down"):
         M.validate_row(M.entry(to_dev([bad])[0], 2), 256, 384)
+
+
+def test_low_rank_plane_decode_and_prefill(golden_dir):
+    """low-rank plane (z = x V^T; g, u += z U2 [+ U4 at level 4]; y += (sw V_d^T)(U2_d [+ U4_d])) alone and together with
+    the 512-wide rotation, against the reference's own moe_ref outputs"""
+    for had, key in ((128, "y_lr"), (512, "y_had512_lr")):
+        z, L, ex, x, sel, rw = _optional_feature_layer(golden_dir, had, True)
+        want = z[key]
+        for cg, cd in (([1, 4, 2], [1, 4, 4]), ([1, 4, 1], [1, 2, 1])):
+            y = L(x, sel, rw, cfg_gu=cg, cfg_dn=cd).clone()
+            torch.cuda.synchronize()
+            assert rel_err(y.cpu().numpy(), want) < 1e-4, (had, cg, cd)
+            assert torch.equal(y, L(x, sel, rw, cfg_gu=cg, cfg_dn=cd))
+        assert rel_err(L.prefill(x, sel, rw).cpu().numpy(), want) < 1e-4, had
+        assert rel_err(want, z["y_had512"]) > 1e-2
+    # a row with a low-rank buffer but no ranks, or ranks above 4, is refused
+    row = M.entry(ex[0], 2).clone(); row[16] = 5
+    with pytest.raises(RuntimeError, match="low-rank"):
+        M.validate_row(row, int(z["H"]), int(z["I"]))
