@@ -20,7 +20,7 @@ def test_slot_layout_and_rows():
     p = lay.parts
     assert p["gu.p3"] == (0, 3145728) and p["gu.p4"] == (3145728, 3145728) and p["dn.p3"][0] == 6291456
     assert p["gu.d3"][1] == 49152 and p["dn.d4"][1] == 24576 and lay.bytes % 256 == 0
-    assert sum(n for _, n in lay.spans(2, 3)) == 4718592 + 73728                # P3 + d3 of one expert (4 718 592 + 73 728)
+    assert sum(n for _, n in lay.spans(2, 3)) == 4718592 + 73728                # P3 + d3 of one expert: 4 718 592 + 73 728 bytes at H 6144, I 2048
     assert sum(n for _, n in lay.spans(3, 4)) == 4718592 + 73728
     assert lay.spans(2, 4) == [(0, lay.bytes)] and lay.bytes >= 2 * (4718592 + 73728)
 

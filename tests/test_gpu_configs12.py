@@ -1,4 +1,4 @@
-"""BASELINE configurations 1 and 2 on the GPU.
+"""The CPU-plumbing and single-projection configurations on the GPU.
 Config 1: one 512 x 256 weight ~ N(0,1), encoded at level 2 (minimal encoder), decoded by the HIP decoder (bit-exact vs
 the oracle), then decode+GEMV against one fp16 activation vector, within 1e-3 of an fp32 matmul over the oracle-dequantised
 weights. Config 2: single projection 6144 -> 2048 at levels 2/3/4 on the same base, token batch 1/4/8."""
