@@ -111,7 +111,9 @@ int nq_pf_pre(const void* x_f16, const int32_t* pt, const int32_t* pe, int np, c
  * row): for every tile t = tiles[t] = {expert, first pair row, rows, 0} (device int32[ntiles][4], rows <= bm,
  * bm in {16, 32, 64, 128, 256}):  C[row][n] = sum_k A[row][k] * W_expert[n][k]  with fp32 accumulation and output.
  * mode 0: gate|up, K = H, N = 2I, A0 = xg feeds weight rows [0, I), A1 = xu feeds rows [I, 2I), C = [np][2I];
- * mode 1: down, K = I, N = H, A0 = h, A1 ignored, C = [np][H]. Replaces pf_decode + the Triton grouped GEMM / aten.mm
+ * mode 1: down, K = I, N = H, A0 = h, A1 ignored, C = [np][H]. mode | 2: the variant for experts in mask mode (flags word of
+ * the table row set): it handles only their tiles, the plain variant only the others, so a layer with such experts makes
+ * both calls. Replaces pf_decode + the Triton grouped GEMM / aten.mm
  * (reference sm120/pf_gemm.py:7-34, sm120/moe.py:303-324); decoded weights never touch HBM. */
 int nq_pf_gemm(const int64_t* table, const int32_t* tiles, int ntiles, int bm, int mode, const void* A0_f16,
                const void* A1_f16, float* C, int E, int H, int I, void* stream);

@@ -35,7 +35,7 @@ extern "C" int nq_validate_row(const int64_t* r, int H, int I)
     NQ_REQUIRE(lv == 0 || lv == 2 || lv == 3 || lv == 4, "table row: level %lld not in {0,2,3,4}", (long long)lv);
     if (lv == 0) return 0;
     NQ_REQUIRE(r[1] && r[5] && r[9], "table row: null base plane or sign vector");
-    NQ_REQUIRE(r[4] == 0 && r[8] == 0, "table row: mask mode (flags) is not implemented");
+    NQ_REQUIRE((r[4] == 0 && r[8] == 0) || lv == 2 || (lv == 4 && r[10] < CODE_L3 && r[11] < CODE_L3), "table row: mask mode (flags) goes with the wide residual plane of level 4 only");
     NQ_REQUIRE(r[14] ? (r[15] != 0 && r[16] >= 0 && r[16] <= 4 && r[17] >= 0 && r[17] <= 4 && r[16] + r[17] > 0) : (r[15] == 0 && r[16] == 0 && r[17] == 0),
                "table row: low-rank plane needs both buffers and ranks r_gu, r_dn in [0, 4] (got %lld, %lld)", (long long)r[16], (long long)r[17]);
     NQ_REQUIRE(r[18] == 0 || r[18] == 128 || (r[18] == 512 && I % 512 == 0), "table row: in_had_down %lld must be 0, 128, or 512 dividing I = %d", (long long)r[18], I);
@@ -136,8 +136,8 @@ extern "C" int nq_pf_gemm(const int64_t* table, const int32_t* tiles, int ntiles
     NQ_REQUIRE(ntiles >= 0, "nq_pf_gemm: ntiles=%d", ntiles);
     if (ntiles == 0) return 0;
     NQ_REQUIRE(table && tiles && A0 && C, "nq_pf_gemm: null pointer");
-    NQ_REQUIRE(mode == 0 || mode == 1, "nq_pf_gemm: mode %d not in {0,1}", mode);
-    NQ_REQUIRE(mode == 1 || A1, "nq_pf_gemm: gate|up needs both activation buffers");
+    NQ_REQUIRE(mode >= 0 && mode <= 3, "nq_pf_gemm: mode %d not in 0..3", mode);
+    NQ_REQUIRE((mode & 1) == 1 || A1, "nq_pf_gemm: gate|up needs both activation buffers");
     NQ_REQUIRE(ntiles <= 65535, "nq_pf_gemm: %d tiles exceed one launch (65535)", ntiles);
     NQ_REQUIRE(E >= 1 && shape_ok(H, I), "nq_pf_gemm: E=%d H=%d I=%d (H, I positive multiples of 128)", E, H, I);
     return launch_pf_gemm(table, tiles, ntiles, bm, mode, A0, A1, C, E, H, I, (hipStream_t)stream);

@@ -224,16 +224,27 @@ __device__ __forceinline__ uint32_t weight_pair(const uint32_t* wb, const uint32
 
 // ---- table row ------------------------------------------------------------------------------------------------------
 // int64[20] per expert (reference sm120/moe.py:216-229, sm120/nqmoe.cu:26-45):
-//   [0] level 0/2/3/4  [1..4] gate|up base, residual plane, block words, flags  [5..8] down  [9] sign/scale vector
+//   [0] level 0/2/3/4  [1..4] gate|up base, residual plane, block words, flags (mask mode, 0 = dense)  [5..8] down  [9] sign/scale vector
 //   [10],[11] residual window code of gate|up, down  [12],[13] sign-variant planes  [14..17] low-rank plane (unsupported)
 //   [18] in_had_down (unsupported unless 0/128)  [19] base codes (unsupported unless 0)
-struct Planes { gp_u4 base; gp_u8 res; gp_u32 dw; gp_u8 var; int code; };
+typedef const NQ_GLOBAL uint64_t* gp_u64;
+struct Planes { gp_u4 base; gp_u8 res; gp_u32 dw; gp_u8 var; int code; gp_u64 flags; };
+
+// Mask mode (reference sm120/nqmoe.cu:22-24,202-206): flags = one uint64 per strip, bit c = chunk c is refined; the residual
+// plane and its block words are compact over the nm = popcount(flags) refined chunks of every strip, in chunk order, and
+// the other chunks decode at level 2. Flags are equal over the 8 strips of a 128-row group.
+struct MaskedUnit { bool on; size_t unit; size_t nrec; };     // refined?; residual unit index; residual records of the plane
+__device__ __forceinline__ MaskedUnit masked_unit(uint64_t f, size_t strip, int c, size_t nstrips)
+{
+    const int nm = __popcll(f);
+    return MaskedUnit{((f >> c) & 1ull) != 0, strip * nm + __popcll(f & ((1ull << c) - 1ull)), nstrips * nm * 32};
+}
 __device__ __forceinline__ Planes planes_of(const int64_t* ent, int mode)
 {
     const int o = mode == 0 ? 1 : 5;
     Planes P;
     P.base = (gp_u4)ent[o]; P.res = (gp_u8)ent[o + 1]; P.dw = (gp_u32)ent[o + 2];
-    P.var = (gp_u8)ent[mode == 0 ? 12 : 13]; P.code = (int)ent[10 + mode];
+    P.var = (gp_u8)ent[mode == 0 ? 12 : 13]; P.code = (int)ent[10 + mode]; P.flags = (gp_u64)ent[o + 3];
     return P;
 }
 

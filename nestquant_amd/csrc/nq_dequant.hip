@@ -35,7 +35,7 @@ __device__ __forceinline__ void decode_to_tile(const uint32_t* wb, const uint32_
 }
 
 // decode unit `unit` of projection planes P (level lv) into tile; all 64 lanes of the wave call this together
-__device__ __forceinline__ void decode_unit(const Planes& P, int lv, size_t unit, size_t nrec, uint32_t* tile, int lane)
+__device__ __forceinline__ void decode_unit(const Planes& P, int lv, size_t unit, size_t nrec, int C, uint32_t* tile, int lane)
 {
     const int lane32 = lane & 31;
     const int src = (lane & ~3) | ((lane + 1) & 3);           // next lane of the ring
@@ -46,17 +46,26 @@ __device__ __forceinline__ void decode_unit(const Planes& P, int lv, size_t unit
         ext_words<128, 4>(wb, __shfl(wb[0], src));
     }
     const uint32_t sgm = P.var ? (((uint32_t)P.var[unit] >> (lane32 >> 2)) & 1u) * 0x80008000u : 0u;
-    if (lv == 2)
+    size_t runit = unit, rnrec = nrec;                          // residual unit / records: compact in mask mode
+    bool on = lv != 2;
+    if (on && P.flags)
+    {   // the two halves of a wavefront may sit in different strips or chunks: this branch may diverge between them, and the
+        // ring neighbour of a lane is always in its own half
+        const size_t strip = unit / C;
+        const MaskedUnit m = masked_unit(P.flags[strip], strip, (int)(unit - strip * C), nrec / 32 / C);
+        on = m.on; runit = m.unit; rnrec = m.nrec;
+    }
+    if (!on)
     {
         decode_to_tile<false, 0>(wb, wb, consts_l2(sgm), tile, lane32);
         return;
     }
-    const uint32_t dw = P.dw[unit];
+    const uint32_t dw = P.dw[runit];
     const FoldK k = consts_fold(dw, sgm);
     dispatch_code(P.code, [&](auto tag) {
         constexpr int CODE = decltype(tag)::value;
         uint32_t wr[Rec<CODE>::NW + 2];
-        load_record<CODE>(wr, P.res, unit * 32 + lane32, nrec);
+        load_record<CODE>(wr, P.res, runit * 32 + lane32, rnrec);
         ext_words<Rec<CODE>::BITS, Rec<CODE>::NW>(wr, __shfl(wr[0], src));
         decode_to_tile<true, CODE>(wb, wr, k, tile, lane32);
     });
@@ -91,7 +100,7 @@ __device__ __forceinline__ void dequant_body(const int64_t* ent, int mode, int l
         return;
     }
     const Planes P = planes_of(ent, mode);
-    decode_unit(P, lv, unit, nrec, tile, lane);
+    decode_unit(P, lv, unit, nrec, C, tile, lane);
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     // each half-wave wrote its own tile; the whole wave now drains both tiles

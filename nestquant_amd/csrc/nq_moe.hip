@@ -134,7 +134,7 @@ __device__ __forceinline__ void route(const MoeArgs& a, int z, RunInfo* R, int l
 {
     const int S = a.B * a.topk;
     int e = -1, lv = 0; bool ok = false;
-    int64_t f_base = 0, f_res = 0, f_dw = 0, f_var = 0, f_code = 0, f_signs = 0, f_had = 0, f_lr = 0, f_lr4 = 0, f_rg = 0, f_rd = 0;
+    int64_t f_base = 0, f_res = 0, f_dw = 0, f_var = 0, f_code = 0, f_signs = 0, f_had = 0, f_lr = 0, f_lr4 = 0, f_rg = 0, f_rd = 0, f_flags = 0;
     if (lane < S)
     {
         const long long ee = sel_at(a, lane);
@@ -145,7 +145,7 @@ __device__ __forceinline__ void route(const MoeArgs& a, int z, RunInfo* R, int l
             constexpr int o = MODE == 0 ? 1 : 5;
             lv = (int)ent[0];
             f_base = ent[o]; f_res = ent[o + 1]; f_dw = ent[o + 2]; f_var = ent[MODE == 0 ? 12 : 13]; f_code = ent[10 + MODE]; f_signs = ent[9]; f_had = ent[18];
-            f_lr = ent[14]; f_lr4 = ent[15]; f_rg = ent[16]; f_rd = ent[17];
+            f_lr = ent[14]; f_lr4 = ent[15]; f_rg = ent[16]; f_rd = ent[17]; f_flags = ent[o + 3];
             ok = rw_at(a, lane) != 0.f && lv > 0;
         }
     }
@@ -167,7 +167,7 @@ __device__ __forceinline__ void route(const MoeArgs& a, int z, RunInfo* R, int l
             if (pos == 0)
             {
                 Planes P;
-                P.base = (gp_u4)f_base; P.res = (gp_u8)f_res; P.dw = (gp_u32)f_dw; P.var = (gp_u8)f_var; P.code = (int)f_code;
+                P.base = (gp_u4)f_base; P.res = (gp_u8)f_res; P.dw = (gp_u32)f_dw; P.var = (gp_u8)f_var; P.code = (int)f_code; P.flags = (gp_u64)f_flags;
                 R->P = P; R->signs = (const _Float16*)f_signs;
                 R->level = a.force_level ? a.force_level : lv;
                 R->had = f_had == 512 ? 512 : 128;
@@ -405,11 +405,11 @@ __global__ void __launch_bounds__(256) nq_gemv_k(MoeArgs a, int NC)
     const int strip = 2 * (blockIdx.x * SB + warp) + ss;
     Planes P;                                                    // block-uniform: keep the plane addresses in scalar registers
     P.base = (gp_u4)uni((uint64_t)R.P.base); P.res = (gp_u8)uni((uint64_t)R.P.res); P.dw = (gp_u32)uni((uint64_t)R.P.dw);
-    P.var = (gp_u8)uni((uint64_t)R.P.var); P.code = __builtin_amdgcn_readfirstlane(R.P.code);
+    P.var = (gp_u8)uni((uint64_t)R.P.var); P.code = __builtin_amdgcn_readfirstlane(R.P.code); P.flags = (gp_u64)uni((uint64_t)R.P.flags);
     LaneCtx L;
     L.unit0 = (size_t)strip * C + chunk0; L.rec0 = L.unit0 * 32 + 4 * g + t4;
     L.nrec = (size_t)(N / 16) * C * 32;
-    L.src = (lane + 16) & 63; L.g = g;
+    L.src = (lane + 16) & 63; L.g = g; L.strip = (size_t)strip; L.nstrips = (size_t)(N / 16); L.chunk0 = chunk0;
     L.xs = (n < ntok ? smem + n * rowstride : zero) + t4 * 16; L.xstep = n < ntok ? 256 : 0;
     const u32x4 nb0 = P.base[L.rec0];
 

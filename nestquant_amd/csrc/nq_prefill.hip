@@ -253,14 +253,16 @@ struct PfGemm
 };
 
 // body for one (RES, CODE): all K / 128 chunks of this wave's two strips against the tile's tokens
-template <int TG, bool RES, int CODE>
+template <int TG, bool RES, int CODE, bool MASKED>
 __device__ __forceinline__ void pf_chunks(const Planes& P, const LaneCtx& L, int C, const _Float16* A, int K, int row0, int nrows,
                                           char* smem, float4_t (*acc)[2])
 {
     constexpr int NW = RES ? Rec<CODE>::NW : 1;
     u32x4 nb = P.base[L.rec0];
     uint32_t nr[NW + 2] = {0}, ndw = 0, nvar = 0;
-    if constexpr (RES) { load_record<CODE>(nr, P.res, L.rec0, L.nrec); ndw = P.dw[L.unit0]; }
+    constexpr bool masked = RES && MASKED;                       // the kernel variant for experts in mask mode
+    const uint64_t mflags = masked ? P.flags[L.strip] : 0ull;
+    if constexpr (RES && !masked) { load_record<CODE>(nr, P.res, L.rec0, L.nrec); ndw = P.dw[L.unit0]; }
     if (P.var) nvar = P.var[L.unit0];
     const int lane = threadIdx.x & 63, warp = threadIdx.x >> 6, t4 = lane >> 4, n = lane & 15;
     // Staging: wavefront w copies rows 16 u + 4 w + (lane >> 4), u = 0 .. TG - 1, of the tile, one 1 KB
@@ -291,28 +293,46 @@ __device__ __forceinline__ void pf_chunks(const Planes& P, const LaneCtx& L, int
         wb[0] = nb.x; wb[1] = nb.y; wb[2] = nb.z; wb[3] = nb.w;
 #pragma unroll
         for (int i = 0; i < NW; ++i) wr[i] = nr[i];
-        const uint32_t dw = ndw, var = nvar;
+        uint32_t dw = ndw;
+        const uint32_t var = nvar;
+        bool on = true;                                          // mask mode: is chunk c refined? (the same for the whole workgroup)
+        if constexpr (masked)
+            {   // residual records are compact over the refined chunks and fetched when needed
+                const MaskedUnit m = masked_unit(mflags, L.strip, c, L.nstrips);
+                on = __builtin_amdgcn_readfirstlane((int)m.on) != 0;
+                if (on) { load_record<CODE>(wr, P.res, m.unit * 32 + (L.rec0 & 31), m.nrec); dw = P.dw[m.unit]; }
+            }
         if (c + 1 < C)
         {
             nb = P.base[L.rec0 + (size_t)(c + 1) * 32];
-            if constexpr (RES) { load_record<CODE>(nr, P.res, L.rec0 + (size_t)(c + 1) * 32, L.nrec); ndw = P.dw[L.unit0 + c + 1]; }
+            if constexpr (RES && !masked) { load_record<CODE>(nr, P.res, L.rec0 + (size_t)(c + 1) * 32, L.nrec); ndw = P.dw[L.unit0 + c + 1]; }
             if (P.var) nvar = P.var[L.unit0 + c + 1];
         }
         ext_words<128, 4>(wb, __shfl(wb[0], L.src));
         const uint32_t sgm = ((var >> L.g) & 1u) * 0x80008000u;
-        FoldK k;
-        if constexpr (RES)
-        {
-            ext_words<Rec<CODE>::BITS, Rec<CODE>::NW>(wr, __shfl(wr[0], L.src));
-            k = consts_fold(dw, sgm);
-        }
-        else k = consts_l2(sgm);
         half8_t aop[4][2];
-        static_for<4>([&](auto mm) {
-            constexpr int MM = decltype(mm)::value;
-            aop[MM][0] = a_operand<RES, CODE, MM, 0>(wb, wr, k);
-            aop[MM][1] = a_operand<RES, CODE, MM, 1>(wb, wr, k);
-        });
+        if (RES && (!masked || on))
+        {
+            if constexpr (RES)
+            {
+                ext_words<Rec<CODE>::BITS, Rec<CODE>::NW>(wr, __shfl(wr[0], L.src));
+                const FoldK k = consts_fold(dw, sgm);
+                static_for<4>([&](auto mm) {
+                    constexpr int MM = decltype(mm)::value;
+                    aop[MM][0] = a_operand<RES, CODE, MM, 0>(wb, wr, k);
+                    aop[MM][1] = a_operand<RES, CODE, MM, 1>(wb, wr, k);
+                });
+            }
+        }
+        else
+        {
+            const FoldK k = consts_l2(sgm);
+            static_for<4>([&](auto mm) {
+                constexpr int MM = decltype(mm)::value;
+                aop[MM][0] = a_operand<false, 0, MM, 0>(wb, wr, k);
+                aop[MM][1] = a_operand<false, 0, MM, 1>(wb, wr, k);
+            });
+        }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");         // this wavefront's share of the tile has landed
         __syncthreads();
         // ---- TG x 8 MFMAs: tokens 16 tg + n as the N dimension (row groups beyond the tile multiply stale LDS rows whose
@@ -371,7 +391,9 @@ __device__ __forceinline__ void pf_chunks(const Planes& P, const LaneCtx& L, int
 // grid (N / 128, ntiles), block 256 (4 wavefronts x 2 strips = 128 weight rows); dynamic LDS = 16 TG * PF_ROW bytes
 // two workgroups per CU at every tile height (the tallest would otherwise need one register too many): while one decodes on
 // the vector ALUs the other runs its MFMAs
-template <int TG>
+// MASKED = false skips the tiles of experts in mask mode (table flags word set), MASKED = true takes only those: the rarely
+// used path keeps its extra registers out of the common kernel
+template <int TG, bool MASKED>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) nq_pf_gemm_k(PfGemm a)
 {
     extern __shared__ __align__(16) char smem[];
@@ -387,15 +409,17 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) n
     const _Float16* A = (a.mode == 0 && (int)(blockIdx.x * 128) >= a.I) ? a.A1 : a.A0;
     const int t4 = lane >> 4, ss = (lane >> 3) & 1, g = lane & 7, n = lane & 15;
     const Planes P = planes_of(ent, a.mode);
+    if ((P.flags != nullptr && lv == 4) != MASKED) return;       // block-uniform
     LaneCtx L;
     L.unit0 = (size_t)(2 * sp + ss) * C; L.rec0 = L.unit0 * 32 + 4 * g + t4;
     L.nrec = (size_t)(N / 16) * C * 32;
     L.src = (lane + 16) & 63; L.g = g; L.xs = nullptr; L.xstep = 0;
+    L.strip = (size_t)(2 * sp + ss); L.nstrips = (size_t)(N / 16); L.chunk0 = 0;
     float4_t acc[TG][2];
 #pragma unroll
     for (int tg = 0; tg < TG; ++tg) { acc[tg][0] = float4_t{0.f, 0.f, 0.f, 0.f}; acc[tg][1] = float4_t{0.f, 0.f, 0.f, 0.f}; }
-    if (lv == 2) pf_chunks<TG, false, 0>(P, L, C, A, K, row0, nrows, smem, acc);
-    else dispatch_code(P.code, [&](auto tag) { pf_chunks<TG, true, decltype(tag)::value>(P, L, C, A, K, row0, nrows, smem, acc); });
+    if (lv == 2) pf_chunks<TG, false, 0, false>(P, L, C, A, K, row0, nrows, smem, acc);
+    else dispatch_code(P.code, [&](auto tag) { pf_chunks<TG, true, decltype(tag)::value, MASKED>(P, L, C, A, K, row0, nrows, smem, acc); });
     // lane (t4, n) holds, for token 16 tg + n, weight rows 32 sp + 16 (t4 >> 1) + 4 (t4 & 1) + i (+ 8 for acc[..][1])
     const int wrow = 32 * sp + 16 * (t4 >> 1) + 4 * (t4 & 1);
 #pragma unroll
@@ -440,16 +464,16 @@ int launch_pf_hits(const int32_t* counts, int32_t* hits, int E, hipStream_t st)
     return 0;
 }
 
-template <int TG>
+template <int TG, bool MASKED>
 static int launch_gemm_tg(const PfGemm& a, int ntiles, int N, hipStream_t st)
 {
     const int shm = 16 * TG * PF_ROW;
     if (shm > 48 * 1024)
     {
-        hipError_t e = hipFuncSetAttribute((const void*)nq_pf_gemm_k<TG>, hipFuncAttributeMaxDynamicSharedMemorySize, shm);
+        hipError_t e = hipFuncSetAttribute((const void*)nq_pf_gemm_k<TG, MASKED>, hipFuncAttributeMaxDynamicSharedMemorySize, shm);
         if (e != hipSuccess) return set_error("nq_pf_gemm: LDS %d bytes: %s", shm, hipGetErrorString(e));
     }
-    nq_pf_gemm_k<TG><<<dim3(N / 128, ntiles), 256, shm, st>>>(a);
+    nq_pf_gemm_k<TG, MASKED><<<dim3(N / 128, ntiles), 256, shm, st>>>(a);
     NQ_LAUNCH_CHECK("nq_pf_gemm");
     return 0;
 }
@@ -458,15 +482,16 @@ int launch_pf_gemm(const int64_t* table, const int32_t* tiles, int ntiles, int b
                    int E, int H, int I, hipStream_t st)
 {
     if (!ntiles) return 0;
-    PfGemm a{table, tiles, (const _Float16*)A0, (const _Float16*)A1, C, mode, E, H, I};
-    const int N = mode == 0 ? 2 * I : H;
+    PfGemm a{table, tiles, (const _Float16*)A0, (const _Float16*)A1, C, mode & 1, E, H, I};
+    const int N = (mode & 1) == 0 ? 2 * I : H;
+    const bool masked = (mode & 2) != 0;
     switch (bm)
     {
-        case 16: return launch_gemm_tg<1>(a, ntiles, N, st);
-        case 32: return launch_gemm_tg<2>(a, ntiles, N, st);
-        case 64: return launch_gemm_tg<4>(a, ntiles, N, st);
-        case 128: return launch_gemm_tg<8>(a, ntiles, N, st);
-        case 256: return launch_gemm_tg<16>(a, ntiles, N, st);
+        case 16: return masked ? launch_gemm_tg<1, true>(a, ntiles, N, st) : launch_gemm_tg<1, false>(a, ntiles, N, st);
+        case 32: return masked ? launch_gemm_tg<2, true>(a, ntiles, N, st) : launch_gemm_tg<2, false>(a, ntiles, N, st);
+        case 64: return masked ? launch_gemm_tg<4, true>(a, ntiles, N, st) : launch_gemm_tg<4, false>(a, ntiles, N, st);
+        case 128: return masked ? launch_gemm_tg<8, true>(a, ntiles, N, st) : launch_gemm_tg<8, false>(a, ntiles, N, st);
+        case 256: return masked ? launch_gemm_tg<16, true>(a, ntiles, N, st) : launch_gemm_tg<16, false>(a, ntiles, N, st);
     }
     return set_error("nq_pf_gemm: tile height %d not in {16, 32, 64, 128, 256}", bm);
 }

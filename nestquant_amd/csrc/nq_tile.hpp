@@ -59,11 +59,63 @@ struct LaneCtx
     int g;                // ring index (sign-variant bit)
     const char* xs;       // this lane's B-operand base in LDS (bytes), kg folded in
     int xstep;            // bytes per chunk (0 for lanes without a token)
+    size_t strip, nstrips; int chunk0;   // mask mode: this lane's strip, strips of the projection, first chunk of the k-slice
 };
+
+// mask mode: chunk by chunk either the folded decode (refined chunks, residual records compact over them) or the level-2
+// decode; the choice is the same for every lane of the workgroup. Residual records are fetched when needed (no prefetch).
+template <int CODE>
+__device__ __forceinline__ void gemv_chunks_masked(const Planes& P, const LaneCtx& L, int NC, float4_t* acc, u32x4 nb)
+{
+    constexpr int NW = Rec<CODE>::NW;
+    const uint64_t f = P.flags[L.strip];
+    uint32_t nvar = P.var ? (uint32_t)P.var[L.unit0] : 0u;
+    for (int c = 0; c < NC; ++c)
+    {
+        uint32_t wb[6], wr[NW + 2] = {0};
+        wb[0] = nb.x; wb[1] = nb.y; wb[2] = nb.z; wb[3] = nb.w;
+        const uint32_t var = nvar;
+        const MaskedUnit m = masked_unit(f, L.strip, L.chunk0 + c, L.nstrips);
+        const bool on = __builtin_amdgcn_readfirstlane((int)m.on) != 0;
+        uint32_t dw = 0;
+        if (on) { load_record<CODE>(wr, P.res, m.unit * 32 + (L.rec0 & 31), m.nrec); dw = P.dw[m.unit]; }
+        if (c + 1 < NC)
+        {
+            nb = P.base[L.rec0 + (size_t)(c + 1) * 32];
+            if (P.var) nvar = P.var[L.unit0 + c + 1];
+        }
+        ext_words<128, 4>(wb, __shfl(wb[0], L.src));
+        const uint32_t sgm = ((var >> L.g) & 1u) * 0x80008000u;
+        const char* xp = L.xs + c * L.xstep;
+        if (on)
+        {
+            ext_words<Rec<CODE>::BITS, Rec<CODE>::NW>(wr, __shfl(wr[0], L.src));
+            const FoldK k = consts_fold(dw, sgm);
+            static_for<4>([&](auto mm) {
+                constexpr int MM = decltype(mm)::value;
+                const half8_t b = *(const half8_t*)(xp + MM * 64);
+                acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_operand<true, CODE, MM, 0>(wb, wr, k), b, acc[0], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_operand<true, CODE, MM, 1>(wb, wr, k), b, acc[1], 0, 0, 0);
+            });
+        }
+        else
+        {
+            const FoldK k = consts_l2(sgm);
+            static_for<4>([&](auto mm) {
+                constexpr int MM = decltype(mm)::value;
+                const half8_t b = *(const half8_t*)(xp + MM * 64);
+                acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_operand<false, 0, MM, 0>(wb, wr, k), b, acc[0], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_operand<false, 0, MM, 1>(wb, wr, k), b, acc[1], 0, 0, 0);
+            });
+        }
+    }
+}
 
 template <bool RES, int CODE>
 __device__ __forceinline__ void gemv_chunks(const Planes& P, const LaneCtx& L, int NC, float4_t* acc, u32x4 nb)
 {
+    if constexpr (RES)
+        if (P.flags) { gemv_chunks_masked<CODE>(P, L, NC, acc, nb); return; }     // block-uniform
     constexpr int NW = RES ? Rec<CODE>::NW : 1;
     uint32_t nr[NW + 2] = {0}, ndw = 0, nvar = 0;
     if constexpr (RES) { load_record<CODE>(nr, P.res, L.rec0, L.nrec); ndw = P.dw[L.unit0]; }

@@ -2,8 +2,8 @@
 
 Host-side mirror of the format half of the reference's sm120/moe.py (RKP/RK_OF :10-12, rbits :17, step_off :18-20,
 proj_sizes :23-26, pack_words/unpack_words :36-66, Proj :76-107, Expert :177-195). Same names and argument meaning, so
-loaders and tests written against the reference read the same here. Mask mode (nm) and base codes other than 0 are not
-implemented and raise.
+loaders and tests written against the reference read the same here. Base codes other than 0 are not implemented and
+raise.
 
 Nested levels of this build (the reference serves levels 0/2/4 only): an expert built with nested=True also carries
 P3 (64 bits / record, K=1 windows, code 10) with block words d3, and P4 (64 bits / record) with block words d4n. Level 3
@@ -42,14 +42,25 @@ def split_bits(bits):
 
 
 def proj_sizes(N, K, nm=None, rk=0, bk=0):
-    """bytes per plane of a projection [N, K]; nm (mask mode) is not implemented"""
-    if nm is not None:
-        raise NotImplementedError("mask mode (nm) is not implemented")
+    """bytes per plane of a projection [N, K] (reference sm120/moe.py:23-26). nm = None: dense residual plane; else mask
+    mode: nm flagged chunks per strip, the residual plane and its block words compact over them, flags = int64 per strip"""
     S, C = N // 16, K // 128
+    R = C if nm is None else nm
     pad = lambda code: 4 if rbits(code) % 16 else 0
-    return dict(S=S, C=C, nm=None, rk=rk, bk=bk, base=S * C * 32 * rbits(bk) // 8 + pad(bk),
-                p4=S * C * 32 * rbits(rk) // 8 + pad(rk), d4=S * C * 4, flags=0, nrec_r=S * C * 32,
+    return dict(S=S, C=C, nm=nm, rk=rk, bk=bk, base=S * C * 32 * rbits(bk) // 8 + pad(bk),
+                p4=S * R * 32 * rbits(rk) // 8 + pad(rk), d4=S * R * 4, flags=0 if nm is None else S * 8, nrec_r=S * R * 32,
                 p3=S * C * 32 * 8, d3=S * C * 4)
+
+
+def make_flags(S, C, nm, gen, grp=8):
+    """nm flagged chunks per strip, identical across each group of `grp` strips (reference sm120/moe.py:28-34):
+    (int64 [S], bit c = chunk c is refined; bool [S, C])"""
+    dev = gen.device
+    ng = (S + grp - 1) // grp
+    idx = torch.rand(ng, C, generator=gen, device=dev).argsort(1)[:, :nm]
+    fl = torch.zeros(ng, C, dtype=torch.bool, device=dev); fl.scatter_(1, idx, True)
+    fl = fl.repeat_interleave(grp, 0)[:S]
+    return (fl.long() << torch.arange(C, device=dev)).sum(1), fl
 
 
 def _bytes_le(t, nb):
@@ -147,34 +158,37 @@ class Proj:
     with the same seed yields the same planes as the reference's Proj."""
 
     def __init__(s, N, K, gen, nm=None, rk=0, mbn="rand", var=False, bk=0, nested=False):
-        if nm is not None or bk != 0:
-            raise NotImplementedError("mask mode and base codes other than 0 are not implemented")
+        if bk != 0:
+            raise NotImplementedError("base codes other than 0 are not implemented")
+        if nm is not None and nested:
+            raise NotImplementedError("mask mode applies to the wide residual plane, not to the nested planes")
         dev = gen.device
-        z = proj_sizes(N, K, None, rk, bk)
+        z = proj_sizes(N, K, nm, rk, bk)
         s.z, s.N, s.K, s.rk, s.bk, s.nested = z, N, K, rk, bk, nested
         S, C = z["S"], z["C"]
-        nr, nb = S * C * 32, S * C
+        R = C if nm is None else nm                      # residual records and block words exist for R chunks per strip
+        nr, nb = S * C * 32, S * R
         bits = rbits(rk); nw = (bits + 31) // 32
         s.base = torch.randint(-2**31, 2**31 - 1, (nr * 4,), generator=gen, dtype=torch.int32, device=dev)
-        w = torch.randint(0, 2**32, (nr, nw), generator=gen, dtype=torch.int64, device=dev)
+        w = torch.randint(0, 2**32, (nb * 32, nw), generator=gen, dtype=torch.int64, device=dev)
         if bits % 32:
             w[:, -1] &= (1 << (bits % 32)) - 1
         s.p4w, s.p4 = w, pack_words(w, bits)
         s.Mb, s.Nn = _block_words(nb, gen, mbn, dev)
         s.d4 = (s.Mb | (s.Nn << 8)).to(torch.int32)
-        s.var = torch.randint(0, 256, (nb,), generator=gen, dtype=torch.int64, device=dev).to(torch.uint8) if var else None
-        s.flags = s.fl = None
+        s.var = torch.randint(0, 256, (S * C,), generator=gen, dtype=torch.int64, device=dev).to(torch.uint8) if var else None
+        s.flags, s.fl = (None, None) if nm is None else make_flags(S, C, nm, gen)
         s.p3 = s.d3 = s.p4n = s.d4n = s.p3w = s.p4nw = None
         if nested:
             s.p3w = torch.randint(0, 2**32, (nr, 2), generator=gen, dtype=torch.int64, device=dev)
             s.p4nw = torch.randint(0, 2**32, (nr, 2), generator=gen, dtype=torch.int64, device=dev)
             s.p3, s.p4n = pack_words(s.p3w, 64), pack_words(s.p4nw, 64)
-            s.Mb3, s.N3 = _block_words(nb, gen, "rand", dev)
-            s.Mb4n, s.N4n = _block_words(nb, gen, "rand", dev)
+            s.Mb3, s.N3 = _block_words(S * C, gen, "rand", dev)
+            s.Mb4n, s.N4n = _block_words(S * C, gen, "rand", dev)
             s.d3 = (s.Mb3 | (s.N3 << 8)).to(torch.int32)
             s.d4n = (s.Mb4n | (s.N4n << 8)).to(torch.int32)
 
-    _TENSORS = ["base", "p4", "d4", "p4w", "Mb", "Nn", "var", "p3", "d3", "p4n", "d4n", "p3w", "p4nw"]
+    _TENSORS = ["base", "p4", "d4", "flags", "fl", "p4w", "Mb", "Nn", "var", "p3", "d3", "p4n", "d4n", "p3w", "p4nw"]
 
     def to(s, dev):
         for k in s._TENSORS:

@@ -136,6 +136,7 @@ class MoELayer:
         s.zd = torch.zeros(S * (I // 128) * 4, dtype=f32, device=dev); s.cnt_h = torch.zeros(S * (I // 128), dtype=i32, device=dev)
         s.out = torch.zeros(Bmax, H, dtype=f32, device=dev)
         s.hits_ptr = 0
+        s.masked = False                              # set once a row with mask-mode flags is installed (set / Mailbox.post)
         s._alloc_partials()
 
     @staticmethod
@@ -166,6 +167,7 @@ class MoELayer:
     def set(s, e, ex, level):
         row = entry(ex, level)
         validate_row(row, s.H, s.I)
+        s.masked |= bool(row[4] or row[8])
         s.table[e].copy_(row.to(s.table.device), non_blocking=False)
 
     def __call__(s, x, sel, rw, out=None, force_level=0, which=3, cfg_gu=None, cfg_dn=None, table=None):
@@ -274,14 +276,17 @@ def prefill(s, x, sel, rw, out=None, R=None, G=None, table=None):
         pts, pes = pt[c:d], pe[c:d]
         _lib.check(Lb.nq_pf_pre(x.data_ptr(), pts.data_ptr(), pes.data_ptr(), n, tb.data_ptr(), S["xg"].data_ptr(),
                                 S["xu"].data_ptr(), S["zg"].data_ptr(), E, H, I, st))
+        variants = (0, 2) if s.masked else (0,)                   # experts in mask mode run in their own kernel variant
         for bm, t in tiles.items():
-            _lib.check(Lb.nq_pf_gemm(tb.data_ptr(), t.data_ptr(), t.shape[0], bm, 0, S["xg"].data_ptr(), S["xu"].data_ptr(),
-                                     S["acc"].data_ptr(), E, H, I, st))
+            for v in variants:
+                _lib.check(Lb.nq_pf_gemm(tb.data_ptr(), t.data_ptr(), t.shape[0], bm, v, S["xg"].data_ptr(), S["xu"].data_ptr(),
+                                         S["acc"].data_ptr(), E, H, I, st))
         _lib.check(Lb.nq_pf_mid(S["acc"].data_ptr(), pes.data_ptr(), n, tb.data_ptr(), S["h"].data_ptr(), S["zg"].data_ptr(),
                                 S["zd"].data_ptr(), E, H, I, st))
         for bm, t in tiles.items():
-            _lib.check(Lb.nq_pf_gemm(tb.data_ptr(), t.data_ptr(), t.shape[0], bm, 1, S["h"].data_ptr(), None,
-                                     S["y"].data_ptr(), E, H, I, st))
+            for v in variants:
+                _lib.check(Lb.nq_pf_gemm(tb.data_ptr(), t.data_ptr(), t.shape[0], bm, 1 | v, S["h"].data_ptr(), None,
+                                         S["y"].data_ptr(), E, H, I, st))
         _lib.check(Lb.nq_pf_post(S["y"].data_ptr(), pos.data_ptr(), selc.data_ptr(), rwc.data_ptr(), T, k, c, n, tb.data_ptr(),
                                  out.data_ptr(), S["zd"].data_ptr(), E, H, I, st))
     return out
@@ -309,6 +314,7 @@ class Mailbox:
         """enqueue on `stream`, after any plane copy already enqueued there: stage[e] = row; seq[e] += 1"""
         assert s.done(e), "one outstanding op per expert"
         validate_row(row, s.L.H, s.L.I)
+        s.L.masked |= bool(row[4] or row[8])
         s.hseq[e] += 1
         r = row.pin_memory(); q = torch.tensor([s.hseq[e]], dtype=torch.int32).pin_memory()
         s.pins += [r, q]

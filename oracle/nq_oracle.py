@@ -250,14 +250,17 @@ def ring_states(words, code, G=4):
 class Plane:
     """planes of one projection as the oracle sees them (all numpy, host memory):
     N, K; base [nrec,4] uint32; level-4 residual: rk code + res [nrec,NW] uint32 + d4 [units] uint32 (Mb | N << 8);
-    nested planes: p3 [nrec,2] + d3 [units], p4n [nrec,2] + d4n [units]; var: uint8 per unit (bit g = ring g negated)."""
+    nested planes: p3 [nrec,2] + d3 [units], p4n [nrec,2] + d4n [units]; var: uint8 per unit (bit g = ring g negated);
+    flags (mask mode, reference sm120/moe.py:134-155): int64 per strip, bit c = chunk c is refined; res and d4 then hold only
+    the popcount(flags) refined chunks of each strip, in chunk order, and the other chunks decode at level 2."""
 
-    def __init__(self, N, K, base, rk=0, res=None, d4=None, p3=None, d3=None, p4n=None, d4n=None, var=None):
+    def __init__(self, N, K, base, rk=0, res=None, d4=None, p3=None, d3=None, p4n=None, d4n=None, var=None, flags=None):
         self.N, self.K = N, K
         self.S, self.C = N // 16, K // 128
         self.base = np.asarray(base, np.uint32).reshape(-1, 4)
         self.rk, self.res, self.d4 = rk, res, d4
         self.p3, self.d3, self.p4n, self.d4n, self.var = p3, d3, p4n, d4n, var
+        self.flags = None if flags is None else np.asarray(flags, np.int64)
         assert self.base.shape[0] == self.S * self.C * 32
 
     def residual(self, level, nested):
@@ -281,9 +284,19 @@ def lane_vals(p, level, nested=False, G=4):
     if level == 2:
         return q2_value(Sb, sign)
     code, words, dw = p.residual(level, nested)
-    Sr = lane_sums(words, code, G).reshape(S, C, 32, 64)
-    dw = np.asarray(dw, np.int64).reshape(S, C, 1, 1)
-    return fold_value(Sb, Sr, dw & 255, (dw >> 8) & 255, sign)
+    if p.flags is None or level == 3 or nested:
+        Sr = lane_sums(words, code, G).reshape(S, C, 32, 64)
+        dw = np.asarray(dw, np.int64).reshape(S, C, 1, 1)
+        return fold_value(Sb, Sr, dw & 255, (dw >> 8) & 255, sign)
+    on = ((p.flags[:, None] >> np.arange(C)[None]) & 1).astype(bool)            # [S, C]
+    R = int(on[0].sum())
+    assert (on.sum(1) == R).all(), "every strip flags the same number of chunks"
+    rank = np.minimum(np.cumsum(on, 1) - on, R - 1)
+    si = np.arange(S)[:, None] + 0 * rank
+    Sr = lane_sums(words, code, G).reshape(S, R, 32, 64)[si, rank]
+    dw = np.asarray(dw, np.int64).reshape(S, R)[si, rank][..., None, None]
+    q4 = fold_value(Sb, Sr, dw & 255, (dw >> 8) & 255, sign)
+    return np.where(on[..., None, None], q4, q2_value(Sb, sign))
 
 
 def lane_to_rowcol():

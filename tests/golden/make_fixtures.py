@@ -121,6 +121,14 @@ def main():
         e.had_dn = 128
     out["y_lr"] = R.moe_ref(ex, levels, x, sel, rw).numpy()
     np.savez_compressed(os.path.join(OUT, "layer_had512_lr.npz"), **out)
+    # 6. mask mode: nm flagged chunks per strip (here 1 of 3), the residual plane compact over them, flags uniform over each
+    #    group of 8 strips (two groups here); unflagged chunks decode at level 2
+    for rk, var in ((0, False), (7, True)):
+        gen = torch.Generator().manual_seed(2000 + rk)
+        p = R.Proj(256, 384, gen, 1, rk, ("exh", 900 * rk + 5), var=var)
+        W4 = R.dense_W(p, 4, 4, torch.float16)
+        np.savez_compressed(os.path.join(OUT, f"mask_rk{rk}.npz"), seed=2000 + rk, N=256, K=384, nm=1, rk=rk, mbn_offset=900 * rk + 5,
+                            var=int(var), flags=p.flags.numpy(), W4=W4.numpy().view(np.uint16))
     print("fixtures written to", OUT)
 
 

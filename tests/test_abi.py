@@ -55,7 +55,7 @@ def test_validate_row_accepts_supported_rows():
 
 
 @pytest.mark.parametrize("bad,word", [
-    (dict(f0=1), "level"), (dict(f0=5), "level"), (dict(f4=8), "mask mode"), (dict(f8=8), "mask mode"),
+    (dict(f0=1), "level"), (dict(f0=5), "level"), (dict(f0=3, f2=8, f3=8, f6=8, f7=8, f10=10, f11=10, f4=8), "mask mode"), (dict(f0=4, f2=8, f3=8, f6=8, f7=8, f10=11, f11=11, f8=8), "mask mode"),
     (dict(f14=8), "low-rank"), (dict(f16=2), "low-rank"), (dict(f18=512), "in_had_down"), (dict(f19=1), "base code"),
     (dict(f0=4), "residual planes"), (dict(f0=4, f2=8, f3=8, f6=8, f7=8, f10=12), "out of range"),
     (dict(f0=3, f2=8, f3=8, f6=8, f7=8, f10=0, f11=10), "level 3"), (dict(f0=4, f2=8, f3=8, f6=8, f7=8, f10=10), "level 4"),

@@ -135,3 +135,48 @@ def test_bad_arguments_raise():
         M.dequant(row, 0, 100, 128, out=out)
     with pytest.raises(RuntimeError, match="proj"):
         _lib.check(_lib.lib().nq_dequant(row.data_ptr(), 2, 0, 128, 128, out.data_ptr(), None))
+
+
+@pytest.mark.parametrize("rk", [0, 7])
+def test_mask_mode_golden(rk):
+    """mask mode (flags per strip, compact residual plane): the reference's own level-4 dense decode, both projections' row
+    fields; nq_pf_decode takes the same path"""
+    from tests.test_oracle_golden import mask_proj
+    z, p = mask_proj(rk)
+    p.to(DEV)
+    want = z["W4"].view(np.float16)
+    for mode in (0, 1):
+        assert same_f16(gpu_dense(p, 4, p.N, p.K, mode), want) == 0
+        assert same_f16(gpu_dense(p, 2, p.N, p.K, mode), O.dense_W(oracle_plane(p), 2)) == 0
+
+
+def test_mask_mode_layer_decode_and_prefill():
+    """a layer whose experts mix dense and masked residual planes: decode path and prefill against the float64 oracle"""
+    from tests.test_gpu_moe import oracle_layer
+    from tests.util import rel_err
+    H, I, NE = 512, 256, 6
+    ex = [F.Expert(H, I, seed=4100 + i, dev="cpu", nm_gu=(2 if i % 2 else None), nm_dn=(1 if i % 2 else None),
+                   rk_gu=(0, 3, 7, 9, 0, 6)[i], rk_dn=(7, 0, 0, 3, 9, 8)[i], var=(i == 3)) for i in range(NE)]
+    planes = [(oracle_plane(e.gu), oracle_plane(e.dn), False) for e in ex]
+    signs = [e.signs.numpy() for e in ex]
+    levels = [4, 4, 2, 4, 4, 4]
+    for e in ex:
+        e.gu.to(DEV); e.dn.to(DEV); e.signs = e.signs.to(DEV)
+    L = M.MoELayer(NE, H, I, Bmax=4, topk=3)
+    for e in range(NE):
+        L.set(e, ex[e], levels[e])
+    g = torch.Generator().manual_seed(3)
+    for B in (1, 4):
+        sel = torch.stack([torch.randperm(NE, generator=g)[:3] for _ in range(B)]).to(DEV)
+        rw = (torch.rand(B, 3, generator=g) + 0.1).half().to(DEV)
+        x = (torch.randn(B, H, generator=g) * 0.05).half().to(DEV)
+        want = oracle_layer(planes, levels, signs, x, sel, rw)
+        for cg, cd in (([1, 4, 2], [1, 4, 1]), ([1, 2, 4], [1, 4, 2])):
+            y = L(x, sel, rw, cfg_gu=cg, cfg_dn=cd)
+            torch.cuda.synchronize()
+            assert rel_err(y.cpu().numpy(), want) < 5e-5, (B, cg, cd)
+        assert rel_err(L.prefill(x, sel, rw).cpu().numpy(), want) < 5e-5, B
+    # the dense decode used by prefill-with-scratch callers agrees with the oracle bit for bit
+    for e in (1, 3):
+        for proj, pl in ((0, planes[e][0]), (1, planes[e][1])):
+            assert same_f16(M.dense_W(ex[e], proj, 4).cpu().numpy(), O.dense_W(pl, 4)) == 0

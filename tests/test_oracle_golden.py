@@ -149,3 +149,30 @@ def test_had512_and_low_rank_plane_match_reference():
     for n in ("U4g", "U4u", "U4d"):
         lr_no4[0][n] = np.zeros_like(lr[0][n])
     assert np.array_equal(O.moe_forward(dense, levels, sg, x, sel, rw, lr=lambda e: lr_no4[e]), y_l)
+
+
+def mask_proj(rk):
+    """the mask-mode fixture: the projection rebuilt from its seed, and the reference's level-4 dense decode of it"""
+    z = np.load(os.path.join(GOLD, f"mask_rk{rk}.npz"))
+    gen = torch.Generator().manual_seed(int(z["seed"]))
+    p = F.Proj(int(z["N"]), int(z["K"]), gen, int(z["nm"]), rk, ("exh", int(z["mbn_offset"])), var=bool(z["var"]))
+    return z, p
+
+
+@pytest.mark.parametrize("rk", [0, 7])
+def test_mask_mode_matches_reference(rk):
+    """flags per strip, residual plane compact over the flagged chunks, the other chunks at level 2 (sm120/moe.py:134-155)"""
+    z, p = mask_proj(rk)
+    assert np.array_equal(p.flags.numpy(), z["flags"])             # same generator order as the reference's Proj
+    assert p.p4w.shape[0] == p.z["nrec_r"] == 16 * 1 * 32 and p.d4.numel() == 16
+    assert len(set(z["flags"][:8].tolist())) == 1 and len(set(z["flags"][8:].tolist())) == 1   # uniform over 8-strip groups
+    P = oracle_plane(p)
+    W4 = O.dense_W(P, 4)
+    assert same_f16(W4, z["W4"].view(np.float16)) == 0
+    # two of three chunks of every strip stay at level 2, the flagged one differs
+    W2 = O.dense_W(P, 2)
+    on = ((z["flags"][:, None] >> np.arange(3)[None]) & 1).astype(bool)
+    for s_ in (0, 9):
+        for c in range(3):
+            blk = (slice(16 * s_, 16 * s_ + 16), slice(128 * c, 128 * c + 128))
+            assert (same_f16(W4[blk], W2[blk]) == 0) == (not on[s_, c])

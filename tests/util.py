@@ -21,13 +21,14 @@ def u32(t):
 def oracle_plane(p):
     """nestquant_amd.format.Proj -> oracle Plane (host numpy)"""
     nrec = p.z["S"] * p.z["C"] * 32
-    res = O.unpack_words(p.p4.cpu().numpy(), nrec, O.rbits(p.rk))
+    res = O.unpack_words(p.p4.cpu().numpy(), p.z["nrec_r"], O.rbits(p.rk))
     kw = {}
     if p.nested:
         kw = dict(p3=O.unpack_words(p.p3.cpu().numpy(), nrec, 64), d3=u32(p.d3),
                   p4n=O.unpack_words(p.p4n.cpu().numpy(), nrec, 64), d4n=u32(p.d4n))
     return O.Plane(p.N, p.K, u32(p.base).reshape(-1, 4), rk=p.rk, res=res, d4=u32(p.d4),
-                   var=None if p.var is None else p.var.cpu().numpy(), **kw)
+                   var=None if p.var is None else p.var.cpu().numpy(),
+                   flags=None if getattr(p, "flags", None) is None else p.flags.cpu().numpy(), **kw)
 
 
 def same_f16(a, b):
