@@ -31,9 +31,10 @@ const char* nq_last_error(void);
  * {gate|up, down}; replaces rk_codes() / bk_codes() (reference sm120/nqmoe.cu:938-940, sm120/moe.py:246-252). */
 int nq_codes(uint32_t out[4]);
 
-/* Validate one table row held in HOST memory [host]: level, window codes, and that every field this library does not
- * implement (flags, low-rank plane, in_had_down > 128, base codes) is zero. Replaces the asserts of MoELayer.set
- * (reference sm120/moe.py:243-252); an unsupported field is an error, never silently ignored. */
+/* Validate one table row held in HOST memory [host]: level, window codes, mask-mode flags (level 2, or level 4 with a wide
+ * residual plane), low-rank plane (both buffers, ranks 0..4), in_had_down (0, 128, or 512 dividing I), and that the base
+ * codes, which this library does not implement, are 0. Replaces the asserts of MoELayer.set (reference
+ * sm120/moe.py:243-252); an unsupported field is an error, never silently ignored. */
 int nq_validate_row(const int64_t* row_host, int H, int I);
 
 /* Dense decode of one projection (proj 0 = gate|up [2I][H], 1 = down [H][I]) of the expert whose table row is at

@@ -119,7 +119,7 @@ int main(int argc, char** argv)
 
     const int cfg_gu[4] = {1, 4, 12, 0}, cfg_dn[4] = {1, 4, 4, 0};
     const int ny_gu = H / 128 / (cfg_gu[0] * cfg_gu[2]), ny_dn = I / 128 / (cfg_dn[0] * cfg_dn[2]);
-    uint16_t *x, *rw, *h; int64_t* sel; float *out, *acc_gu, *acc_d; int32_t *cnt_gu, *cnt_d, *cnt_h;
+    uint16_t *x, *rw, *h; int64_t* sel; float *out, *acc_gu, *acc_d, *zd; int32_t *cnt_gu, *cnt_d, *cnt_h;
     HIPCHK(hipMalloc(&x, (size_t)B * H * 2)); fill_half<<<64, 256>>>(x, (size_t)B * H, 0x2A66);   // 0.05
     HIPCHK(hipMalloc(&rw, (size_t)S * 2)); fill_half<<<1, 64>>>(rw, S, 0x3000);                    // 0.125
     HIPCHK(hipMalloc(&sel, (size_t)steps * S * 8));
@@ -127,6 +127,7 @@ int main(int argc, char** argv)
     HIPCHK(hipMalloc(&acc_gu, (size_t)ny_gu * S * 2 * I * 4)); HIPCHK(hipMalloc(&acc_d, (size_t)ny_dn * S * H * 4));
     HIPCHK(hipMalloc(&cnt_gu, (size_t)S * (I / 128) * 4)); HIPCHK(hipMalloc(&cnt_d, (size_t)(H / 128) * 4));
     HIPCHK(hipMalloc(&cnt_h, (size_t)S * (I / 128) * 4)); HIPCHK(hipMemset(cnt_h, 0, (size_t)S * (I / 128) * 4));
+    HIPCHK(hipMalloc(&zd, (size_t)S * (I / 128) * 4 * sizeof(float)));
     HIPCHK(hipMemset(cnt_gu, 0, (size_t)S * (I / 128) * 4)); HIPCHK(hipMemset(cnt_d, 0, (size_t)(H / 128) * 4));
     std::vector<int64_t> hsel((size_t)steps * S);
     for (int st = 0; st < steps; ++st)                                        // distinct picks; a step never reuses the previous step's experts
@@ -146,7 +147,7 @@ int main(int argc, char** argv)
     NqMoeArgs a; memset(&a, 0, sizeof a);
     a.x = x; a.rw = rw; a.table = d_table; a.out = out; a.acc_gu = acc_gu; a.h = h; a.acc_d = acc_d; a.cnt_gu = cnt_gu; a.cnt_d = cnt_d;
     a.acc_gu_elems = (int64_t)ny_gu * S * 2 * I; a.acc_d_elems = (int64_t)ny_dn * S * H; a.h_elems = (int64_t)S * I; a.out_elems = (int64_t)B * H;
-    a.cnt_gu_elems = (int64_t)S * (I / 128); a.cnt_d_elems = H / 128; a.cnt_h = cnt_h; a.cnt_h_elems = (int64_t)S * (I / 128); a.zd = acc_d; a.zd_elems = (int64_t)S * (I / 128) * 4;   /* no low-rank planes here: never touched */
+    a.cnt_gu_elems = (int64_t)S * (I / 128); a.cnt_d_elems = H / 128; a.cnt_h = cnt_h; a.cnt_h_elems = (int64_t)S * (I / 128); a.zd = zd; a.zd_elems = (int64_t)S * (I / 128) * 4;
     a.B = B; a.topk = topk; a.E = E; a.H = H; a.I = I; a.which = 3;
     memcpy(a.cfg_gu, cfg_gu, sizeof cfg_gu); memcpy(a.cfg_dn, cfg_dn, sizeof cfg_dn);
     hipEvent_t e0, e1; HIPCHK(hipEventCreate(&e0)); HIPCHK(hipEventCreate(&e1));

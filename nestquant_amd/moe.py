@@ -49,8 +49,8 @@ def entry(ex, level):
             e[off + 1] = slot.data_ptr()
             e[off + 2] = (p.d3 if level == 3 else p.d4n).data_ptr()
         else:
-            e[off + 1] = p.p4.data_ptr()
-            e[off + 2] = p.d4.data_ptr()
+            e[off + 1] = 0 if p.p4 is None else p.p4.data_ptr()      # None: resident-only expert, a record slot supplies them
+            e[off + 2] = 0 if p.d4 is None else p.d4.data_ptr()
         if getattr(p, "flags", None) is not None:
             e[off + 3] = p.flags.data_ptr()
     e[9] = ex.signs.data_ptr()

@@ -1,0 +1,73 @@
+"""A layer served from the on-disk formats (resident file + level-4 records in a slot pool, promoted through the mailbox)
+gives bitwise the outputs of the same experts set into a layer directly, in the decode path and in prefill."""
+import types
+
+import pytest
+import torch
+
+from nestquant_amd import format as F, moe as M, p4rec, resident
+from tests.test_formats import _lr_expert, _rank_layer
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def test_layer_from_resident_file_and_record_slots(tmp_path):
+    H, I, E, topk, B = 256, 512, 6, 3, 4
+    ranks = [(0, 0), (2, 1), (4, 4), (1, 0), (0, 3), (2, 2)]
+    exs = [_lr_expert(H, I, 40 + e, *ranks[e], rk=(3, 9)) for e in range(E)]
+    exs[0].lr = exs[0].lr4 = None
+    levels = [2, 4, 4, 2, 4, 0]
+    for x in exs:
+        x.gu.to(DEV); x.dn.to(DEV); x.signs = x.signs.to(DEV); x.sc = {k: v.to(DEV) for k, v in x.sc.items()}
+        x.lr, x.lr4 = (None, None) if x.lr is None else (x.lr.to(DEV), x.lr4.to(DEV))
+        x.had_dn = 512
+
+    # direct layer: rows straight from the experts' own tensors (level-4 rows with the level-4 scale vector)
+    direct = M.MoELayer(E, H, I, Bmax=B, topk=topk)
+    for e in range(E):
+        row = M.entry(exs[e], levels[e])
+        if levels[e] == 4:
+            row[9] = exs[e].sc[4].data_ptr()
+        M.validate_row(row, H, I)
+        direct.table[e].copy_(row.to(DEV))
+
+    # served layer: resident file -> level-2 rows; records -> pinned staging -> slots on a side stream -> mailbox
+    path = str(tmp_path / "L7.pt")
+    resident.save(_rank_layer(exs[:5], list(range(5)), H, I, had_dn=512), path)          # expert 5 is absent (level 0)
+    got, h, i = resident.load(path, DEV)
+    assert (h, i) == (H, I)
+    lay = p4rec.layout(exs[1], H, I)
+    served = M.MoELayer(E, H, I, Bmax=B, topk=topk)
+    for e in range(5):
+        served.set(e, got[e], 2)
+    mb = M.Mailbox(served)
+    pool = torch.zeros(3, lay["rec_bytes"], dtype=torch.uint8, device=DEV)
+    stage = torch.empty(3, lay["rec_bytes"], dtype=torch.uint8).pin_memory()
+    side = torch.cuda.Stream()
+    for slot, e in enumerate(e for e in range(5) if levels[e] == 4):
+        p4rec.pack_into(exs[e], lay, stage[slot])
+        with torch.cuda.stream(side):
+            pool[slot].copy_(stage[slot], non_blocking=True)
+        mb.post(e, p4rec.row(got[e], lay, pool[slot].data_ptr(), M.entry), side)
+    side.synchronize()
+
+    g = torch.Generator().manual_seed(9)
+    x = (torch.randn(B, H, generator=g) * 0.5).half().to(DEV)
+    sel = torch.stack([torch.randperm(E, generator=g)[:topk] for _ in range(B)]).to(DEV)
+    rw = torch.softmax(torch.randn(B, topk, generator=g), -1).half().to(DEV)
+    mb.apply()
+    y = served(x, sel, rw).clone()
+    want = direct(x, sel, rw).clone()
+    torch.cuda.synchronize()
+    assert all(mb.done(e) for e in range(E))
+    assert [int(v) for v in served.table[:, 0].cpu()] == levels
+    assert torch.isfinite(want).all() and want.abs().max() > 0
+    assert torch.equal(y, want)
+    # level 2 everywhere differs (the records matter), and prefill agrees bitwise too
+    assert not torch.equal(served(x, sel, rw, force_level=2), want)
+    T = 40
+    xt = (torch.randn(T, H, generator=g) * 0.5).half().to(DEV)
+    st = torch.stack([torch.randperm(E, generator=g)[:topk] for _ in range(T)]).to(DEV)
+    wt = torch.softmax(torch.randn(T, topk, generator=g), -1).half().to(DEV)
+    assert torch.equal(served.prefill(xt, st, wt), direct.prefill(xt, st, wt))
