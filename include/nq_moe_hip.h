@@ -98,6 +98,15 @@ int nq_moe_forward(const NqMoeArgs* args, void* stream);
 int nq_mailbox(int64_t* table, const int64_t* stage, const int32_t* seq, int32_t* applied, int32_t* applied_host, int E,
                void* stream);
 
+/* Decode salience export: acc[e] += sum over the picks (t, k) with ids[t][k] == e of (rsf * w[t][k])^2 * sum_i x[t][i]^2, for
+ * T <= 8 tokens of K <= 8 picks; acc fp64 [E] on the device, every touched entry also stored to host [host-mapped fp64 [E]].
+ * x [T][H] with row stride x_row_stride elements, NQ_DT_F16 / NQ_DT_BF16 (or NQ_DT_F32, rounded through fp16); w [T][K]
+ * likewise (rounded through fp16); ids NQ_DT_I64 / NQ_DT_I32. Picks with w == 0 or an id outside [0, E) are skipped. fp32
+ * sums in the reference kernel's order, so the exported values are the same bits. Calls on one layer must be stream-ordered
+ * (acc is updated without atomics). Replaces sal (reference sm120/nqsal.cu:19-78, called at sm120/serve/nq_vllm.py:558,572). */
+int nq_sal(const void* x, int x_dtype, int64_t x_row_stride, const void* w, int w_dtype, const void* ids, int ids_dtype, int T,
+           int H, int K, int E, double rsf, double* acc, double* host, void* stream);
+
 /* ---- prefill (more tokens than a decode call takes): pairs (token, expert) sorted by expert ------------------------------
  * pt / pe: int32[np] token and expert of each pair. Pairs whose expert is at level <= 0,
  * outside [0, E), or whose weight is 0 contribute nothing. Activation buffers xg, xu [np][H] and h [np][I] are fp16 with

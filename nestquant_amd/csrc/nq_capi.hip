@@ -75,6 +75,18 @@ extern "C" int nq_pf_decode(const int64_t* table, const int32_t* experts, int G,
     return launch_pf_decode(table, experts, G, Wgu, Wdn, H, I, (hipStream_t)stream);
 }
 
+extern "C" int nq_sal(const void* x, int x_dtype, int64_t x_row_stride, const void* w, int w_dtype, const void* ids, int ids_dtype,
+                      int T, int H, int K, int E, double rsf, double* acc, double* host, void* stream)
+{
+    NQ_REQUIRE(T >= 0 && T <= 8 && K >= 1 && K <= 8, "nq_sal: T=%d K=%d (at most 8 tokens of at most 8 picks)", T, K);
+    if (T == 0) return 0;
+    NQ_REQUIRE(x && w && ids && acc && host, "nq_sal: null pointer");
+    NQ_REQUIRE(H >= 1 && E >= 1 && x_row_stride >= H, "nq_sal: H=%d E=%d row stride %lld", H, E, (long long)x_row_stride);
+    NQ_REQUIRE(x_dtype >= 0 && x_dtype <= 2 && w_dtype >= 0 && w_dtype <= 2 && ids_dtype >= 0 && ids_dtype <= 1,
+               "nq_sal: dtype codes x=%d w=%d ids=%d", x_dtype, w_dtype, ids_dtype);
+    return launch_sal(x, x_dtype, x_row_stride, w, w_dtype, ids, ids_dtype, T, H, K, E, (float)rsf, acc, host, (hipStream_t)stream);
+}
+
 extern "C" int nq_moe_forward(const NqMoeArgs* p, void* stream)
 {
     NQ_REQUIRE(p, "nq_moe_forward: null args");

@@ -334,17 +334,21 @@ MoELayer.prefill = prefill
 PF_MIN = 384         # tokens from which a step goes through prefill() (reference NQ_PF_MIN, sm120/serve/nq_vllm.py:187)
 
 
-def forward(layer, mailbox, x, topk_weights, topk_ids, pf_min=PF_MIN):
+def forward(layer, mailbox, x, topk_weights, topk_ids, pf_min=PF_MIN, sal=None):
     """One MoE layer step as the reference's serving caller runs it (sm120/serve/nq_vllm.py:520-574): apply the mailbox,
     then up to Bmax tokens in one decode call, pf_min tokens or more through prefill() (never under graph capture), anything
     between in slices of Bmax tokens. x [T, H] in fp16 / bf16 / fp32, weights [T, topk] likewise, ids int64 / int32;
-    returns [T, H] in x's dtype. The decode calls read the caller's dtypes and write the result dtype themselves."""
+    returns [T, H] in x's dtype. The decode calls read the caller's dtypes and write the result dtype themselves. `sal`: an
+    optional salience.Salience, fed by the decode steps as the reference does (every step of up to Bmax tokens, the slices of
+    a step of up to 16 tokens; longer steps count as prefill and are left out)."""
     T = x.shape[0]
     x, w, ids = x.contiguous(), topk_weights.contiguous(), topk_ids.contiguous()
     if mailbox is not None:
         mailbox.apply()
     odt = x.dtype if x.dtype in _DT_OUT else torch.float32
     if T <= layer.Bmax:
+        if sal is not None and T:
+            sal(x, w, ids)
         return layer(x, ids, w, out=torch.empty(T, layer.H, dtype=odt, device=x.device))
     if T >= pf_min and not torch.cuda.is_current_stream_capturing():
         return layer.prefill(x.half(), ids.long(), w.half()).to(x.dtype)
@@ -352,6 +356,8 @@ def forward(layer, mailbox, x, topk_weights, topk_ids, pf_min=PF_MIN):
     for i in range(0, T, layer.Bmax):
         j = min(T, i + layer.Bmax)
         layer(x[i:j], ids[i:j], w[i:j], out=out[i:j])
+        if sal is not None and T <= 16:
+            sal(x[i:j], w[i:j], ids[i:j])
     return out
 
 
