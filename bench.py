@@ -361,7 +361,7 @@ def main():
     kdt = e0.elapsed_time(e1) / 1e3 / (nrep * R)
     kbytes = sum(code_bytes(ex, levels, routes[i][2], "gu") for i in range(R)) / R
     achieved = kbytes / kdt / 1e9
-    roofline = dict(bound="hbm", kernel="nq_gemv_k<0> (gate|up decode+GEMV)", achieved=round(achieved, 1), peak=HBM_PEAK_GBS, unit="GB/s",
+    roofline = dict(bound="hbm", kernel="nq_gemv_k<0, false> (gate|up decode+GEMV)", achieved=round(achieved, 1), peak=HBM_PEAK_GBS, unit="GB/s",
                     frac=round(achieved / HBM_PEAK_GBS, 4), traffic=int(kbytes * TRAFFIC_RATIO), us_per_launch=round(kdt * 1e6, 2),
                     algorithmic_bytes_per_launch=int(kbytes))
     cpu = None

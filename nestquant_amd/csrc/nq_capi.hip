@@ -23,7 +23,7 @@ extern "C" int nq_codes(uint32_t out[4])
 {
     NQ_REQUIRE(out, "nq_codes: null output");
     out[0] = out[1] = (1u << NCODES) - 1u;   // residual codes 0..11 in both kernels
-    out[2] = out[3] = 1u;                     // base code 0 (K = 2 ring base) only
+    out[2] = out[3] = 3u;                     // base codes 0 (K = 2 ring base) and 1 (K = 1.75, sub-array layout)
     return 0;
 }
 
@@ -39,7 +39,7 @@ extern "C" int nq_validate_row(const int64_t* r, int H, int I)
     NQ_REQUIRE(r[14] ? (r[15] != 0 && r[16] >= 0 && r[16] <= 4 && r[17] >= 0 && r[17] <= 4 && r[16] + r[17] > 0) : (r[15] == 0 && r[16] == 0 && r[17] == 0),
                "table row: low-rank plane needs both buffers and ranks r_gu, r_dn in [0, 4] (got %lld, %lld)", (long long)r[16], (long long)r[17]);
     NQ_REQUIRE(r[18] == 0 || r[18] == 128 || (r[18] == 512 && I % 512 == 0), "table row: in_had_down %lld must be 0, 128, or 512 dividing I = %d", (long long)r[18], I);
-    NQ_REQUIRE(r[19] == 0, "table row: base code %lld is not implemented (K=2 ring base only)", (long long)r[19]);
+    NQ_REQUIRE((r[19] & ~0x0101ll) == 0, "table row: base codes 0x%llx (gate|up | down << 8): only 0 (K=2) and 1 (K=1.75) are implemented", (long long)r[19]);
     if (lv >= 3)
     {
         NQ_REQUIRE(r[2] && r[3] && r[6] && r[7], "table row: level %lld needs residual planes and block words", (long long)lv);
@@ -122,6 +122,8 @@ extern "C" int nq_moe_forward(const NqMoeArgs* p, void* stream)
     a.cnt_h = p->cnt_h;
     NQ_REQUIRE(p->zd && p->zd_elems >= S * (p->I / 128) * 4, "workspace too small: zd");
     a.zd = (float*)p->zd;
+    NQ_REQUIRE((p->base_codes & ~3) == 0, "nq_moe_forward: base_codes=%d (bits 0 and 1 only)", p->base_codes);
+    a.base_codes = p->base_codes;
     return launch_moe(a, p->cfg_gu, p->cfg_dn, p->which, (hipStream_t)stream);
 }
 

@@ -197,10 +197,11 @@ __device__ __forceinline__ uint32_t pk_fma(uint32_t h, uint32_t a, uint32_t c)
 // ---- pair decode ----------------------------------------------------------------------------------------------------
 // fp16 pair (1024 + S or 1024 + F) of lane weights JA (low half) and JB (high half); exact integers in fp16.
 // RES = false: base only. wb: extended base record (6 words); wr: extended residual record.
-template <bool RES, int CODE, int JA, int JB>
+// BK = window code of the base plane (0: two bits per step; 1: the 1.75-bit pattern), wb extended accordingly.
+template <bool RES, int CODE, int JA, int JB, int BK = 0>
 __device__ __forceinline__ uint32_t code_pair(const uint32_t* wb, const uint32_t* wr, const FoldK& k)
 {
-    const uint32_t xa = hash_at<2 * JA>(wb), xb = hash_at<2 * JB>(wb);
+    const uint32_t xa = hash_at<Rec<BK>::off(JA)>(wb), xb = hash_at<Rec<BK>::off(JB)>(wb);
     if constexpr (!RES)
     {
         const uint32_t t = __builtin_amdgcn_sad_u8(xa, 0u, 0x64006400u);
@@ -216,19 +217,43 @@ __device__ __forceinline__ uint32_t code_pair(const uint32_t* wb, const uint32_t
     }
 }
 // decoded fp16 weight pair (bit-exact values)
-template <bool RES, int CODE, int JA, int JB>
+template <bool RES, int CODE, int JA, int JB, int BK = 0>
 __device__ __forceinline__ uint32_t weight_pair(const uint32_t* wb, const uint32_t* wr, const FoldK& k)
 {
-    return pk_fma(code_pair<RES, CODE, JA, JB>(wb, wr, k), k.A2, k.C2);
+    return pk_fma(code_pair<RES, CODE, JA, JB, BK>(wb, wr, k), k.A2, k.C2);
 }
 
 // ---- table row ------------------------------------------------------------------------------------------------------
 // int64[20] per expert (reference sm120/moe.py:216-229, sm120/nqmoe.cu:26-45):
 //   [0] level 0/2/3/4  [1..4] gate|up base, residual plane, block words, flags (mask mode, 0 = dense)  [5..8] down  [9] sign/scale vector
-//   [10],[11] residual window code of gate|up, down  [12],[13] sign-variant planes  [14..17] low-rank plane (unsupported)
-//   [18] in_had_down (unsupported unless 0/128)  [19] base codes (unsupported unless 0)
+//   [10],[11] residual window code of gate|up, down  [12],[13] sign-variant planes  [14..17] low-rank plane (buffers, ranks)
+//   [18] in_had_down (0 / 128 / 512)  [19] base window codes, gate|up | down << 8 (0 or 1)
+template <int C> struct CodeTag { static constexpr int value = C; };
 typedef const NQ_GLOBAL uint64_t* gp_u64;
-struct Planes { gp_u4 base; gp_u8 res; gp_u32 dw; gp_u8 var; int code; gp_u64 flags; };
+struct Planes { gp_u4 base; gp_u8 res; gp_u32 dw; gp_u8 var; int code; gp_u64 flags; int bcode; };
+
+// Base record of a lane: code 0 = one uint4 per record; other codes = the residual plane's sub-array layout at
+// Rec<BK>::BITS bits per record (reference sm120/NQ_RES_V2.md:38-46), at most 128 bits.
+template <int BK>
+__device__ __forceinline__ u32x4 load_base(const Planes& P, size_t rec, size_t nrec)
+{
+    if constexpr (BK == 0) return P.base[rec];
+    else
+    {
+        static_assert(Rec<BK>::BITS <= 128, "base records are at most four words");
+        uint32_t w[4] = {0u, 0u, 0u, 0u};
+        load_record<BK>(w, (gp_u8)P.base, rec, nrec);
+        return u32x4{w[0], w[1], w[2], w[3]};
+    }
+}
+// wb[0..3] = the record's words -> wb[0..5] = the record followed by the ring neighbour's first word `nb`
+template <int BK>
+__device__ __forceinline__ void ext_base(uint32_t* wb, uint32_t nb) { ext_words<Rec<BK>::BITS, Rec<BK>::NW>(wb, nb); }
+template <class F>
+__device__ __forceinline__ void dispatch_base(int bcode, F&& f)
+{
+    if (bcode == 1) f(CodeTag<1>{}); else f(CodeTag<0>{});
+}
 
 // Mask mode (reference sm120/nqmoe.cu:22-24,202-206): flags = one uint64 per strip, bit c = chunk c is refined; the residual
 // plane and its block words are compact over the nm = popcount(flags) refined chunks of every strip, in chunk order, and
@@ -245,11 +270,11 @@ __device__ __forceinline__ Planes planes_of(const int64_t* ent, int mode)
     Planes P;
     P.base = (gp_u4)ent[o]; P.res = (gp_u8)ent[o + 1]; P.dw = (gp_u32)ent[o + 2];
     P.var = (gp_u8)ent[mode == 0 ? 12 : 13]; P.code = (int)ent[10 + mode]; P.flags = (gp_u64)ent[o + 3];
+    P.bcode = (int)((ent[19] >> (8 * mode)) & 0xFF);
     return P;
 }
 
 // compile-time dispatch over the residual code; F is a generic lambda taking std::integral_constant<int, CODE>
-template <int C> struct CodeTag { static constexpr int value = C; };
 template <class F>
 __device__ __forceinline__ void dispatch_code(int code, F&& f)
 {

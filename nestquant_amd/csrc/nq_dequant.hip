@@ -10,7 +10,7 @@ namespace nq {
 
 constexpr int TS = 68;                        // LDS tile row stride in 32-bit words (64 + 4: conflict-free pair stores)
 
-template <bool RES, int CODE>
+template <bool RES, int CODE, int BK>
 __device__ __forceinline__ void decode_to_tile(const uint32_t* wb, const uint32_t* wr, const FoldK& k, uint32_t* tile, int lane32)
 {
     const int g = lane32 >> 2, t4 = lane32 & 3;
@@ -21,10 +21,10 @@ __device__ __forceinline__ void decode_to_tile(const uint32_t* wb, const uint32_
         // a switch keeps every window offset a compile-time constant while t stays a loop variable
         switch (t)
         {
-#define NQ_T(T) case T: a[0] = weight_pair<RES, CODE, 8 * T + 0, 8 * T + 1>(wb, wr, k); \
-                        a[1] = weight_pair<RES, CODE, 8 * T + 2, 8 * T + 3>(wb, wr, k); \
-                        a[2] = weight_pair<RES, CODE, 8 * T + 4, 8 * T + 5>(wb, wr, k); \
-                        a[3] = weight_pair<RES, CODE, 8 * T + 6, 8 * T + 7>(wb, wr, k); break;
+#define NQ_T(T) case T: a[0] = weight_pair<RES, CODE, 8 * T + 0, 8 * T + 1, BK>(wb, wr, k); \
+                        a[1] = weight_pair<RES, CODE, 8 * T + 2, 8 * T + 3, BK>(wb, wr, k); \
+                        a[2] = weight_pair<RES, CODE, 8 * T + 4, 8 * T + 5, BK>(wb, wr, k); \
+                        a[3] = weight_pair<RES, CODE, 8 * T + 6, 8 * T + 7, BK>(wb, wr, k); break;
             NQ_T(0) NQ_T(1) NQ_T(2) NQ_T(3) NQ_T(4) NQ_T(5) NQ_T(6) default: NQ_T(7)
 #undef NQ_T
         }
@@ -35,15 +35,23 @@ __device__ __forceinline__ void decode_to_tile(const uint32_t* wb, const uint32_
 }
 
 // decode unit `unit` of projection planes P (level lv) into tile; all 64 lanes of the wave call this together
+template <int BK>
+__device__ __forceinline__ void decode_unit_bk(const Planes& P, int lv, size_t unit, size_t nrec, int C, uint32_t* tile, int lane);
 __device__ __forceinline__ void decode_unit(const Planes& P, int lv, size_t unit, size_t nrec, int C, uint32_t* tile, int lane)
+{
+    dispatch_base(P.bcode, [&](auto bk) { decode_unit_bk<decltype(bk)::value>(P, lv, unit, nrec, C, tile, lane); });
+}
+
+template <int BK>
+__device__ __forceinline__ void decode_unit_bk(const Planes& P, int lv, size_t unit, size_t nrec, int C, uint32_t* tile, int lane)
 {
     const int lane32 = lane & 31;
     const int src = (lane & ~3) | ((lane + 1) & 3);           // next lane of the ring
     uint32_t wb[6];
     {
-        const u32x4 v = P.base[unit * 32 + lane32];
+        const u32x4 v = load_base<BK>(P, unit * 32 + lane32, nrec);
         wb[0] = v.x; wb[1] = v.y; wb[2] = v.z; wb[3] = v.w;
-        ext_words<128, 4>(wb, __shfl(wb[0], src));
+        ext_base<BK>(wb, __shfl(wb[0], src));
     }
     const uint32_t sgm = P.var ? (((uint32_t)P.var[unit] >> (lane32 >> 2)) & 1u) * 0x80008000u : 0u;
     size_t runit = unit, rnrec = nrec;                          // residual unit / records: compact in mask mode
@@ -57,7 +65,7 @@ __device__ __forceinline__ void decode_unit(const Planes& P, int lv, size_t unit
     }
     if (!on)
     {
-        decode_to_tile<false, 0>(wb, wb, consts_l2(sgm), tile, lane32);
+        decode_to_tile<false, 0, BK>(wb, wb, consts_l2(sgm), tile, lane32);
         return;
     }
     const uint32_t dw = P.dw[runit];
@@ -67,7 +75,7 @@ __device__ __forceinline__ void decode_unit(const Planes& P, int lv, size_t unit
         uint32_t wr[Rec<CODE>::NW + 2];
         load_record<CODE>(wr, P.res, runit * 32 + lane32, rnrec);
         ext_words<Rec<CODE>::BITS, Rec<CODE>::NW>(wr, __shfl(wr[0], src));
-        decode_to_tile<true, CODE>(wb, wr, k, tile, lane32);
+        decode_to_tile<true, CODE, BK>(wb, wr, k, tile, lane32);
     });
 }
 

@@ -1,13 +1,13 @@
 // Decode-path MoE layer for 1..8 tokens (reference sm120/nqmoe.cu:375-449 route, :493-771 do_item, :858-907 moe_forward,
 // :908-929 mailbox). Two launches on one stream, every routing / level / pointer decision read on the device:
 //
-//   nq_gemv_k<0>  gate|up: grid (strip-pair blocks, k-slices, runs). A run = one distinct routed expert + the tokens that
+//   nq_gemv_k<0, *>  gate|up: grid (strip-pair blocks, k-slices, runs). A run = one distinct routed expert + the tokens that
 //                 picked it. The block rotates those tokens' x (x * su -> Hadamard-128 -> fp16) into LDS, then every
 //                 wavefront decodes the records of two strips chunk by chunk straight into MFMA A operands
 //                 (v_mfma_f32_16x16x32_f16, tokens as the N dimension) and writes its k-slice partial sums. The block
 //                 that arrives last at a (run, 128-column group) counter sums the partials and finishes them:
 //                 Hadamard * sv, SwiGLU, * su_d, Hadamard -> h fp16.
-//   nq_gemv_k<1>  down: same kernel on h; the last block of a 128-row output group (counter over all runs) combines:
+//   nq_gemv_k<1, *>  down: same kernel on h; the last block of a 128-row output group (counter over all runs) combines:
 //                 out[b] = sum_k rw[b,k] * sv_o (.) Hadamard(sum of partials).
 //
 // Lane mapping of the GEMV (wave64): lane = 16 * t4 + 8 * ss + g decodes the record of lane (4 g + t4) of unit
@@ -134,7 +134,7 @@ __device__ __forceinline__ void route(const MoeArgs& a, int z, RunInfo* R, int l
 {
     const int S = a.B * a.topk;
     int e = -1, lv = 0; bool ok = false;
-    int64_t f_base = 0, f_res = 0, f_dw = 0, f_var = 0, f_code = 0, f_signs = 0, f_had = 0, f_lr = 0, f_lr4 = 0, f_rg = 0, f_rd = 0, f_flags = 0;
+    int64_t f_base = 0, f_res = 0, f_dw = 0, f_var = 0, f_code = 0, f_signs = 0, f_had = 0, f_lr = 0, f_lr4 = 0, f_rg = 0, f_rd = 0, f_flags = 0, f_bk = 0;
     if (lane < S)
     {
         const long long ee = sel_at(a, lane);
@@ -145,7 +145,7 @@ __device__ __forceinline__ void route(const MoeArgs& a, int z, RunInfo* R, int l
             constexpr int o = MODE == 0 ? 1 : 5;
             lv = (int)ent[0];
             f_base = ent[o]; f_res = ent[o + 1]; f_dw = ent[o + 2]; f_var = ent[MODE == 0 ? 12 : 13]; f_code = ent[10 + MODE]; f_signs = ent[9]; f_had = ent[18];
-            f_lr = ent[14]; f_lr4 = ent[15]; f_rg = ent[16]; f_rd = ent[17]; f_flags = ent[o + 3];
+            f_lr = ent[14]; f_lr4 = ent[15]; f_rg = ent[16]; f_rd = ent[17]; f_flags = ent[o + 3]; f_bk = ent[19];
             ok = rw_at(a, lane) != 0.f && lv > 0;
         }
     }
@@ -168,6 +168,7 @@ __device__ __forceinline__ void route(const MoeArgs& a, int z, RunInfo* R, int l
             {
                 Planes P;
                 P.base = (gp_u4)f_base; P.res = (gp_u8)f_res; P.dw = (gp_u32)f_dw; P.var = (gp_u8)f_var; P.code = (int)f_code; P.flags = (gp_u64)f_flags;
+                P.bcode = (int)((f_bk >> (8 * MODE)) & 0xFF);
                 R->P = P; R->signs = (const _Float16*)f_signs;
                 R->level = a.force_level ? a.force_level : lv;
                 R->had = f_had == 512 ? 512 : 128;
@@ -372,8 +373,12 @@ __device__ __forceinline__ uint64_t uni(uint64_t v)
 // MODE 0: gate|up (N = 2I, K = H, input x rotated here). MODE 1: down (N = H, K = I, input h).
 // grid (N / 32 / SB, C / NC, S); block 64 * SB threads (SB = 1, 2 or 4: a block covers at most one 128-row group);
 // dynamic LDS = rows * (NC * 256 + 16) + 256 bytes (>= SB * 512 for the combine), one row per token of the call
-template <int MODE>
-__global__ void __launch_bounds__(256) nq_gemv_k(MoeArgs a, int NC)
+// ANYBK = false: the kernel of a layer whose rows all have base window code 0 (the host says so, MoeArgs::base_codes == 1).
+// A run whose row nevertheless names another base code is not decoded as if it were code 0: its partial sums are NaN, so
+// every token that picked it comes out NaN. ANYBK = true also carries the decode loops of the other base codes, which
+// cost registers the common kernel does not have to pay for.
+template <int MODE, bool ANYBK>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) nq_gemv_k(MoeArgs a, int NC)
 {
     extern __shared__ __align__(16) char smem[];
     __shared__ RunInfo R;
@@ -406,12 +411,16 @@ __global__ void __launch_bounds__(256) nq_gemv_k(MoeArgs a, int NC)
     Planes P;                                                    // block-uniform: keep the plane addresses in scalar registers
     P.base = (gp_u4)uni((uint64_t)R.P.base); P.res = (gp_u8)uni((uint64_t)R.P.res); P.dw = (gp_u32)uni((uint64_t)R.P.dw);
     P.var = (gp_u8)uni((uint64_t)R.P.var); P.code = __builtin_amdgcn_readfirstlane(R.P.code); P.flags = (gp_u64)uni((uint64_t)R.P.flags);
+    P.bcode = __builtin_amdgcn_readfirstlane(R.P.bcode);
     LaneCtx L;
     L.unit0 = (size_t)strip * C + chunk0; L.rec0 = L.unit0 * 32 + 4 * g + t4;
     L.nrec = (size_t)(N / 16) * C * 32;
     L.src = (lane + 16) & 63; L.g = g; L.strip = (size_t)strip; L.nstrips = (size_t)(N / 16); L.chunk0 = chunk0;
     L.xs = (n < ntok ? smem + n * rowstride : zero) + t4 * 16; L.xstep = n < ntok ? 256 : 0;
-    const u32x4 nb0 = P.base[L.rec0];
+    const bool foreign = !ANYBK && P.bcode != 0;                  // block-uniform; a smaller plane is not read as 128-bit records
+    u32x4 nb0 = {0u, 0u, 0u, 0u};
+    if constexpr (ANYBK) { if (P.bcode == 1) nb0 = load_base<1>(P, L.rec0, L.nrec); else nb0 = P.base[L.rec0]; }
+    else if (!foreign) nb0 = P.base[L.rec0];
 
     // ---- stage the run's tokens for this k-slice in B-operand order
     if constexpr (MODE == 0)
@@ -460,7 +469,18 @@ __global__ void __launch_bounds__(256) nq_gemv_k(MoeArgs a, int NC)
 
     // ---- decode + MFMA over the k-slice
     float4_t acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
-    if (R.level == 2) gemv_chunks<false, 0>(P, L, NC, acc, nb0);
+    if constexpr (ANYBK)
+        dispatch_base(P.bcode, [&](auto bk) {
+            constexpr int BK = decltype(bk)::value;
+            if (R.level == 2) gemv_chunks<false, 0, BK>(P, L, NC, acc, nb0);
+            else dispatch_code(P.code, [&](auto tag) { gemv_chunks<true, decltype(tag)::value, BK>(P, L, NC, acc, nb0); });
+        });
+    else if (foreign)
+    {
+        const float nan = __builtin_nanf("");
+        acc[0] = float4_t{nan, nan, nan, nan}; acc[1] = acc[0];
+    }
+    else if (R.level == 2) gemv_chunks<false, 0>(P, L, NC, acc, nb0);
     else dispatch_code(P.code, [&](auto tag) { gemv_chunks<true, decltype(tag)::value>(P, L, NC, acc, nb0); });
 
     // ---- k-slice partial sums: lane (t4, n) holds rows 16 (strip0 + t4 / 2) + 4 (t4 & 1) + i (+ 8 for acc[1]) of token n
@@ -515,7 +535,8 @@ int launch_moe(const MoeArgs& a, const int* cfg_gu, const int* cfg_dn, int which
         const int N = mode == 0 ? 2 * a.I : a.H, K = mode == 0 ? a.H : a.I, C = K / 128;
         const int NX = N / 32 / SB, NY = C / NC;
         const int shm = std::max(a.B * (NC * 256 + 16) + 256, SB * 512);
-        auto kern = mode == 0 ? nq_gemv_k<0> : nq_gemv_k<1>;
+        const bool anybk = a.base_codes != 1;                      // 1 = every live row has base code 0; anything else: both paths
+        auto kern = mode == 0 ? (anybk ? nq_gemv_k<0, true> : nq_gemv_k<0, false>) : (anybk ? nq_gemv_k<1, true> : nq_gemv_k<1, false>);
         if (shm > 48 * 1024)
         {
             hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, shm);

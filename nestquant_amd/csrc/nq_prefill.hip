@@ -253,15 +253,17 @@ struct PfGemm
 };
 
 // body for one (RES, CODE): all K / 128 chunks of this wave's two strips against the tile's tokens
-template <int TG, bool RES, int CODE, bool MASKED>
+template <int TG, bool RES, int CODE, bool MASKED, int BK = 0>
 __device__ __forceinline__ void pf_chunks(const Planes& P, const LaneCtx& L, int C, const _Float16* A, int K, int row0, int nrows,
                                           char* smem, float4_t (*acc)[2])
 {
     constexpr int NW = RES ? Rec<CODE>::NW : 1;
-    u32x4 nb = P.base[L.rec0];
+    u32x4 nb = load_base<BK>(P, L.rec0, L.nrec);
     uint32_t nr[NW + 2] = {0}, ndw = 0, nvar = 0;
     constexpr bool masked = RES && MASKED;                       // the kernel variant for experts in mask mode
-    const uint64_t mflags = masked ? P.flags[L.strip] : 0ull;
+    // an expert without flags that comes through this variant (base code other than 0) reads as "every chunk refined",
+    // for which the compact residual indexing is the dense one
+    const uint64_t mflags = masked ? (P.flags ? P.flags[L.strip] : (C >= 64 ? ~0ull : (1ull << C) - 1ull)) : 0ull;
     if constexpr (RES && !masked) { load_record<CODE>(nr, P.res, L.rec0, L.nrec); ndw = P.dw[L.unit0]; }
     if (P.var) nvar = P.var[L.unit0];
     const int lane = threadIdx.x & 63, warp = threadIdx.x >> 6, t4 = lane >> 4, n = lane & 15;
@@ -304,11 +306,11 @@ __device__ __forceinline__ void pf_chunks(const Planes& P, const LaneCtx& L, int
             }
         if (c + 1 < C)
         {
-            nb = P.base[L.rec0 + (size_t)(c + 1) * 32];
+            nb = load_base<BK>(P, L.rec0 + (size_t)(c + 1) * 32, L.nrec);
             if constexpr (RES && !masked) { load_record<CODE>(nr, P.res, L.rec0 + (size_t)(c + 1) * 32, L.nrec); ndw = P.dw[L.unit0 + c + 1]; }
             if (P.var) nvar = P.var[L.unit0 + c + 1];
         }
-        ext_words<128, 4>(wb, __shfl(wb[0], L.src));
+        ext_base<BK>(wb, __shfl(wb[0], L.src));
         const uint32_t sgm = ((var >> L.g) & 1u) * 0x80008000u;
         half8_t aop[4][2];
         if (RES && (!masked || on))
@@ -319,8 +321,8 @@ __device__ __forceinline__ void pf_chunks(const Planes& P, const LaneCtx& L, int
                 const FoldK k = consts_fold(dw, sgm);
                 static_for<4>([&](auto mm) {
                     constexpr int MM = decltype(mm)::value;
-                    aop[MM][0] = a_operand<RES, CODE, MM, 0>(wb, wr, k);
-                    aop[MM][1] = a_operand<RES, CODE, MM, 1>(wb, wr, k);
+                    aop[MM][0] = a_operand<RES, CODE, MM, 0, BK>(wb, wr, k);
+                    aop[MM][1] = a_operand<RES, CODE, MM, 1, BK>(wb, wr, k);
                 });
             }
         }
@@ -329,8 +331,8 @@ __device__ __forceinline__ void pf_chunks(const Planes& P, const LaneCtx& L, int
             const FoldK k = consts_l2(sgm);
             static_for<4>([&](auto mm) {
                 constexpr int MM = decltype(mm)::value;
-                aop[MM][0] = a_operand<false, 0, MM, 0>(wb, wr, k);
-                aop[MM][1] = a_operand<false, 0, MM, 1>(wb, wr, k);
+                aop[MM][0] = a_operand<false, 0, MM, 0, BK>(wb, wr, k);
+                aop[MM][1] = a_operand<false, 0, MM, 1, BK>(wb, wr, k);
             });
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");         // this wavefront's share of the tile has landed
@@ -391,8 +393,8 @@ __device__ __forceinline__ void pf_chunks(const Planes& P, const LaneCtx& L, int
 // grid (N / 128, ntiles), block 256 (4 wavefronts x 2 strips = 128 weight rows); dynamic LDS = 16 TG * PF_ROW bytes
 // two workgroups per CU at every tile height (the tallest would otherwise need one register too many): while one decodes on
 // the vector ALUs the other runs its MFMAs
-// MASKED = false skips the tiles of experts in mask mode (table flags word set), MASKED = true takes only those: the rarely
-// used path keeps its extra registers out of the common kernel
+// MASKED = false skips the tiles of experts in mask mode (table flags word set) or with a base window code other than 0,
+// MASKED = true takes only those: the rarely used paths keep their extra registers out of the common kernel
 template <int TG, bool MASKED>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) nq_pf_gemm_k(PfGemm a)
 {
@@ -409,7 +411,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) n
     const _Float16* A = (a.mode == 0 && (int)(blockIdx.x * 128) >= a.I) ? a.A1 : a.A0;
     const int t4 = lane >> 4, ss = (lane >> 3) & 1, g = lane & 7, n = lane & 15;
     const Planes P = planes_of(ent, a.mode);
-    if ((P.flags != nullptr && lv == 4) != MASKED) return;       // block-uniform
+    if (((P.flags != nullptr && lv == 4) || P.bcode != 0) != MASKED) return;       // block-uniform
     LaneCtx L;
     L.unit0 = (size_t)(2 * sp + ss) * C; L.rec0 = L.unit0 * 32 + 4 * g + t4;
     L.nrec = (size_t)(N / 16) * C * 32;
@@ -418,8 +420,17 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) n
     float4_t acc[TG][2];
 #pragma unroll
     for (int tg = 0; tg < TG; ++tg) { acc[tg][0] = float4_t{0.f, 0.f, 0.f, 0.f}; acc[tg][1] = float4_t{0.f, 0.f, 0.f, 0.f}; }
-    if (lv == 2) pf_chunks<TG, false, 0, false>(P, L, C, A, K, row0, nrows, smem, acc);
-    else dispatch_code(P.code, [&](auto tag) { pf_chunks<TG, true, decltype(tag)::value, MASKED>(P, L, C, A, K, row0, nrows, smem, acc); });
+    if constexpr (!MASKED)
+    {
+        if (lv == 2) pf_chunks<TG, false, 0, false>(P, L, C, A, K, row0, nrows, smem, acc);
+        else dispatch_code(P.code, [&](auto tag) { pf_chunks<TG, true, decltype(tag)::value, false>(P, L, C, A, K, row0, nrows, smem, acc); });
+    }
+    else
+        dispatch_base(P.bcode, [&](auto bk) {
+            constexpr int BK = decltype(bk)::value;
+            if (lv == 2) pf_chunks<TG, false, 0, false, BK>(P, L, C, A, K, row0, nrows, smem, acc);
+            else dispatch_code(P.code, [&](auto tag) { pf_chunks<TG, true, decltype(tag)::value, true, BK>(P, L, C, A, K, row0, nrows, smem, acc); });
+        });
     // lane (t4, n) holds, for token 16 tg + n, weight rows 32 sp + 16 (t4 >> 1) + 4 (t4 & 1) + i (+ 8 for acc[..][1])
     const int wrow = 32 * sp + 16 * (t4 >> 1) + 4 * (t4 & 1);
 #pragma unroll

@@ -38,15 +38,15 @@ template <int... Is, class F> __device__ __forceinline__ void static_for_impl(F&
 template <int N, class F> __device__ __forceinline__ void static_for(F&& f) { static_for_impl(f, std::make_integer_sequence<int, N>{}); }
 
 // A operand of MFMA (MM, RHO): rows g + 8 RHO, columns of t = 2 MM and 2 MM + 1
-template <bool RES, int CODE, int MM, int RHO>
+template <bool RES, int CODE, int MM, int RHO, int BK = 0>
 __device__ __forceinline__ half8_t a_operand(const uint32_t* wb, const uint32_t* wr, const FoldK& k)
 {
     constexpr int J = 16 * MM + 2 * RHO;
     uint32_t u[4];
-    u[0] = weight_pair<RES, CODE, J + 0, J + 8>(wb, wr, k);
-    u[1] = weight_pair<RES, CODE, J + 1, J + 9>(wb, wr, k);
-    u[2] = weight_pair<RES, CODE, J + 4, J + 12>(wb, wr, k);
-    u[3] = weight_pair<RES, CODE, J + 5, J + 13>(wb, wr, k);
+    u[0] = weight_pair<RES, CODE, J + 0, J + 8, BK>(wb, wr, k);
+    u[1] = weight_pair<RES, CODE, J + 1, J + 9, BK>(wb, wr, k);
+    u[2] = weight_pair<RES, CODE, J + 4, J + 12, BK>(wb, wr, k);
+    u[3] = weight_pair<RES, CODE, J + 5, J + 13, BK>(wb, wr, k);
     return __builtin_bit_cast(half8_t, *(u32x4*)u);
 }
 
@@ -64,7 +64,7 @@ struct LaneCtx
 
 // mask mode: chunk by chunk either the folded decode (refined chunks, residual records compact over them) or the level-2
 // decode; the choice is the same for every lane of the workgroup. Residual records are fetched when needed (no prefetch).
-template <int CODE>
+template <int CODE, int BK>
 __device__ __forceinline__ void gemv_chunks_masked(const Planes& P, const LaneCtx& L, int NC, float4_t* acc, u32x4 nb)
 {
     constexpr int NW = Rec<CODE>::NW;
@@ -81,10 +81,10 @@ __device__ __forceinline__ void gemv_chunks_masked(const Planes& P, const LaneCt
         if (on) { load_record<CODE>(wr, P.res, m.unit * 32 + (L.rec0 & 31), m.nrec); dw = P.dw[m.unit]; }
         if (c + 1 < NC)
         {
-            nb = P.base[L.rec0 + (size_t)(c + 1) * 32];
+            nb = load_base<BK>(P, L.rec0 + (size_t)(c + 1) * 32, L.nrec);
             if (P.var) nvar = P.var[L.unit0 + c + 1];
         }
-        ext_words<128, 4>(wb, __shfl(wb[0], L.src));
+        ext_base<BK>(wb, __shfl(wb[0], L.src));
         const uint32_t sgm = ((var >> L.g) & 1u) * 0x80008000u;
         const char* xp = L.xs + c * L.xstep;
         if (on)
@@ -94,8 +94,8 @@ __device__ __forceinline__ void gemv_chunks_masked(const Planes& P, const LaneCt
             static_for<4>([&](auto mm) {
                 constexpr int MM = decltype(mm)::value;
                 const half8_t b = *(const half8_t*)(xp + MM * 64);
-                acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_operand<true, CODE, MM, 0>(wb, wr, k), b, acc[0], 0, 0, 0);
-                acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_operand<true, CODE, MM, 1>(wb, wr, k), b, acc[1], 0, 0, 0);
+                acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_operand<true, CODE, MM, 0, BK>(wb, wr, k), b, acc[0], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_operand<true, CODE, MM, 1, BK>(wb, wr, k), b, acc[1], 0, 0, 0);
             });
         }
         else
@@ -104,18 +104,18 @@ __device__ __forceinline__ void gemv_chunks_masked(const Planes& P, const LaneCt
             static_for<4>([&](auto mm) {
                 constexpr int MM = decltype(mm)::value;
                 const half8_t b = *(const half8_t*)(xp + MM * 64);
-                acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_operand<false, 0, MM, 0>(wb, wr, k), b, acc[0], 0, 0, 0);
-                acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_operand<false, 0, MM, 1>(wb, wr, k), b, acc[1], 0, 0, 0);
+                acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_operand<false, 0, MM, 0, BK>(wb, wr, k), b, acc[0], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_operand<false, 0, MM, 1, BK>(wb, wr, k), b, acc[1], 0, 0, 0);
             });
         }
     }
 }
 
-template <bool RES, int CODE>
+template <bool RES, int CODE, int BK = 0>
 __device__ __forceinline__ void gemv_chunks(const Planes& P, const LaneCtx& L, int NC, float4_t* acc, u32x4 nb)
 {
     if constexpr (RES)
-        if (P.flags) { gemv_chunks_masked<CODE>(P, L, NC, acc, nb); return; }     // block-uniform
+        if (P.flags) { gemv_chunks_masked<CODE, BK>(P, L, NC, acc, nb); return; }     // block-uniform
     constexpr int NW = RES ? Rec<CODE>::NW : 1;
     uint32_t nr[NW + 2] = {0}, ndw = 0, nvar = 0;
     if constexpr (RES) { load_record<CODE>(nr, P.res, L.rec0, L.nrec); ndw = P.dw[L.unit0]; }
@@ -129,11 +129,11 @@ __device__ __forceinline__ void gemv_chunks(const Planes& P, const LaneCtx& L, i
         const uint32_t dw = ndw, var = nvar;
         if (c + 1 < NC)                                         // prefetch the next chunk's records
         {
-            nb = P.base[L.rec0 + (size_t)(c + 1) * 32];
+            nb = load_base<BK>(P, L.rec0 + (size_t)(c + 1) * 32, L.nrec);
             if constexpr (RES) { load_record<CODE>(nr, P.res, L.rec0 + (size_t)(c + 1) * 32, L.nrec); ndw = P.dw[L.unit0 + c + 1]; }
             if (P.var) nvar = P.var[L.unit0 + c + 1];
         }
-        ext_words<128, 4>(wb, __shfl(wb[0], L.src));
+        ext_base<BK>(wb, __shfl(wb[0], L.src));
         const uint32_t sgm = ((var >> L.g) & 1u) * 0x80008000u;
         FoldK k;
         if constexpr (RES)
@@ -146,8 +146,8 @@ __device__ __forceinline__ void gemv_chunks(const Planes& P, const LaneCtx& L, i
         static_for<4>([&](auto mm) {
             constexpr int MM = decltype(mm)::value;
             const half8_t b = *(const half8_t*)(xp + MM * 64);
-            acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_operand<RES, CODE, MM, 0>(wb, wr, k), b, acc[0], 0, 0, 0);
-            acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_operand<RES, CODE, MM, 1>(wb, wr, k), b, acc[1], 0, 0, 0);
+            acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_operand<RES, CODE, MM, 0, BK>(wb, wr, k), b, acc[0], 0, 0, 0);
+            acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_operand<RES, CODE, MM, 1, BK>(wb, wr, k), b, acc[1], 0, 0, 0);
         });
     }
 }

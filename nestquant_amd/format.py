@@ -2,8 +2,8 @@
 
 Host-side mirror of the format half of the reference's sm120/moe.py (RKP/RK_OF :10-12, rbits :17, step_off :18-20,
 proj_sizes :23-26, pack_words/unpack_words :36-66, Proj :76-107, Expert :177-195). Same names and argument meaning, so
-loaders and tests written against the reference read the same here. Base codes other than 0 are not implemented and
-raise.
+loaders and tests written against the reference read the same here. Base codes 0 (K = 2, one uint4 per record) and 1
+(K = 1.75, the residual plane's sub-array layout at 112 bits per record) are implemented; others raise.
 
 Nested levels of this build (the reference serves levels 0/2/4 only): an expert built with nested=True also carries
 P3 (64 bits / record, K=1 windows, code 10) with block words d3, and P4 (64 bits / record) with block words d4n. Level 3
@@ -158,8 +158,8 @@ class Proj:
     with the same seed yields the same planes as the reference's Proj."""
 
     def __init__(s, N, K, gen, nm=None, rk=0, mbn="rand", var=False, bk=0, nested=False):
-        if bk != 0:
-            raise NotImplementedError("base codes other than 0 are not implemented")
+        if bk not in (0, 1):
+            raise NotImplementedError("base codes other than 0 (K = 2) and 1 (K = 1.75) are not implemented")
         if nm is not None and nested:
             raise NotImplementedError("mask mode applies to the wide residual plane, not to the nested planes")
         dev = gen.device
@@ -169,7 +169,15 @@ class Proj:
         R = C if nm is None else nm                      # residual records and block words exist for R chunks per strip
         nr, nb = S * C * 32, S * R
         bits = rbits(rk); nw = (bits + 31) // 32
-        s.base = torch.randint(-2**31, 2**31 - 1, (nr * 4,), generator=gen, dtype=torch.int32, device=dev)
+        if bk == 0:
+            s.base = torch.randint(-2**31, 2**31 - 1, (nr * 4,), generator=gen, dtype=torch.int32, device=dev)
+            s.bw = None
+        else:                                           # record words of the base code, stored in the sub-array layout
+            bb = rbits(bk)
+            s.bw = torch.randint(0, 2**32, (nr, (bb + 31) // 32), generator=gen, dtype=torch.int64, device=dev)
+            if bb % 32:
+                s.bw[:, -1] &= (1 << (bb % 32)) - 1
+            s.base = pack_words(s.bw, bb)
         w = torch.randint(0, 2**32, (nb * 32, nw), generator=gen, dtype=torch.int64, device=dev)
         if bits % 32:
             w[:, -1] &= (1 << (bits % 32)) - 1
@@ -188,7 +196,7 @@ class Proj:
             s.d3 = (s.Mb3 | (s.N3 << 8)).to(torch.int32)
             s.d4n = (s.Mb4n | (s.N4n << 8)).to(torch.int32)
 
-    _TENSORS = ["base", "p4", "d4", "flags", "fl", "p4w", "Mb", "Nn", "var", "p3", "d3", "p4n", "d4n", "p3w", "p4nw"]
+    _TENSORS = ["base", "bw", "p4", "d4", "flags", "fl", "p4w", "Mb", "Nn", "var", "p3", "d3", "p4n", "d4n", "p3w", "p4nw"]
 
     def to(s, dev):
         for k in s._TENSORS:
@@ -198,7 +206,7 @@ class Proj:
 
     def drop_host_words(s):
         """free the unpacked word tensors (only tests need them)"""
-        s.p4w = s.p3w = s.p4nw = None
+        s.p4w = s.p3w = s.p4nw = s.bw = None
         return s
 
     def nested_plane(s):

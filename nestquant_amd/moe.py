@@ -136,7 +136,11 @@ class MoELayer:
         s.zd = torch.zeros(S * (I // 128) * 4, dtype=f32, device=dev); s.cnt_h = torch.zeros(S * (I // 128), dtype=i32, device=dev)
         s.out = torch.zeros(Bmax, H, dtype=f32, device=dev)
         s.hits_ptr = 0
-        s.masked = False                              # set once a row with mask-mode flags is installed (set / Mailbox.post)
+        s.base_codes = 1                              # bit c = a row with base window code c was installed (set / Mailbox.post). The
+                                                      # decode call passes it on; callers that write table rows themselves with other
+                                                      # base codes must OR them in (or set 0 = unknown), else such picks give NaN
+        s.masked = False                              # set once a row in mask mode or with a base code other than 0 is installed
+                                                      # (set / Mailbox.post): prefill then also launches the variant kernel for such rows
         s._alloc_partials()
 
     @staticmethod
@@ -167,7 +171,8 @@ class MoELayer:
     def set(s, e, ex, level):
         row = entry(ex, level)
         validate_row(row, s.H, s.I)
-        s.masked |= bool(row[4] or row[8])
+        s.masked |= bool(row[4] or row[8] or row[19])
+        s.base_codes |= 1 << (int(row[19]) & 0xFF) | 1 << (int(row[19]) >> 8 & 0xFF)
         s.table[e].copy_(row.to(s.table.device), non_blocking=False)
 
     def __call__(s, x, sel, rw, out=None, force_level=0, which=3, cfg_gu=None, cfg_dn=None, table=None):
@@ -195,6 +200,7 @@ class MoELayer:
         a.force_level, a.which = force_level, which
         a.cnt_h, a.cnt_h_elems = s.cnt_h.data_ptr(), s.cnt_h.numel()
         a.zd, a.zd_elems = s.zd.data_ptr(), s.zd.numel()
+        a.base_codes = s.base_codes if table is None else 0          # a caller's own table: unknown
         a.x_dtype, a.sel_dtype, a.rw_dtype, a.out_dtype = _DT_IN[x.dtype], _DT_SEL[sel.dtype], _DT_IN[rw.dtype], _DT_OUT[out.dtype]
         _lib.check(s.M.nq_moe_forward(C.byref(a), _lib.stream_ptr()))
         return out
@@ -314,7 +320,8 @@ class Mailbox:
         """enqueue on `stream`, after any plane copy already enqueued there: stage[e] = row; seq[e] += 1"""
         assert s.done(e), "one outstanding op per expert"
         validate_row(row, s.L.H, s.L.I)
-        s.L.masked |= bool(row[4] or row[8])
+        s.L.masked |= bool(row[4] or row[8] or row[19])
+        s.L.base_codes |= 1 << (int(row[19]) & 0xFF) | 1 << (int(row[19]) >> 8 & 0xFF)
         s.hseq[e] += 1
         r = row.pin_memory(); q = torch.tensor([s.hseq[e]], dtype=torch.int32).pin_memory()
         s.pins += [r, q]

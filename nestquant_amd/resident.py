@@ -19,8 +19,8 @@ loaded expert has p4 = d4 = None, so its level-2 row comes from moe.entry(ex, 2)
 p4rec.row(ex, lay, slot_ptr, moe.entry).
 
 Files are read with torch.load(weights_only=True): the dict holds tensors, lists, ints and strings only, so nothing in a
-file is executed. v2 files load (each projection gets its `bk`), and the table-row check of this build then refuses
-experts whose base code is not 0, loudly, when they are set into a layer.
+file is executed. v2 files load with each projection's `bk`; the kernels serve base codes 0 and 1, and the table-row
+check refuses any other, loudly, when such an expert is set into a layer.
 """
 import functools
 import json

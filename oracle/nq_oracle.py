@@ -253,12 +253,15 @@ class Plane:
     N, K; base [nrec,4] uint32; level-4 residual: rk code + res [nrec,NW] uint32 + d4 [units] uint32 (Mb | N << 8);
     nested planes: p3 [nrec,2] + d3 [units], p4n [nrec,2] + d4n [units]; var: uint8 per unit (bit g = ring g negated);
     flags (mask mode, reference sm120/moe.py:134-155): int64 per strip, bit c = chunk c is refined; res and d4 then hold only
-    the popcount(flags) refined chunks of each strip, in chunk order, and the other chunks decode at level 2."""
+    the popcount(flags) refined chunks of each strip, in chunk order, and the other chunks decode at level 2.
+    bk: window code of the base plane (reference sm120/moe.py:138-140, sm120/NQ_RES_V2.md:36-49): 0 = two bits per step,
+    128-bit records; otherwise base holds the record words [nrec, ceil(rbits(bk) / 32)] of that code's pattern."""
 
-    def __init__(self, N, K, base, rk=0, res=None, d4=None, p3=None, d3=None, p4n=None, d4n=None, var=None, flags=None):
+    def __init__(self, N, K, base, rk=0, res=None, d4=None, p3=None, d3=None, p4n=None, d4n=None, var=None, flags=None, bk=0):
         self.N, self.K = N, K
         self.S, self.C = N // 16, K // 128
-        self.base = np.asarray(base, np.uint32).reshape(-1, 4)
+        self.bk = bk
+        self.base = np.asarray(base, np.uint32).reshape(-1, (rbits(bk) + 31) // 32)
         self.rk, self.res, self.d4 = rk, res, d4
         self.p3, self.d3, self.p4n, self.d4n, self.var = p3, d3, p4n, d4n, var
         self.flags = None if flags is None else np.asarray(flags, np.int64)
@@ -276,7 +279,7 @@ class Plane:
 def lane_vals(p, level, nested=False, G=4):
     """decoded weights in lane-weight order -> fp16 [S, C, 32, 64]"""
     S, C = p.S, p.C
-    Sb = lane_sums(p.base, 0, G).reshape(S, C, 32, 64)
+    Sb = lane_sums(p.base, p.bk, G).reshape(S, C, 32, 64)
     sign = 1.0
     if p.var is not None:
         ring = np.arange(32) >> 2

@@ -18,7 +18,7 @@ REF = "/root/reference/sm120"
 OUT = os.path.dirname(os.path.abspath(__file__))
 
 
-def main():
+def load_reference():
     sys.modules["build"] = types.SimpleNamespace(get=lambda *a, **k: None, get_sal=lambda *a, **k: None)
     sys.path.insert(0, REF)
     import moe as R          # reference torch decoder (CPU)
@@ -26,6 +26,25 @@ def main():
     # The reference's Proj.to() reads s.bw, which Proj.__init__ only sets for base codes != 0 (sm120/moe.py:84-88,105);
     # a class-level default lets its Expert constructor run for the K=2 base used everywhere here.
     R.Proj.bw = None
+    return R, SP
+
+
+def base_code(R):
+    """7. base window code 1 (K = 1.75 base plane in the sub-array layout, table word 19): planes from the reference
+    generator, dense decode by the reference at levels 2 and 4; residual codes 3 and 9 as in the build that uses it"""
+    for rk, var in ((3, False), (9, True)):
+        seed = 3000 + rk
+        gen = torch.Generator().manual_seed(seed)
+        p = R.Proj(32, 256, gen, None, rk, ("exh", 700 * rk + 3), var=var, bk=1)
+        W2 = R.dense_W(p, 2, 4, torch.float16)
+        W4 = R.dense_W(p, 4, 4, torch.float16)
+        np.savez_compressed(os.path.join(OUT, f"proj_bk1_rk{rk}.npz"), seed=seed, N=32, K=256, rk=rk, bk=1, mbn_offset=700 * rk + 3,
+                            base=p.base.numpy(), p4=p.p4.numpy(), d4=p.d4.numpy(), var=(p.var.numpy() if var else np.zeros(0, np.uint8)),
+                            W2=W2.numpy().view(np.uint16), W4=W4.numpy().view(np.uint16))
+
+
+def main():
+    R, SP = load_reference()
 
     # 1. projections: planes from the reference generator, dense decode by the reference at levels 2 and 4
     for rk in (0, 3, 6, 7, 8, 9):
@@ -129,8 +148,12 @@ def main():
         W4 = R.dense_W(p, 4, 4, torch.float16)
         np.savez_compressed(os.path.join(OUT, f"mask_rk{rk}.npz"), seed=2000 + rk, N=256, K=384, nm=1, rk=rk, mbn_offset=900 * rk + 5,
                             var=int(var), flags=p.flags.numpy(), W4=W4.numpy().view(np.uint16))
+    base_code(R)
     print("fixtures written to", OUT)
 
 
 if __name__ == "__main__":
-    main()
+    if sys.argv[1:] == ["base_code"]:            # only the fixtures of section 7
+        base_code(load_reference()[0])
+    else:
+        main()

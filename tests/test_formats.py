@@ -145,7 +145,7 @@ def test_resident_optional_keys_and_refusals(tmp_path):
     resident._rank_layers.cache_clear()
     (root / "rank1.json").write_text(json.dumps({"layers": {"7": {"in_had_down": 512}, "8": {}}}))
     assert resident.load(p2, "cpu")[0][0].had_dn == 512
-    # base codes other than 0 -> v2 with per-expert lists; the loaded expert carries them and the row check refuses it
+    # base codes other than 0 -> v2 with per-expert lists; the loaded expert carries them into table word 19
     exs[0].gu.bk = 1
     p3 = str(tmp_path / "b.pt")
     resident.save(_rank_layer(exs, [0], H, I), p3)

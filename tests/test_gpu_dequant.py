@@ -180,3 +180,73 @@ def test_mask_mode_layer_decode_and_prefill():
     for e in (1, 3):
         for proj, pl in ((0, planes[e][0]), (1, planes[e][1])):
             assert same_f16(M.dense_W(ex[e], proj, 4).cpu().numpy(), O.dense_W(pl, 4)) == 0
+
+
+@pytest.mark.parametrize("rk", [3, 9])
+def test_base_code_1_golden(rk):
+    """K = 1.75 base plane (table word 19, 112-bit records in the sub-array layout): the reference's own dense decode at
+    levels 2 and 4, through both projections' row fields"""
+    z = np.load(os.path.join(GOLD, f"proj_bk1_rk{rk}.npz"))
+    gen = torch.Generator().manual_seed(int(z["seed"]))
+    p = F.Proj(int(z["N"]), int(z["K"]), gen, None, rk, ("exh", int(z["mbn_offset"])), var=bool(z["var"].size), bk=1).to(DEV)
+    for mode in (0, 1):
+        assert same_f16(gpu_dense(p, 2, p.N, p.K, mode), z["W2"].view(np.float16)) == 0
+        assert same_f16(gpu_dense(p, 4, p.N, p.K, mode), z["W4"].view(np.float16)) == 0
+
+
+def test_base_code_1_layer_decode_and_prefill():
+    """a layer that mixes K = 2 and K = 1.75 base planes (one of the latter also in mask mode, one with a different code per
+    projection): decode path at several k-splits, prefill and the dense decoders against the oracle"""
+    from tests.test_gpu_moe import oracle_layer
+    from tests.util import rel_err
+    H, I, NE = 512, 256, 6
+    bk = [(1, 1), (0, 0), (1, 0), (0, 1), (1, 1), (1, 1)]
+    ex = [F.Expert(H, I, seed=5100 + i, dev="cpu", nm_gu=(2 if i == 4 else None), nm_dn=(1 if i == 4 else None),
+                   rk_gu=(3, 0, 7, 9, 0, 3)[i], rk_dn=(9, 0, 0, 3, 9, 9)[i], var=(i in (0, 3)), bk_gu=bk[i][0], bk_dn=bk[i][1])
+          for i in range(NE)]
+    planes = [(oracle_plane(e.gu), oracle_plane(e.dn), False) for e in ex]
+    signs = [e.signs.numpy() for e in ex]
+    levels = [4, 4, 4, 4, 4, 2]
+    for e in ex:
+        e.gu.to(DEV); e.dn.to(DEV); e.signs = e.signs.to(DEV)
+    assert M.bk_codes() == [3, 3]
+    L = M.MoELayer(NE, H, I, Bmax=4, topk=3)
+    for e in range(NE):
+        L.set(e, ex[e], levels[e])
+    assert int(L.table[2, 19]) == 1 and int(L.table[3, 19]) == 256 and int(L.table[0, 19]) == 257
+    g = torch.Generator().manual_seed(4)
+    for B in (1, 4):
+        sel = torch.stack([torch.randperm(NE, generator=g)[:3] for _ in range(B)]).to(DEV)
+        rw = (torch.rand(B, 3, generator=g) + 0.1).half().to(DEV)
+        x = (torch.randn(B, H, generator=g) * 0.05).half().to(DEV)
+        want = oracle_layer(planes, levels, signs, x, sel, rw)
+        for cg, cd in (([1, 4, 2], [1, 4, 1]), ([1, 2, 4], [1, 4, 2]), ([1, 1, 1], [1, 2, 1])):
+            y = L(x, sel, rw, cfg_gu=cg, cfg_dn=cd)
+            torch.cuda.synchronize()
+            assert rel_err(y.cpu().numpy(), want) < 5e-5, (B, cg, cd)
+        assert rel_err(L.prefill(x, sel, rw).cpu().numpy(), want) < 5e-5, B
+        want2 = oracle_layer(planes, [2] * NE, signs, x, sel, rw)
+        assert rel_err(L(x, sel, rw, force_level=2).cpu().numpy(), want2) < 5e-5
+    for e in (0, 2, 3, 4, 5):
+        for proj, pl in ((0, planes[e][0]), (1, planes[e][1])):
+            assert same_f16(M.dense_W(ex[e], proj, levels[e]).cpu().numpy(), O.dense_W(pl, levels[e])) == 0
+    # other base codes are refused when a row is set
+    bad = M.entry(ex[0], 4); bad[19] = 5
+    with pytest.raises(RuntimeError, match="base codes"):
+        M.validate_row(bad, H, I)
+    # what the host says about the base codes in its table selects the kernel: 0 (unknown) and 3 run the one with every decode
+    # loop; 1 (K=2 rows only) runs the common one, and a wrong 1 is loud: tokens that picked a K=1.75 row come out NaN
+    assert L.base_codes == 3
+    sel = torch.tensor([[1, 1, 1], [0, 1, 2]], device=DEV)
+    rw = torch.tensor([[0.5, 0.25, 0.25], [0.3, 0.3, 0.4]], dtype=torch.float16, device=DEV)
+    x = (torch.randn(2, H, generator=g) * 0.05).half().to(DEV)
+    ref = L(x, sel, rw).clone()
+    L.base_codes = 0
+    assert torch.equal(L(x, sel, rw), ref)
+    L.base_codes = 1
+    y = L(x, sel, rw).clone()
+    torch.cuda.synchronize()
+    assert torch.equal(y[0], ref[0]) and bool(torch.isnan(y[1]).all()) and bool(torch.isfinite(ref).all())
+    assert not L.cnt_gu.any() and not L.cnt_d.any()                  # the workspace contract holds on that path too
+    L.base_codes = 3
+    assert torch.equal(L(x, sel, rw), ref)

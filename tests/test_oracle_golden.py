@@ -17,7 +17,7 @@ PROJ_FILES = sorted(glob.glob(os.path.join(GOLD, "proj_rk*_var*.npz")))
 
 
 def test_fixture_inventory():
-    assert len(PROJ_FILES) == 8
+    assert len(PROJ_FILES) == 8 and len(glob.glob(os.path.join(GOLD, "proj_bk1_rk*.npz"))) == 2
     for f in ("nested_units.npz", "layer_small.npz", "pack_words.npz"):
         assert os.path.exists(os.path.join(GOLD, f))
 
@@ -176,3 +176,26 @@ def test_mask_mode_matches_reference(rk):
         for c in range(3):
             blk = (slice(16 * s_, 16 * s_ + 16), slice(128 * c, 128 * c + 128))
             assert (same_f16(W4[blk], W2[blk]) == 0) == (not on[s_, c])
+
+
+BK_FILES = sorted(glob.glob(os.path.join(GOLD, "proj_bk1_rk*.npz")))
+
+
+@pytest.mark.parametrize("path", BK_FILES, ids=[os.path.basename(p)[:-4] for p in BK_FILES])
+def test_base_code_1_matches_reference(path):
+    """K = 1.75 base plane (window pattern (1, 0xEEEE), 112-bit records in the sub-array layout, table word 19) against the
+    reference's dense decode (sm120/moe.py:138-140); the package's generator draws the same planes from the same seed"""
+    z = np.load(path)
+    N, K, rk = int(z["N"]), int(z["K"]), int(z["rk"])
+    gen = torch.Generator().manual_seed(int(z["seed"]))
+    p = F.Proj(N, K, gen, None, rk, ("exh", int(z["mbn_offset"])), var=bool(z["var"].size), bk=1)
+    assert np.array_equal(p.base.numpy(), z["base"]) and np.array_equal(p.p4.numpy(), z["p4"]) and np.array_equal(p.d4.numpy(), z["d4"])
+    assert p.base.numel() * 4 == F.proj_sizes(N, K, None, rk, 1)["base"] == (N // 16) * (K // 128) * 32 * 14
+    op = oracle_plane(p)
+    assert op.bk == 1 and op.base.shape == ((N // 16) * (K // 128) * 32, 4) and int(op.base[:, 3].max()) < 1 << 16
+    W2 = O.dense_W(op, 2); W4 = O.dense_W(op, 4)
+    assert same_f16(W2, z["W2"].view(np.float16)) == 0 and same_f16(W4, z["W4"].view(np.float16)) == 0
+    # the two independent state walks agree on the 112-bit records, and reading them as K = 2 records is far off
+    assert np.array_equal(O.lane_sums(op.base, 1), O.hash_sum(O.ring_states(op.base, 1)).reshape(-1, 64))
+    wrong = O.Plane(N, K, np.concatenate([op.base, op.base], 0)[: op.base.shape[0]], rk=rk, res=op.res, d4=op.d4, var=op.var, bk=0)
+    assert same_f16(O.dense_W(wrong, 2), z["W2"].view(np.float16)) > 1000

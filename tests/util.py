@@ -26,7 +26,9 @@ def oracle_plane(p):
     if p.nested:
         kw = dict(p3=O.unpack_words(p.p3.cpu().numpy(), nrec, 64), d3=u32(p.d3),
                   p4n=O.unpack_words(p.p4n.cpu().numpy(), nrec, 64), d4n=u32(p.d4n))
-    return O.Plane(p.N, p.K, u32(p.base).reshape(-1, 4), rk=p.rk, res=res, d4=u32(p.d4),
+    bk = int(getattr(p, "bk", 0) or 0)
+    base = u32(p.base).reshape(-1, 4) if bk == 0 else O.unpack_words(p.base.cpu().numpy(), nrec, O.rbits(bk))
+    return O.Plane(p.N, p.K, base, rk=p.rk, bk=bk, res=res, d4=u32(p.d4),
                    var=None if p.var is None else p.var.cpu().numpy(),
                    flags=None if getattr(p, "flags", None) is None else p.flags.cpu().numpy(), **kw)
 
