@@ -90,10 +90,11 @@ typedef struct NqMoeArgs
     void* zd;                 /* fp32 [B*topk * I/128 * 4]: low-rank plane, z_d partials written by the gate|up launch and read by the
                                  down launch (reference zd, sm120/nqmoe.cu:860); needs no zeroing */
     int64_t zd_elems;
-    int32_t base_codes;       /* what the host knows of table word 19 of the rows that can be picked: bit c set = base window code c
-                                 may occur; 0 = unknown (the default: correct for every table). 1 (every row has code 0, the
-                                 K=2 base) selects a kernel without the other codes' decode loops, a few percent faster; should
-                                 a row with another base code be picked under it, the tokens that picked it come out NaN. */
+    int32_t common_rows;      /* 0 (the default): nothing is known about the rows, correct for every table. 1: the host vouches that
+                                 every row that can be picked is of the common kind -- base window code 0 (table word 19) and no
+                                 mask-mode flags (words 4 / 8) -- which selects a kernel without the other kinds' decode loops,
+                                 a few percent faster; should a row of another kind be picked under it, its planes are not
+                                 read and the tokens that picked it come out NaN. */
 } NqMoeArgs;
 int nq_moe_forward(const NqMoeArgs* args, void* stream);
 

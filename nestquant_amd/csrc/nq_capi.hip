@@ -122,8 +122,8 @@ extern "C" int nq_moe_forward(const NqMoeArgs* p, void* stream)
     a.cnt_h = p->cnt_h;
     NQ_REQUIRE(p->zd && p->zd_elems >= S * (p->I / 128) * 4, "workspace too small: zd");
     a.zd = (float*)p->zd;
-    NQ_REQUIRE((p->base_codes & ~3) == 0, "nq_moe_forward: base_codes=%d (bits 0 and 1 only)", p->base_codes);
-    a.base_codes = p->base_codes;
+    NQ_REQUIRE(p->common_rows == 0 || p->common_rows == 1, "nq_moe_forward: common_rows=%d (0 or 1)", p->common_rows);
+    a.common_rows = p->common_rows;
     return launch_moe(a, p->cfg_gu, p->cfg_dn, p->which, (hipStream_t)stream);
 }
 

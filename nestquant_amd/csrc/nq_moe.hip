@@ -373,12 +373,14 @@ __device__ __forceinline__ uint64_t uni(uint64_t v)
 // MODE 0: gate|up (N = 2I, K = H, input x rotated here). MODE 1: down (N = H, K = I, input h).
 // grid (N / 32 / SB, C / NC, S); block 64 * SB threads (SB = 1, 2 or 4: a block covers at most one 128-row group);
 // dynamic LDS = rows * (NC * 256 + 16) + 256 bytes (>= SB * 512 for the combine), one row per token of the call
-// ANYBK = false: the kernel of a layer whose rows all have base window code 0 (the host says so, MoeArgs::base_codes == 1).
-// A run whose row nevertheless names another base code is not decoded as if it were code 0: its partial sums are NaN, so
-// every token that picked it comes out NaN. ANYBK = true also carries the decode loops of the other base codes, which
-// cost registers the common kernel does not have to pay for.
-template <int MODE, bool ANYBK>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) nq_gemv_k(MoeArgs a, int NC)
+// ANYROW = false: the kernel of a layer whose rows are all of the common kind, base window code 0 and no mask-mode flags (the
+// host says so, MoeArgs::common_rows). A run whose row is nevertheless of another kind is not decoded as if it were common:
+// its plane is not read and its partial sums are NaN, so every token that picked it comes out NaN. ANYROW = true also
+// carries the decode loops of the other base codes and of mask mode, which cost ~35 registers that the common kernel does
+// not have to pay for. Four wavefronts per SIMD is the measured optimum for both (three: +4 us per layer; five, which the
+// common kernel reaches at 92 registers: +1.5 us), so the register allocator is told to aim at exactly that.
+template <int MODE, bool ANYROW>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) nq_gemv_k(MoeArgs a, int NC)
 {
     extern __shared__ __align__(16) char smem[];
     __shared__ RunInfo R;
@@ -417,9 +419,10 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) n
     L.nrec = (size_t)(N / 16) * C * 32;
     L.src = (lane + 16) & 63; L.g = g; L.strip = (size_t)strip; L.nstrips = (size_t)(N / 16); L.chunk0 = chunk0;
     L.xs = (n < ntok ? smem + n * rowstride : zero) + t4 * 16; L.xstep = n < ntok ? 256 : 0;
-    const bool foreign = !ANYBK && P.bcode != 0;                  // block-uniform; a smaller plane is not read as 128-bit records
+    // block-uniform: a row the common kernel has no loop for (its plane is not read: the records have another size or order)
+    const bool foreign = !ANYROW && (P.bcode != 0 || (P.flags != nullptr && R.level != 2));
     u32x4 nb0 = {0u, 0u, 0u, 0u};
-    if constexpr (ANYBK) { if (P.bcode == 1) nb0 = load_base<1>(P, L.rec0, L.nrec); else nb0 = P.base[L.rec0]; }
+    if constexpr (ANYROW) { if (P.bcode == 1) nb0 = load_base<1>(P, L.rec0, L.nrec); else nb0 = P.base[L.rec0]; }
     else if (!foreign) nb0 = P.base[L.rec0];
 
     // ---- stage the run's tokens for this k-slice in B-operand order
@@ -469,7 +472,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) n
 
     // ---- decode + MFMA over the k-slice
     float4_t acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
-    if constexpr (ANYBK)
+    if constexpr (ANYROW)
         dispatch_base(P.bcode, [&](auto bk) {
             constexpr int BK = decltype(bk)::value;
             if (R.level == 2) gemv_chunks<false, 0, BK>(P, L, NC, acc, nb0);
@@ -480,8 +483,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) n
         const float nan = __builtin_nanf("");
         acc[0] = float4_t{nan, nan, nan, nan}; acc[1] = acc[0];
     }
-    else if (R.level == 2) gemv_chunks<false, 0>(P, L, NC, acc, nb0);
-    else dispatch_code(P.code, [&](auto tag) { gemv_chunks<true, decltype(tag)::value>(P, L, NC, acc, nb0); });
+    else if (R.level == 2) gemv_chunks<false, 0, 0, false>(P, L, NC, acc, nb0);
+    else dispatch_code(P.code, [&](auto tag) { gemv_chunks<true, decltype(tag)::value, 0, false>(P, L, NC, acc, nb0); });
 
     // ---- k-slice partial sums: lane (t4, n) holds rows 16 (strip0 + t4 / 2) + 4 (t4 & 1) + i (+ 8 for acc[1]) of token n
     if (n < ntok)
@@ -535,8 +538,8 @@ int launch_moe(const MoeArgs& a, const int* cfg_gu, const int* cfg_dn, int which
         const int N = mode == 0 ? 2 * a.I : a.H, K = mode == 0 ? a.H : a.I, C = K / 128;
         const int NX = N / 32 / SB, NY = C / NC;
         const int shm = std::max(a.B * (NC * 256 + 16) + 256, SB * 512);
-        const bool anybk = a.base_codes != 1;                      // 1 = every live row has base code 0; anything else: both paths
-        auto kern = mode == 0 ? (anybk ? nq_gemv_k<0, true> : nq_gemv_k<0, false>) : (anybk ? nq_gemv_k<1, true> : nq_gemv_k<1, false>);
+        const bool any = a.common_rows != 1;
+        auto kern = mode == 0 ? (any ? nq_gemv_k<0, true> : nq_gemv_k<0, false>) : (any ? nq_gemv_k<1, true> : nq_gemv_k<1, false>);
         if (shm > 48 * 1024)
         {
             hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, shm);

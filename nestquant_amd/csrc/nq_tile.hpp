@@ -111,10 +111,11 @@ __device__ __forceinline__ void gemv_chunks_masked(const Planes& P, const LaneCt
     }
 }
 
-template <bool RES, int CODE, int BK = 0>
+// MASKOK = false leaves the mask-mode loop out (the caller has made sure that P.flags is null)
+template <bool RES, int CODE, int BK = 0, bool MASKOK = true>
 __device__ __forceinline__ void gemv_chunks(const Planes& P, const LaneCtx& L, int NC, float4_t* acc, u32x4 nb)
 {
-    if constexpr (RES)
+    if constexpr (RES && MASKOK)
         if (P.flags) { gemv_chunks_masked<CODE, BK>(P, L, NC, acc, nb); return; }     // block-uniform
     constexpr int NW = RES ? Rec<CODE>::NW : 1;
     uint32_t nr[NW + 2] = {0}, ndw = 0, nvar = 0;

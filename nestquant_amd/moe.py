@@ -136,11 +136,11 @@ class MoELayer:
         s.zd = torch.zeros(S * (I // 128) * 4, dtype=f32, device=dev); s.cnt_h = torch.zeros(S * (I // 128), dtype=i32, device=dev)
         s.out = torch.zeros(Bmax, H, dtype=f32, device=dev)
         s.hits_ptr = 0
-        s.base_codes = 1                              # bit c = a row with base window code c was installed (set / Mailbox.post). The
-                                                      # decode call passes it on; callers that write table rows themselves with other
-                                                      # base codes must OR them in (or set 0 = unknown), else such picks give NaN
-        s.masked = False                              # set once a row in mask mode or with a base code other than 0 is installed
-                                                      # (set / Mailbox.post): prefill then also launches the variant kernel for such rows
+        s.rare_rows = False                           # set once a row in mask mode or with a base window code other than 0 is
+                                                      # installed (set / Mailbox.post): the decode call then runs the kernel that
+                                                      # carries their loops and prefill also launches its variant kernel. A caller
+                                                      # that writes such rows into the table itself must set it, else the tokens
+                                                      # that pick them come out NaN
         s._alloc_partials()
 
     @staticmethod
@@ -171,8 +171,7 @@ class MoELayer:
     def set(s, e, ex, level):
         row = entry(ex, level)
         validate_row(row, s.H, s.I)
-        s.masked |= bool(row[4] or row[8] or row[19])
-        s.base_codes |= 1 << (int(row[19]) & 0xFF) | 1 << (int(row[19]) >> 8 & 0xFF)
+        s.rare_rows |= bool(row[4] or row[8] or row[19])
         s.table[e].copy_(row.to(s.table.device), non_blocking=False)
 
     def __call__(s, x, sel, rw, out=None, force_level=0, which=3, cfg_gu=None, cfg_dn=None, table=None):
@@ -200,7 +199,7 @@ class MoELayer:
         a.force_level, a.which = force_level, which
         a.cnt_h, a.cnt_h_elems = s.cnt_h.data_ptr(), s.cnt_h.numel()
         a.zd, a.zd_elems = s.zd.data_ptr(), s.zd.numel()
-        a.base_codes = s.base_codes if table is None else 0          # a caller's own table: unknown
+        a.common_rows = int(table is None and not s.rare_rows)     # a caller's own table: unknown
         a.x_dtype, a.sel_dtype, a.rw_dtype, a.out_dtype = _DT_IN[x.dtype], _DT_SEL[sel.dtype], _DT_IN[rw.dtype], _DT_OUT[out.dtype]
         _lib.check(s.M.nq_moe_forward(C.byref(a), _lib.stream_ptr()))
         return out
@@ -282,7 +281,7 @@ def prefill(s, x, sel, rw, out=None, R=None, G=None, table=None):
         pts, pes = pt[c:d], pe[c:d]
         _lib.check(Lb.nq_pf_pre(x.data_ptr(), pts.data_ptr(), pes.data_ptr(), n, tb.data_ptr(), S["xg"].data_ptr(),
                                 S["xu"].data_ptr(), S["zg"].data_ptr(), E, H, I, st))
-        variants = (0, 2) if s.masked else (0,)                   # experts in mask mode run in their own kernel variant
+        variants = (0, 2) if s.rare_rows else (0,)                # mask mode / other base codes run in their own kernel variant
         for bm, t in tiles.items():
             for v in variants:
                 _lib.check(Lb.nq_pf_gemm(tb.data_ptr(), t.data_ptr(), t.shape[0], bm, v, S["xg"].data_ptr(), S["xu"].data_ptr(),
@@ -320,8 +319,7 @@ class Mailbox:
         """enqueue on `stream`, after any plane copy already enqueued there: stage[e] = row; seq[e] += 1"""
         assert s.done(e), "one outstanding op per expert"
         validate_row(row, s.L.H, s.L.I)
-        s.L.masked |= bool(row[4] or row[8] or row[19])
-        s.L.base_codes |= 1 << (int(row[19]) & 0xFF) | 1 << (int(row[19]) >> 8 & 0xFF)
+        s.L.rare_rows |= bool(row[4] or row[8] or row[19])
         s.hseq[e] += 1
         r = row.pin_memory(); q = torch.tensor([s.hseq[e]], dtype=torch.int32).pin_memory()
         s.pins += [r, q]
