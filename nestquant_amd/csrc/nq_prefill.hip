@@ -24,14 +24,21 @@ __device__ __forceinline__ void store_bop(_Float16* dst, float v0, float v1, int
 {
     const bool hi = (lane >> 3) & 1;
     const float mine = hi ? v1 : v0, give = hi ? v0 : v1;
-    const float got = __shfl_xor(give, 8);                        // low lanes get the partner's v0, high lanes the partner's v1
+    const float got = dpp_lane<0x128>(give);                      // lane ^ 8 (row rotate): low lanes get the partner's v0, high lanes the partner's v1
     half2_t w;
     w.x = (_Float16)(hi ? got : mine); w.y = (_Float16)(hi ? mine : got);
     const int c = hi ? 2 * (lane ^ 8) + 1 : 2 * lane;           // the pair's low column: (c, c + 16)
     *(half2_t*)(dst + bop_index(c)) = w;
 }
 
-// grid (npairs), block 256: wave w handles 128-column groups w, w + 4, ... of gate then up
+// order the LDS accesses of one wavefront's lanes among themselves (a wavefront-private buffer needs no workgroup barrier)
+__device__ __forceinline__ void wave_sync()
+{
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
+
+// grid (npairs), block 256: wave w handles the 512-column segments w, w + 4, ... of the pair's row, gate and up together
 __global__ void __launch_bounds__(256) nq_pf_pre_k(const _Float16* __restrict__ x, const int32_t* __restrict__ pt, const int32_t* __restrict__ pe,
                                                     const int64_t* __restrict__ table, _Float16* xg, _Float16* xu, float* zg, int E, int H, int I)
 {
@@ -65,9 +72,56 @@ __global__ void __launch_bounds__(256) nq_pf_pre_k(const _Float16* __restrict__ 
         __syncthreads();
         if (threadIdx.x < 4) zg[(size_t)p * 4 + threadIdx.x] = zsh[0][threadIdx.x] + zsh[1][threadIdx.x] + zsh[2][threadIdx.x] + zsh[3][threadIdx.x];
     }
-    for (int task = warp; task < 2 * ng; task += 4)
+    // A wavefront takes 512-column segments: x and the two scale vectors arrive as one 16-byte load per lane each and pass
+    // through a wavefront-private LDS buffer to the WHT's layout (lane = columns 2 lane, 2 lane + 1 of a 128-column chunk);
+    // the eight rotated chunks (4 chunks x gate / up) go back through the same buffer in B-operand order and leave as
+    // 16-byte stores. Full segments only when H is a multiple of 512; the remaining chunks take the narrow path below.
+    __shared__ __align__(16) _Float16 seg[4][3 * 512];
+    _Float16* sb = seg[warp];
+    const int nseg = H / 512;
+    for (int sgi = warp; sgi < nseg; sgi += 4)
     {
-        const int up = task / ng, grp = task % ng, k = grp * 128 + 2 * lane;
+        const int k0 = sgi * 512;
+        float v[2][4][2];
+        if (live)
+        {
+            const _Float16* sug = signs, *suu = signs + 2 * H + 3 * I;
+            const uint4 xi = *(const uint4*)(xr + k0 + 8 * lane), gi = *(const uint4*)(sug + k0 + 8 * lane), ui = *(const uint4*)(suu + k0 + 8 * lane);
+            *(uint4*)(sb + 8 * lane) = xi; *(uint4*)(sb + 512 + 8 * lane) = gi; *(uint4*)(sb + 1024 + 8 * lane) = ui;
+            wave_sync();
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+            {
+                const half2_t xv = *(const half2_t*)(sb + 128 * c + 2 * lane), sg = *(const half2_t*)(sb + 512 + 128 * c + 2 * lane),
+                              su = *(const half2_t*)(sb + 1024 + 128 * c + 2 * lane);
+                v[0][c][0] = (float)xv.x * (float)sg.x; v[0][c][1] = (float)xv.y * (float)sg.y;
+                v[1][c][0] = (float)xv.x * (float)su.x; v[1][c][1] = (float)xv.y * (float)su.y;
+            }
+#pragma unroll
+            for (int up = 0; up < 2; ++up)
+#pragma unroll
+                for (int c = 0; c < 4; ++c) wht128(v[up][c][0], v[up][c][1], lane);
+        }
+        else
+        {
+#pragma unroll
+            for (int up = 0; up < 2; ++up)
+#pragma unroll
+                for (int c = 0; c < 4; ++c) v[up][c][0] = v[up][c][1] = 0.f;
+        }
+        wave_sync();       // every lane has read its inputs before the buffer is reused
+#pragma unroll
+        for (int up = 0; up < 2; ++up)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) store_bop(sb + up * 512 + c * 128, v[up][c][0], v[up][c][1], lane);
+        wave_sync();
+        *(uint4*)(xg + (size_t)p * H + k0 + 8 * lane) = *(const uint4*)(sb + 8 * lane);
+        *(uint4*)(xu + (size_t)p * H + k0 + 8 * lane) = *(const uint4*)(sb + 512 + 8 * lane);
+        wave_sync();       // the stores' LDS reads are done before the next segment's writes
+    }
+    for (int task = 8 * nseg + warp; task < 2 * ng; task += 4)       // chunks beyond the last full segment (task = 2 * chunk + up)
+    {
+        const int up = task & 1, grp = task >> 1, k = grp * 128 + 2 * lane;
         _Float16* dst = (up ? xu : xg) + (size_t)p * H + grp * 128;
         float v0 = 0.f, v1 = 0.f;
         if (live)

@@ -13,16 +13,47 @@
 namespace nq {
 
 // ---- Hadamard-128 on one wavefront: lane holds elements 2 lane, 2 lane + 1 --------------------------------------------
+// One in-lane butterfly, then six cross-lane stages: lanes l and l ^ m exchange, the lane with bit m clear keeps a + a',
+// the other a' - a (a' = the partner's value), all in fp32 in this order. The exchanges use no LDS: DPP lane selects for
+// m = 1, 2, 4, 8 (quad permutes, a half-row mirror, a row rotate), and for m = 16, 32 the row / half swaps of gfx950, which
+// leave both partners' values in both lanes. The per-lane sign is a sign-bit flip (or a factor +-1 in an FMA), so every sum
+// is the same single rounding as a plain add or subtract. All 64 lanes must be active.
+template <int CTRL> __device__ __forceinline__ float dpp_lane(float v)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
+}
+__device__ __forceinline__ float flip_sign(float v, uint32_t m) { return __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, v) ^ m); }
+// lo / hi = the value of the lane with bit 16 (bit 32) clear / set, in both lanes. The swap exchanges the odd 16-lane rows
+// (the upper half) of its first register with the even rows (the lower half) of its second; the two read-write operands
+// force two distinct registers that start as the same value. Written as asm because the compiler's builtin for it hands
+// back the first register for both results; the compiler therefore does not see the instruction and cannot place the wait
+// states it needs after the writes that feed it and before the reads of its results, so they are written out here.
+__device__ __forceinline__ void swap_rows16(float v, float& lo, float& hi)
+{
+    lo = v; hi = v;
+    asm volatile("s_nop 3\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 3" : "+v"(lo), "+v"(hi));
+}
+__device__ __forceinline__ void swap_halves32(float v, float& lo, float& hi)
+{
+    lo = v; hi = v;
+    asm volatile("s_nop 3\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 3" : "+v"(lo), "+v"(hi));
+}
 __device__ __forceinline__ void wht128(float& a, float& b, int lane)
 {
     const float s = a + b, d = a - b; a = s; b = d;
-#pragma unroll
-    for (int m = 1; m < 64; m <<= 1)
-    {
-        const float oa = __shfl_xor(a, m), ob = __shfl_xor(b, m);
-        a = (lane & m) ? oa - a : a + oa;
-        b = (lane & m) ? ob - b : b + ob;
-    }
+    const uint32_t l = (uint32_t)lane;
+    const uint32_t n1 = (l << 31) & 0x80000000u, n2 = (l << 30) & 0x80000000u, n4 = (l << 29) & 0x80000000u, n8 = (l << 28) & 0x80000000u;
+    a = dpp_lane<0xB1>(a) + flip_sign(a, n1); b = dpp_lane<0xB1>(b) + flip_sign(b, n1);                   // quad_perm [1,0,3,2]
+    a = dpp_lane<0x4E>(a) + flip_sign(a, n2); b = dpp_lane<0x4E>(b) + flip_sign(b, n2);                   // quad_perm [2,3,0,1]
+    a = dpp_lane<0x141>(dpp_lane<0x1B>(a)) + flip_sign(a, n4);                                            // l ^ 3 then l ^ 7 = l ^ 4
+    b = dpp_lane<0x141>(dpp_lane<0x1B>(b)) + flip_sign(b, n4);
+    a = dpp_lane<0x128>(a) + flip_sign(a, n8); b = dpp_lane<0x128>(b) + flip_sign(b, n8);                 // row_ror 8
+    const float s16 = (lane & 16) ? -1.f : 1.f, s32 = (lane & 32) ? -1.f : 1.f;
+    float lo, hi;
+    swap_rows16(a, lo, hi); a = __builtin_fmaf(hi, s16, lo);
+    swap_rows16(b, lo, hi); b = __builtin_fmaf(hi, s16, lo);
+    swap_halves32(a, lo, hi); a = __builtin_fmaf(hi, s32, lo);
+    swap_halves32(b, lo, hi); b = __builtin_fmaf(hi, s32, lo);
     a *= 0.08838834764f; b *= 0.08838834764f;
 }
 
