@@ -148,6 +148,14 @@ int nq_pf_mid(const float* acc_gu, const int32_t* pe, int np, const int64_t* tab
 int nq_pf_post(const float* y, const int32_t* pos, const int64_t* sel, const void* rw_f16, int T, int topk, int row_lo,
                int nrows, const int64_t* table, float* out, const float* zd, int E, int H, int I, void* stream);
 
+/* Tile lists of one chunk of pair rows, built on the device. counts int32 [E] = pairs per expert over the whole call (pairs
+ * sorted by expert); the chunk holds the pair rows [row_lo, row_lo + nrows). tiles: int32 [5][cap][4], list k for tile height
+ * 16 << k, cap >= E + nrows / 256 + 1. An expert's rows inside the chunk are cut into 256-row tiles (indices E.. of list 4);
+ * the remainder goes to index e of the list of the smallest height that holds it; every other entry gets expert -1, which
+ * nq_pf_gemm skips. Launch nq_pf_gemm on list k with ntiles = E (k < 4) or cap (k = 4). Replaces the host loop over the
+ * expert counts of the reference's prefill (sm120/moe.py:296-302) and the host synchronisation that feeds it. */
+int nq_pf_plan(const int32_t* counts, int E, int row_lo, int nrows, int32_t* tiles, int cap, void* stream);
+
 /* hits[e] += counts[e] (hits may be host-mapped). Replaces pf_hits (reference sm120/nqmoe.cu:1241-1245,1288-1293). */
 int nq_pf_hits(const int32_t* counts, int32_t* hits, int E, void* stream);
 

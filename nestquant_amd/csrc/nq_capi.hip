@@ -177,6 +177,14 @@ extern "C" int nq_pf_post(const float* y, const int32_t* pos, const int64_t* sel
     return launch_pf_post(y, pos, sel, rw, T, topk, row_lo, nrows, table, out, zd, E, H, I, (hipStream_t)stream);
 }
 
+extern "C" int nq_pf_plan(const int32_t* counts, int E, int row_lo, int nrows, int32_t* tiles, int cap, void* stream)
+{
+    NQ_REQUIRE(counts && tiles, "nq_pf_plan: null pointer");
+    NQ_REQUIRE(E >= 1 && E <= 4096 && row_lo >= 0 && nrows >= 0, "nq_pf_plan: E=%d (1..4096) row_lo=%d nrows=%d", E, row_lo, nrows);
+    NQ_REQUIRE(cap >= E + nrows / 256 + 1, "nq_pf_plan: cap=%d, need at least E + nrows / 256 + 1 = %d", cap, E + nrows / 256 + 1);
+    return launch_pf_plan(counts, E, row_lo, nrows, tiles, cap, (hipStream_t)stream);
+}
+
 extern "C" int nq_pf_hits(const int32_t* counts, int32_t* hits, int E, void* stream)
 {
     NQ_REQUIRE(counts && E >= 1, "nq_pf_hits: null counts or E=%d", E);

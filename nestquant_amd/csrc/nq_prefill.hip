@@ -299,6 +299,72 @@ __global__ void nq_pf_hits_k(const int32_t* counts, int32_t* hits, int E)
     if (e < E && counts[e]) __hip_atomic_fetch_add(hits + e, counts[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
+// ---- tile lists on the device ------------------------------------------------------------------------------------------
+// One workgroup. counts[e] = pairs of expert e over the whole call (pairs sorted by expert, so expert e owns the pair rows
+// [sum of counts before e, + counts[e])); the chunk is the pair rows [row_lo, row_lo + nrows). Every expert's rows inside
+// the chunk are cut into 256-row tiles; the remainder goes to the list of the smallest compiled height (16 << k) that holds
+// it, at index e of list k; the full tiles follow at indices E.. of list 4. tiles: int32 [5][cap][4] = (expert, first row in
+// the chunk, rows, 0); entries without a tile get expert -1, which the GEMM skips. Replaces the host loop over the expert
+// counts and with it the call's one host synchronisation.
+__device__ __forceinline__ void block_scan(int* a, int* b, int E)
+{   // inclusive prefix sum of a[0..E) in place (b: scratch of the same size); all threads of the block call it
+    int *src = a, *dst = b;
+    for (int off = 1; off < E; off <<= 1)
+    {
+        for (int e = threadIdx.x; e < E; e += blockDim.x) dst[e] = src[e] + (e >= off ? src[e - off] : 0);
+        __syncthreads();
+        int* t = src; src = dst; dst = t;
+    }
+    if (src != a)
+    {
+        for (int e = threadIdx.x; e < E; e += blockDim.x) a[e] = src[e];
+        __syncthreads();
+    }
+}
+
+__global__ void __launch_bounds__(256) nq_pf_plan_k(const int32_t* __restrict__ counts, int E, int row_lo, int nrows, int32_t* tiles, int cap)
+{
+    extern __shared__ int plan_sh[];
+    int *incl = plan_sh, *tmp = plan_sh + E, *full = plan_sh + 2 * E;
+    for (int e = threadIdx.x; e < E; e += blockDim.x) incl[e] = counts[e] > 0 ? counts[e] : 0;
+    __syncthreads();
+    block_scan(incl, tmp, E);
+    const int row_hi = row_lo + nrows;
+    for (int e = threadIdx.x; e < E; e += blockDim.x)
+    {
+        const int c = counts[e] > 0 ? counts[e] : 0, start = incl[e] - c;
+        const int u = start > row_lo ? start : row_lo, v = start + c < row_hi ? start + c : row_hi;
+        const int n = v > u ? v - u : 0;
+        full[e] = n / 256;
+    }
+    __syncthreads();
+    int* fincl = tmp;                                            // inclusive scan of the full-tile counts
+    for (int e = threadIdx.x; e < E; e += blockDim.x) fincl[e] = full[e];
+    __syncthreads();
+    block_scan(fincl, full, E);                                  // clobbers full[]: recomputed below
+    int4* T4 = (int4*)tiles;
+    for (int e = threadIdx.x; e < E; e += blockDim.x)
+    {
+        const int c = counts[e] > 0 ? counts[e] : 0, start = incl[e] - c;
+        const int u = start > row_lo ? start : row_lo, v = start + c < row_hi ? start + c : row_hi;
+        const int n = v > u ? v - u : 0, r0 = u - row_lo, nf = n / 256, rem = n % 256;
+        const int k = rem == 0 ? -1 : rem <= 16 ? 0 : rem <= 32 ? 1 : rem <= 64 ? 2 : rem <= 128 ? 3 : 4;
+#pragma unroll
+        for (int q = 0; q < 5; ++q) T4[(size_t)q * cap + e] = q == k ? make_int4(e, r0 + 256 * nf, rem, 0) : make_int4(-1, 0, 0, 0);
+        const int base = E + fincl[e] - nf;
+        for (int j = 0; j < nf; ++j) T4[(size_t)4 * cap + base + j] = make_int4(e, r0 + 256 * j, 256, 0);
+    }
+    const int total = E + fincl[E - 1];
+    for (int i = total + threadIdx.x; i < cap; i += blockDim.x) T4[(size_t)4 * cap + i] = make_int4(-1, 0, 0, 0);
+}
+
+int launch_pf_plan(const int32_t* counts, int E, int row_lo, int nrows, int32_t* tiles, int cap, hipStream_t st)
+{
+    nq_pf_plan_k<<<1, 256, 3 * E * sizeof(int), st>>>(counts, E, row_lo, nrows, tiles, cap);
+    NQ_LAUNCH_CHECK("nq_pf_plan");
+    return 0;
+}
+
 struct PfGemm
 {
     const int64_t* table; const int32_t* tiles;   // tiles [ntiles][4]: expert, first row, rows (<= 16 TG), unused

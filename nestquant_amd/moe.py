@@ -244,7 +244,8 @@ def pf_tiles(segs):
 def prefill(s, x, sel, rw, out=None, R=None, G=None, table=None):
     """T > Bmax tokens (reference sm120/moe.py:282-326): pairs sorted by expert, each routed expert decoded inside the
     grouped GEMMs at the level of its live table row, same math as the decode path (fp32 accumulation order differs).
-    One host sync (expert counts). Not graph-capturable. Exports routing hits like the decode kernel."""
+    No host synchronisation (the reference's prefill reads the expert counts back; here the tile lists are built on the
+    device by nq_pf_plan). Exports routing hits like the decode kernel."""
     assert x.dtype == torch.float16 and rw.dtype == torch.float16 and sel.dtype == torch.int64, (x.dtype, rw.dtype, sel.dtype)
     assert x.is_contiguous()
     T, k = sel.shape
@@ -263,34 +264,32 @@ def prefill(s, x, sel, rw, out=None, R=None, G=None, table=None):
     if s.hits_ptr:
         hc = torch.zeros(E + 1, dtype=torch.int32, device=dev).scatter_add_(0, torch.where(rwf != 0, flat, E), one)[:E].contiguous()
         _lib.check(Lb.nq_pf_hits(hc.data_ptr(), s.hits_ptr, E, st))
-    cnt = cnt.cpu().tolist()                                         # the one host sync
-    start, o = [0] * E, 0
-    for e in range(E):
-        start[e] = o; o += cnt[e]
     P = T * k
+    if P == 0:
+        return out
     R = min(P, R or int(__import__("os").environ.get("NQ_PF_ROWS", "32768")))
     S = pf_scratch(dev, H, I, R)
+    cap = E + R // 256 + 1
+    variants = (0, 2) if s.rare_rows else (0,)                    # mask mode / other base codes run in their own kernel variant
     for c in range(0, P, R):
         d = min(P, c + R); n = d - c
-        segs = []
-        for e in range(E):
-            u, v = max(start[e], c), min(start[e] + cnt[e], d)
-            if v > u:
-                segs.append((e, u - c, v - u))
-        tiles = {bm: t.pin_memory().to(dev, non_blocking=True) for bm, t in pf_tiles(segs).items()}
+        # tile lists of the chunk, built on the device from the expert counts: list i = tiles of height 16 << i, entries
+        # without a tile are skipped by the GEMM (no host synchronisation anywhere in the call)
+        tiles = torch.empty(5, cap, 4, dtype=torch.int32, device=dev)
+        _lib.check(Lb.nq_pf_plan(cnt.data_ptr(), E, c, n, tiles.data_ptr(), cap, st))
+        lists = [(16 << i, tiles[i], E if i < 4 else cap) for i in (4, 3, 2, 1, 0)]          # tallest first
         pts, pes = pt[c:d], pe[c:d]
         _lib.check(Lb.nq_pf_pre(x.data_ptr(), pts.data_ptr(), pes.data_ptr(), n, tb.data_ptr(), S["xg"].data_ptr(),
                                 S["xu"].data_ptr(), S["zg"].data_ptr(), E, H, I, st))
-        variants = (0, 2) if s.rare_rows else (0,)                # mask mode / other base codes run in their own kernel variant
-        for bm, t in tiles.items():
+        for bm, t, nt in lists:
             for v in variants:
-                _lib.check(Lb.nq_pf_gemm(tb.data_ptr(), t.data_ptr(), t.shape[0], bm, v, S["xg"].data_ptr(), S["xu"].data_ptr(),
+                _lib.check(Lb.nq_pf_gemm(tb.data_ptr(), t.data_ptr(), nt, bm, v, S["xg"].data_ptr(), S["xu"].data_ptr(),
                                          S["acc"].data_ptr(), E, H, I, st))
         _lib.check(Lb.nq_pf_mid(S["acc"].data_ptr(), pes.data_ptr(), n, tb.data_ptr(), S["h"].data_ptr(), S["zg"].data_ptr(),
                                 S["zd"].data_ptr(), E, H, I, st))
-        for bm, t in tiles.items():
+        for bm, t, nt in lists:
             for v in variants:
-                _lib.check(Lb.nq_pf_gemm(tb.data_ptr(), t.data_ptr(), t.shape[0], bm, 1 | v, S["h"].data_ptr(), None,
+                _lib.check(Lb.nq_pf_gemm(tb.data_ptr(), t.data_ptr(), nt, bm, 1 | v, S["h"].data_ptr(), None,
                                          S["y"].data_ptr(), E, H, I, st))
         _lib.check(Lb.nq_pf_post(S["y"].data_ptr(), pos.data_ptr(), selc.data_ptr(), rwc.data_ptr(), T, k, c, n, tb.data_ptr(),
                                  out.data_ptr(), S["zd"].data_ptr(), E, H, I, st))

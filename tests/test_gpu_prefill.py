@@ -103,3 +103,39 @@ def test_prefill_argument_errors_and_empty():
     y = L.prefill(x, sel, rw)                                    # every expert at level 0: output is zero, nothing faults
     torch.cuda.synchronize()
     assert not y.any()
+
+
+def test_device_tile_planner_matches_host_lists():
+    """nq_pf_plan against pf_tiles (the host construction the reference's prefill uses) for random expert counts and chunk
+    windows: the same set of tiles per height, everything else marked as skipped"""
+    from nestquant_amd import _lib
+    g = torch.Generator().manual_seed(21)
+    for E, scale in ((7, 40), (256, 300), (300, 5), (64, 2000)):
+        cnt = (torch.rand(E, generator=g) ** 3 * scale).int()
+        cnt[torch.randint(0, E, (max(1, E // 5),), generator=g)] = 0
+        if E == 64:
+            cnt[3] = 256; cnt[4] = 512; cnt[5] = 257; cnt[6] = 16; cnt[7] = 17
+        P = int(cnt.sum())
+        start = torch.cumsum(cnt, 0) - cnt
+        for lo, n in ((0, P), (P // 3, P // 2), (0, 0), (P - 1, 1)) if P else ((0, 0),):
+            segs = []
+            for e in range(E):
+                u, v = max(int(start[e]), lo), min(int(start[e] + cnt[e]), lo + n)
+                if v > u:
+                    segs.append((e, u - lo, v - u))
+            want = {bm: sorted(map(tuple, t.tolist())) for bm, t in M.pf_tiles(segs).items()}
+            cap = E + n // 256 + 1
+            tiles = torch.full((5, cap, 4), 77, dtype=torch.int32, device=DEV)
+            _lib.check(_lib.lib().nq_pf_plan(cnt.to(DEV).data_ptr(), E, lo, n, tiles.data_ptr(), cap, None))
+            torch.cuda.synchronize()
+            t = tiles.cpu()
+            for i in range(5):
+                used = t[i, : (E if i < 4 else cap)]
+                live = used[used[:, 0] >= 0]
+                assert sorted(map(tuple, live.tolist())) == want.get(16 << i, []), (E, lo, n, i)
+                assert bool((used[used[:, 0] < 0][:, 0] == -1).all())
+                covered = sum(r for _, _, r, _ in live.tolist())
+            total = sum(int(t[i, : (E if i < 4 else cap)][t[i, : (E if i < 4 else cap), 0] >= 0][:, 2].sum()) for i in range(5))
+            assert total == n
+    with pytest.raises(RuntimeError, match="cap"):
+        _lib.check(_lib.lib().nq_pf_plan(cnt.to(DEV).data_ptr(), 64, 0, 1024, tiles.data_ptr(), 64, None))
