@@ -95,6 +95,9 @@ typedef struct NqMoeArgs
                                  mask-mode flags (words 4 / 8) -- which selects a kernel without the other kinds' decode loops,
                                  a few percent faster; should a row of another kind be picked under it, its planes are not
                                  read and the tokens that picked it come out NaN. */
+    int32_t G;                /* lanes per ring (reference moe_forward's G, sm120/nqmoe.cu:223-228,862): 0 or 4 = rings of four
+                                 records (the format every artifact uses), 2 = the same planes read as rings of two records
+                                 (the reference's test variant; not with sign-variant planes, not in prefill) */
 } NqMoeArgs;
 int nq_moe_forward(const NqMoeArgs* args, void* stream);
 

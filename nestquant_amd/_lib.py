@@ -22,7 +22,7 @@ class NqMoeArgs(C.Structure):
                 ("cfg_gu", C.c_int32 * 4), ("cfg_dn", C.c_int32 * 4), ("force_level", C.c_int32), ("which", C.c_int32),
                 ("x_dtype", C.c_int32), ("sel_dtype", C.c_int32), ("rw_dtype", C.c_int32), ("out_dtype", C.c_int32),
                 ("cnt_h", C.c_void_p), ("cnt_h_elems", C.c_int64), ("zd", C.c_void_p), ("zd_elems", C.c_int64),
-                ("common_rows", C.c_int32)]
+                ("common_rows", C.c_int32), ("G", C.c_int32)]
 
 
 # name -> (restype, argtypes); every symbol declared in include/nq_moe_hip.h

@@ -124,6 +124,8 @@ extern "C" int nq_moe_forward(const NqMoeArgs* p, void* stream)
     a.zd = (float*)p->zd;
     NQ_REQUIRE(p->common_rows == 0 || p->common_rows == 1, "nq_moe_forward: common_rows=%d (0 or 1)", p->common_rows);
     a.common_rows = p->common_rows;
+    NQ_REQUIRE(p->G == 0 || p->G == 4 || p->G == 2, "nq_moe_forward: G=%d (rings of 4 lanes, or 2)", p->G);
+    a.G = p->G == 2 ? 2 : 4;
     return launch_moe(a, p->cfg_gu, p->cfg_dn, p->which, (hipStream_t)stream);
 }
 

@@ -31,6 +31,7 @@ struct MoeArgs
     int* cnt_gu; int* cnt_d;          // arrival counters [S * I/128] and [H/128]: zero on entry, zero on exit
     float* zd;                        // low-rank plane: z_d partials [S][I/128][4], written by gate|up, read by down; may be null
     int* cnt_h;                       // arrival counters of the 512-column blocks (in_had_down = 512) [S * I/128]; may be null
+    int G;                            // lanes per ring: 4, or 2 (the same planes read as rings of two records)
     int common_rows;                  // 1 = every row that can be picked has base window code 0 and no mask-mode flags; 0 = unknown
 };
 

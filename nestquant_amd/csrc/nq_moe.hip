@@ -417,7 +417,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
     LaneCtx L;
     L.unit0 = (size_t)strip * C + chunk0; L.rec0 = L.unit0 * 32 + 4 * g + t4;
     L.nrec = (size_t)(N / 16) * C * 32;
-    L.src = (lane + 16) & 63; L.g = g; L.strip = (size_t)strip; L.nstrips = (size_t)(N / 16); L.chunk0 = chunk0;
+    L.src = a.G == 2 ? lane ^ 16 : (lane + 16) & 63;             // next record of the ring: rings of four lanes, or of two
+    L.g = g; L.strip = (size_t)strip; L.nstrips = (size_t)(N / 16); L.chunk0 = chunk0;
     L.xs = (n < ntok ? smem + n * rowstride : zero) + t4 * 16; L.xstep = n < ntok ? 256 : 0;
     // block-uniform: a row the common kernel has no loop for (its plane is not read: the records have another size or order)
     const bool foreign = !ANYROW && (P.bcode != 0 || (P.flags != nullptr && R.level != 2));

@@ -122,8 +122,8 @@ class MoELayer:
     compatibility and stay zero."""
 
     def __init__(s, E, H, I, nm_gu=0, nm_dn=0, Bmax=4, topk=8, G=4, dev="cuda", mod=None):
-        if G != 4:
-            raise NotImplementedError("rings of G=4 lanes only")
+        if G not in (4, 2):
+            raise NotImplementedError("rings of G = 4 lanes (every artifact) or G = 2 (the reference's test variant) only")
         s.M = mod or _lib.lib()
         s.E, s.H, s.I, s.nm_gu, s.nm_dn, s.G, s.Bmax, s.topk = E, H, I, nm_gu, nm_dn, G, Bmax, topk
         s.table = torch.zeros(E, TBL_W, dtype=torch.int64, device=dev)
@@ -170,6 +170,8 @@ class MoELayer:
 
     def set(s, e, ex, level):
         row = entry(ex, level)
+        if s.G != 4 and (row[12] or row[13]):
+            raise ValueError("sign-variant planes are defined for rings of G = 4 lanes only (reference sm120/moe.py:143)")
         validate_row(row, s.H, s.I)
         s.rare_rows |= bool(row[4] or row[8] or row[19])
         s.table[e].copy_(row.to(s.table.device), non_blocking=False)
@@ -199,6 +201,7 @@ class MoELayer:
         a.force_level, a.which = force_level, which
         a.cnt_h, a.cnt_h_elems = s.cnt_h.data_ptr(), s.cnt_h.numel()
         a.zd, a.zd_elems = s.zd.data_ptr(), s.zd.numel()
+        a.G = s.G
         a.common_rows = int(table is None and not s.rare_rows)     # a caller's own table: unknown
         a.x_dtype, a.sel_dtype, a.rw_dtype, a.out_dtype = _DT_IN[x.dtype], _DT_SEL[sel.dtype], _DT_IN[rw.dtype], _DT_OUT[out.dtype]
         _lib.check(s.M.nq_moe_forward(C.byref(a), _lib.stream_ptr()))
@@ -246,6 +249,8 @@ def prefill(s, x, sel, rw, out=None, R=None, G=None, table=None):
     grouped GEMMs at the level of its live table row, same math as the decode path (fp32 accumulation order differs).
     No host synchronisation (the reference's prefill reads the expert counts back; here the tile lists are built on the
     device by nq_pf_plan). Exports routing hits like the decode kernel."""
+    if s.G != 4:
+        raise NotImplementedError("prefill decodes rings of G = 4 lanes only (as the reference's pf_decode)")
     assert x.dtype == torch.float16 and rw.dtype == torch.float16 and sel.dtype == torch.int64, (x.dtype, rw.dtype, sel.dtype)
     assert x.is_contiguous()
     T, k = sel.shape

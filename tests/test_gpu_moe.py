@@ -36,10 +36,10 @@ def to_dev(ex):
     return ex
 
 
-def oracle_layer(ex_cpu_planes, levels, signs, x, sel, rw, **kw):
+def oracle_layer(ex_cpu_planes, levels, signs, x, sel, rw, G=4, **kw):
     def dense(e):
         pg, pd, nested = ex_cpu_planes[e]
-        return (O.dense_W(pg, levels[e], nested=nested).astype(np.float32), O.dense_W(pd, levels[e], nested=nested).astype(np.float32))
+        return (O.dense_W(pg, levels[e], nested=nested, G=G).astype(np.float32), O.dense_W(pd, levels[e], nested=nested, G=G).astype(np.float32))
     kw.setdefault("dtype", np.float64)
     return O.moe_forward(dense, levels, lambda e: signs[e], x.cpu().numpy(), sel.cpu().numpy(), rw.cpu().numpy(), **kw)
 
@@ -308,3 +308,34 @@ def test_low_rank_plane_decode_and_prefill(golden_dir):
     row = M.entry(ex[0], 2).clone(); row[16] = 5
     with pytest.raises(RuntimeError, match="low-rank"):
         M.validate_row(row, int(z["H"]), int(z["I"]))
+
+
+def test_rings_of_two_lanes():
+    """MoELayer(G=2): the same planes read as rings of two records (the reference's second kernel variant,
+    sm120/nqmoe.cu:223-228, exercised by its sm120/verify15.py:42): decode path against the oracle's G = 2 decode"""
+    H, I, NE = 256, 384, 5
+    ex = experts_on_gpu(H, I, NE, 900, nested_ids=(3,), rk=[(0, 0), (3, 9), (7, 0), (0, 0), (6, 8)])
+    planes = [(oracle_plane(e.gu), oracle_plane(e.dn), e.nested) for e in ex]
+    signs = [e.signs.numpy() for e in ex]
+    levels = [2, 4, 4, 3, 4]
+    to_dev(ex)
+    L2 = M.MoELayer(NE, H, I, Bmax=4, topk=3, G=2)
+    L4 = M.MoELayer(NE, H, I, Bmax=4, topk=3)
+    for e in range(NE):
+        L2.set(e, ex[e], levels[e]); L4.set(e, ex[e], levels[e])
+    g = torch.Generator().manual_seed(8)
+    sel = torch.stack([torch.randperm(NE, generator=g)[:3] for _ in range(4)]).to(DEV)
+    rw = (torch.rand(4, 3, generator=g) + 0.1).half().to(DEV)
+    x = (torch.randn(4, H, generator=g) * 0.05).half().to(DEV)
+    want2 = oracle_layer(planes, levels, signs, x, sel, rw, G=2)
+    want4 = oracle_layer(planes, levels, signs, x, sel, rw)
+    for cg, cd in (([1, 4, 2], [1, 4, 3]), ([1, 2, 1], [1, 1, 1])):
+        assert rel_err(L2(x, sel, rw, cfg_gu=cg, cfg_dn=cd).cpu().numpy(), want2) < 5e-5
+        assert rel_err(L4(x, sel, rw, cfg_gu=cg, cfg_dn=cd).cpu().numpy(), want4) < 5e-5
+    assert rel_err(want2, want4) > 1e-2                              # the two readings of the planes differ
+    with pytest.raises(NotImplementedError):
+        L2.prefill(x, sel, rw)
+    with pytest.raises(ValueError, match="sign-variant"):
+        L2.set(0, to_dev(experts_on_gpu(H, I, 1, 950, var_ids=(0,)))[0], 2)
+    with pytest.raises(NotImplementedError):
+        M.MoELayer(NE, H, I, G=1)

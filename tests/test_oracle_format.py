@@ -156,6 +156,10 @@ def test_lane_view_equals_ring_view(code):
     lane = O.lane_sums(w, code)                                # [64 records, 64]
     ring = O.hash_sum(O.ring_states(w, code))                  # [16 rings, 256], position p = t4 * 64 + j
     assert np.array_equal(lane.reshape(16, 256), ring)
+    # rings of two records (the reference's G = 2 reading of the same planes): both walks agree there too, and differ from G = 4
+    lane2 = O.lane_sums(w, code, G=2)
+    assert np.array_equal(lane2.reshape(32, 128), O.hash_sum(O.ring_states(w, code, G=2)))
+    assert not np.array_equal(lane2, lane)
 
 
 def test_tail_biting_is_real():
