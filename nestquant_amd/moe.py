@@ -1,7 +1,7 @@
 """NestQuant grouped MoE layer on MI355X: device table, workspaces, launch wrappers.
 
 Host-side mirror of the reference's Python op surface (sm120/moe.py): `entry` :216-229, `MoELayer` :231-260,
-`prefill` :282-326, `Mailbox` :329-342, `dense_W` :156-166, `H128` :168-172. The kernels behind it are the HIP kernels of
+`prefill` :282-326, `Mailbox` :329-342, `dense_W` :156-166, `H128` :168-172, `Expert.ref` :196-210, `moe_ref` :344-351. The kernels behind it are the HIP kernels of
 libnq_moe_hip.so, reached through ctypes with raw device pointers; there is no CPU path in this module.
 """
 import ctypes as C
@@ -9,7 +9,7 @@ import ctypes as C
 import torch
 
 from . import _lib
-from .format import (CODE_L3, CODE_L4N, RK_OF, RKP, TBL_W, Expert, Proj, all_MbN, pack_words, popc, proj_sizes,  # noqa: F401
+from .format import (CODE_L3, CODE_L4N, RK_OF, RKP, TBL_W, Expert, Proj, all_MbN, make_flags, pack_words, popc, proj_sizes,  # noqa: F401
                      rbits, split_bits, step_off, unpack_words)
 
 
@@ -368,6 +368,64 @@ def forward(layer, mailbox, x, topk_weights, topk_ids, pf_min=PF_MIN, sal=None):
         if sal is not None and T <= 16:
             sal(x[i:j], w[i:j], ids[i:j])
     return out
+
+
+def _lr_parts(ex, level):
+    """the low-rank factors of `ex` as fp32 matrices, read back from the two table buffers (lr = V_g | U2_g | U2_u | V_d | U2_d,
+    lr4 = U4_g | U4_u | U4_d): (V_g [rg, H], U_g [rg, I], U_u [rg, I], V_d [rd, I], U_d [rd, H]) with U = U2 (+ U4 at level 4)"""
+    H, I, rg, rd = ex.H, ex.I, ex.rg, ex.rd
+    cut = lambda t, sizes: [c.float() for c in torch.split(t[: sum(sizes)], sizes)]
+    Vg, U2g, U2u, Vd, U2d = cut(ex.lr, [rg * H, rg * I, rg * I, rd * I, rd * H])
+    Ug, Uu, Ud = U2g, U2u, U2d
+    if level == 4:
+        U4g, U4u, U4d = cut(ex.lr4, [rg * I, rg * I, rd * H])
+        Ug, Uu, Ud = Ug + U4g, Uu + U4u, Ud + U4d
+    return Vg.view(rg, H), Ug.view(rg, I), Uu.view(rg, I), Vd.view(rd, I), Ud.view(rd, H)
+
+
+def expert_ref(ex, x, level, G=4):
+    """One expert's MLP through dense weights (reference Expert.ref, sm120/moe.py:196-210): x [T, H] fp32 -> [T, H] fp32 on the
+    expert's device. The weights are decoded by the HIP decoder (bit-exact values); rotations, products and sums are plain
+    torch fp32 with the two fp16 roundings of the activations, so this is the slow, transparent twin of the fused kernels that
+    check scripts compare them with. Rings of G = 4 lanes."""
+    if G != 4:
+        raise NotImplementedError("the dense decoder reads rings of G = 4 lanes")
+    H, I, dev = ex.H, ex.I, ex.signs.device
+    x = x.to(dev, torch.float32)
+    had = lambda v, n=128: (v.reshape(*v.shape[:-1], -1, n) @ H128(dev, n)).reshape(v.shape)
+    su_g, sv_g, sv_u, su_d, sv_o, su_u = torch.split(ex.signs.float(), [H, I, I, I, H, H])
+    Wgu, Wdn = dense_W(ex, 0, level, torch.float32), dense_W(ex, 1, level, torch.float32)
+    g = had(had(x * su_g).half().float() @ Wgu[:I].T) * sv_g
+    u = had(had(x * su_u).half().float() @ Wgu[I:].T) * sv_u
+    lowrank = getattr(ex, "lr", None) is not None
+    if lowrank:
+        Vg, Ug, Uu, Vd, Ud = _lr_parts(ex, level)
+        z = x @ Vg.T
+        g, u = g + z @ Ug, u + z @ Uu
+    sw = torch.nn.functional.silu(g) * u
+    y = had(had(sw * su_d, had_dn(ex)).half().float() @ Wdn.T) * sv_o
+    if lowrank:
+        y = y + (sw @ Vd.T) @ Ud
+    return y
+
+
+def moe_ref(experts, levels, x, sel, rw, G=4):
+    """The layer through expert_ref (reference moe_ref, sm120/moe.py:344-351): out[t] = sum over the picks of rw * expert(x[t]),
+    picks of level <= 0 or weight 0 skipped. Every distinct routed expert is decoded once and applied to all its tokens."""
+    T, H = x.shape
+    y = torch.zeros(T, H, dtype=torch.float32, device=x.device)
+    xf, w = x.float(), rw.float()
+    for e in sorted(set(sel.flatten().tolist())):
+        if not 0 <= e < len(experts) or levels[e] <= 0:
+            continue
+        hit = (sel == e) & (w != 0)
+        rows = hit.any(1).nonzero().flatten()
+        if rows.numel():
+            y[rows] += (w * hit)[rows].sum(1, keepdim=True) * expert_ref(experts[e], xf[rows], levels[e], G).to(x.device)
+    return y
+
+
+Expert.ref = expert_ref
 
 
 def proj_gemv(layer, x, e=0, cfg=None):

@@ -92,6 +92,10 @@ def test_golden_layer_fixture(golden_dir):
     y = L(x, sel, rw)
     torch.cuda.synchronize()
     assert rel_err(y.cpu().numpy(), z["y"]) < 1e-4               # the fixture is the reference's fp32 torch result
+    # the package's own torch twin (moe_ref / Expert.ref over HIP-decoded dense weights) reproduces the reference's numbers
+    levels = [int(v) for v in z["levels"]]
+    assert rel_err(M.moe_ref(ex, levels, x, sel, rw).cpu().numpy(), z["y"]) < 1e-4   # two fp32 summation orders around the fp16 roundings
+    assert rel_err(ex[1].ref(x.float(), 4).cpu().numpy(), z["y_expert1_level4"]) < 1e-4
 
 
 def _dense_from_gpu(ex, levels):
@@ -297,6 +301,7 @@ def test_low_rank_plane_decode_and_prefill(golden_dir):
     for had, key in ((128, "y_lr"), (512, "y_had512_lr")):
         z, L, ex, x, sel, rw = _optional_feature_layer(golden_dir, had, True)
         want = z[key]
+        assert rel_err(M.moe_ref(ex, [int(v) for v in z["levels"]], x, sel, rw).cpu().numpy(), want) < 1e-4, had
         for cg, cd in (([1, 4, 2], [1, 4, 4]), ([1, 4, 1], [1, 2, 1])):
             y = L(x, sel, rw, cfg_gu=cg, cfg_dn=cd).clone()
             torch.cuda.synchronize()
