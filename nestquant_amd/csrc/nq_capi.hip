@@ -12,6 +12,8 @@ char* error_buffer()
     return buf;
 }
 static bool shape_ok(int H, int I) { return H > 0 && I > 0 && H % 128 == 0 && I % 128 == 0; }
+// the kernels move 16 bytes per lane; rows are multiples of 256 bytes, so the base address decides
+static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 }  // namespace nq
 
 using namespace nq;
@@ -98,6 +100,8 @@ extern "C" int nq_moe_forward(const NqMoeArgs* p, void* stream)
     NQ_REQUIRE(p->force_level == 0 || p->force_level == 2 || p->force_level == 3 || p->force_level == 4, "nq_moe_forward: force_level=%d", p->force_level);
     NQ_REQUIRE(p->x_dtype >= 0 && p->x_dtype <= 2 && p->rw_dtype >= 0 && p->rw_dtype <= 2 && p->sel_dtype >= 0 && p->sel_dtype <= 1 && p->out_dtype >= 0 && p->out_dtype <= 2,
                "nq_moe_forward: dtype codes x=%d sel=%d rw=%d out=%d", p->x_dtype, p->sel_dtype, p->rw_dtype, p->out_dtype);
+    NQ_REQUIRE(aligned16(p->x) && aligned16(p->out) && aligned16(p->acc_gu) && aligned16(p->acc_d) && aligned16(p->h),
+               "nq_moe_forward: x, out, acc_gu, acc_d and h must be 16-byte aligned");
     const int64_t S = (int64_t)p->B * p->topk;
     for (int mode = 0; mode < 2; ++mode)
     {
@@ -143,6 +147,7 @@ extern "C" int nq_pf_pre(const void* x, const int32_t* pt, const int32_t* pe, in
     if (np == 0) return 0;
     NQ_REQUIRE(x && pt && pe && table && xg && xu, "nq_pf_pre: null pointer");
     NQ_REQUIRE(E >= 1 && shape_ok(H, I), "nq_pf_pre: E=%d H=%d I=%d (H, I positive multiples of 128)", E, H, I);
+    NQ_REQUIRE(aligned16(x) && aligned16(xg) && aligned16(xu), "nq_pf_pre: x, xg and xu must be 16-byte aligned");
     return launch_pf_pre(x, pt, pe, np, table, xg, xu, zg, E, H, I, (hipStream_t)stream);
 }
 
@@ -156,6 +161,7 @@ extern "C" int nq_pf_gemm(const int64_t* table, const int32_t* tiles, int ntiles
     NQ_REQUIRE((mode & 1) == 1 || A1, "nq_pf_gemm: gate|up needs both activation buffers");
     NQ_REQUIRE(ntiles <= 65535, "nq_pf_gemm: %d tiles exceed one launch (65535)", ntiles);
     NQ_REQUIRE(E >= 1 && shape_ok(H, I), "nq_pf_gemm: E=%d H=%d I=%d (H, I positive multiples of 128)", E, H, I);
+    NQ_REQUIRE(aligned16(A0) && aligned16(A1) && aligned16(C) && aligned16(tiles), "nq_pf_gemm: tiles, activations and C must be 16-byte aligned");
     return launch_pf_gemm(table, tiles, ntiles, bm, mode, A0, A1, C, E, H, I, (hipStream_t)stream);
 }
 
@@ -166,6 +172,7 @@ extern "C" int nq_pf_mid(const float* acc_gu, const int32_t* pe, int np, const i
     if (np == 0) return 0;
     NQ_REQUIRE(acc_gu && pe && table && h, "nq_pf_mid: null pointer");
     NQ_REQUIRE(E >= 1 && shape_ok(H, I), "nq_pf_mid: E=%d H=%d I=%d (H, I positive multiples of 128)", E, H, I);
+    NQ_REQUIRE(aligned16(acc_gu) && aligned16(h), "nq_pf_mid: acc_gu and h must be 16-byte aligned");
     return launch_pf_mid(acc_gu, pe, np, table, h, zg, zd, E, H, I, (hipStream_t)stream);
 }
 
@@ -176,6 +183,7 @@ extern "C" int nq_pf_post(const float* y, const int32_t* pos, const int64_t* sel
     if (T == 0 || nrows == 0) return 0;
     NQ_REQUIRE(y && pos && sel && rw && table && out, "nq_pf_post: null pointer");
     NQ_REQUIRE(E >= 1 && shape_ok(H, I), "nq_pf_post: E=%d H=%d I=%d (H, I positive multiples of 128)", E, H, I);
+    NQ_REQUIRE(aligned16(y) && aligned16(out), "nq_pf_post: y and out must be 16-byte aligned");
     return launch_pf_post(y, pos, sel, rw, T, topk, row_lo, nrows, table, out, zd, E, H, I, (hipStream_t)stream);
 }
 
@@ -183,6 +191,7 @@ extern "C" int nq_pf_plan(const int32_t* counts, int E, int row_lo, int nrows, i
 {
     NQ_REQUIRE(counts && tiles, "nq_pf_plan: null pointer");
     NQ_REQUIRE(E >= 1 && E <= 4096 && row_lo >= 0 && nrows >= 0, "nq_pf_plan: E=%d (1..4096) row_lo=%d nrows=%d", E, row_lo, nrows);
+    NQ_REQUIRE(aligned16(tiles), "nq_pf_plan: tiles must be 16-byte aligned");
     NQ_REQUIRE(cap >= E + nrows / 256 + 1, "nq_pf_plan: cap=%d, need at least E + nrows / 256 + 1 = %d", cap, E + nrows / 256 + 1);
     return launch_pf_plan(counts, E, row_lo, nrows, tiles, cap, (hipStream_t)stream);
 }

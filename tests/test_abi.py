@@ -75,3 +75,38 @@ def test_shape_errors_and_code_masks():
     assert out[0] == out[1] == 0xFFF and out[2] == out[3] == 3
     with pytest.raises(RuntimeError, match="multiples of 128"):
         _lib.check(_validate(_row(), I=100))
+
+
+def test_argument_checks_run_before_any_device_work():
+    """bad arguments are refused on the host, with a message, before anything is launched (so this runs without a GPU)"""
+    L = _lib.lib()
+    err = lambda: L.nq_last_error().decode()
+    buf = (C.c_char * 4096)()
+    base = C.addressof(buf)
+    base += (-base) % 16                                           # a 16-byte aligned address inside the buffer
+    a = _lib.NqMoeArgs()
+    for f in ("x", "sel", "rw", "table", "out", "acc_gu", "h", "acc_d", "cnt_gu", "cnt_d", "cnt_h", "zd"):
+        setattr(a, f, base)
+    a.B, a.topk, a.E, a.H, a.I = 1, 8, 256, 6144, 2048
+    a.cfg_gu = (C.c_int32 * 4)(1, 4, 12, 0); a.cfg_dn = (C.c_int32 * 4)(1, 4, 4, 0)
+    a.which = 3
+    assert L.nq_moe_forward(C.byref(a), None) != 0 and "workspace too small" in err()
+    a.x = base + 2
+    assert L.nq_moe_forward(C.byref(a), None) != 0 and "16-byte aligned" in err()
+    a.x = base; a.B = 9
+    assert L.nq_moe_forward(C.byref(a), None) != 0 and "B=9" in err()
+    a.B = 1; a.cfg_gu = (C.c_int32 * 4)(1, 3, 12, 0)
+    assert L.nq_moe_forward(C.byref(a), None) != 0 and "bad cfg" in err()
+    a.cfg_gu = (C.c_int32 * 4)(1, 4, 12, 0); a.G = 3
+    a.acc_gu_elems = a.acc_d_elems = a.h_elems = a.out_elems = a.cnt_gu_elems = a.cnt_d_elems = a.cnt_h_elems = a.zd_elems = 1 << 40
+    assert L.nq_moe_forward(C.byref(a), None) != 0 and "G=3" in err()
+    a.G = 0; a.common_rows = 2
+    assert L.nq_moe_forward(C.byref(a), None) != 0 and "common_rows" in err()
+    assert L.nq_pf_plan(base, 256, 0, 1024, base, 256, None) != 0 and "cap" in err()
+    assert L.nq_pf_plan(base, 256, 0, 1024, base + 4, 512, None) != 0 and "aligned" in err()
+    assert L.nq_pf_gemm(base, base, 1, 48, 0, base, base, base, 4, 256, 256, None) != 0 and "tile height" in err()
+    assert L.nq_pf_gemm(base, base, 1, 16, 0, base + 8, base, base, 4, 256, 256, None) != 0 and "aligned" in err()
+    assert L.nq_pf_pre(base + 2, base, base, 1, base, base, base, None, 4, 256, 256, None) != 0 and "aligned" in err()
+    assert L.nq_sal(base, 0, 64, base, 0, base, 0, 9, 64, 8, 16, 1.0, base, base, None) != 0 and "at most 8" in err()
+    assert L.nq_dequant(base, 2, 0, 256, 256, base, None) != 0 and "proj" in err()
+    assert L.nq_mailbox(None, base, base, base, None, 4, None) != 0 and "null" in err()
