@@ -383,6 +383,7 @@ template <int MODE, bool ANYROW>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) nq_gemv_k(MoeArgs a, int NC)
 {
     extern __shared__ __align__(16) char smem[];
+    __builtin_amdgcn_s_setprio(3);                               // routing and staging are chains of latencies (see progress_priority)
     __shared__ RunInfo R;
     __shared__ int last;
     const int lane = threadIdx.x & 63, warp = threadIdx.x >> 6, SB = blockDim.x >> 6;
@@ -486,6 +487,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
     }
     else if (R.level == 2) gemv_chunks<false, 0, 0, false>(P, L, NC, acc, nb0);
     else dispatch_code(P.code, [&](auto tag) { gemv_chunks<true, decltype(tag)::value, 0, false>(P, L, NC, acc, nb0); });
+
+    __builtin_amdgcn_s_setprio(3);                               // the tail is a chain of latencies: nothing should wait behind decoders
 
     // ---- k-slice partial sums: lane (t4, n) holds rows 16 (strip0 + t4 / 2) + 4 (t4 & 1) + i (+ 8 for acc[1]) of token n
     if (n < ntok)

@@ -150,7 +150,7 @@ class MoELayer:
             nc = max(d for d in range(1, want + 1) if C % d == 0)
             sb = max(d for d in (4, 2, 1) if (N // 32) % d == 0 and (I // 32) % d == 0)
             return [1, sb, nc]
-        return pick(H // 128, 2 * I, 12), pick(I // 128, H, 4)
+        return pick(H // 128, 2 * I, 12), pick(I // 128, H, 8)
 
     def _ny(s, cfg, C):
         return C // (cfg[0] * cfg[2])
