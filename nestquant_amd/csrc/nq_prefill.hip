@@ -457,6 +457,7 @@ __device__ __forceinline__ void pf_chunks(const Planes& P, const LaneCtx& L, int
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");         // this wavefront's share of the tile has landed
         __syncthreads();
+        __builtin_amdgcn_s_setprio(3);                           // MFMA phase first: see below
         // ---- TG x 8 MFMAs: tokens 16 tg + n as the N dimension (row groups beyond the tile multiply stale LDS rows whose
         // results are never stored). Two row groups are interleaved so that four different accumulators separate an MFMA
         // from the next one that depends on it.
@@ -506,6 +507,7 @@ __device__ __forceinline__ void pf_chunks(const Planes& P, const LaneCtx& L, int
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
+        __builtin_amdgcn_s_setprio(0);
         __syncthreads();                                         // every wavefront has read chunk c before chunk c + 1 overwrites it
     }
 }
