@@ -121,6 +121,29 @@ def unpack_words(t, nrec, bits):
     return w
 
 
+def lane_words_from_rings(raw, bits, G=4):
+    """Ring streams -> lane records (the repack step of the reference's shard loader, sm120/nqload.py:51-55, and the inverse
+    of sm120/ref15_spec.py:132-137). raw: uint8, per unit 32 / G rings of G * bits bits each, LSB-first within every byte;
+    lane l of a ring holds the stream's bits [l * bits, (l + 1) * bits). -> int64 [records, ceil(bits / 32)] (uint32 values),
+    records in (unit, ring, lane) order, the layout pack_words() takes."""
+    raw = torch.as_tensor(raw, dtype=torch.uint8).reshape(-1)
+    per_unit = 32 * bits // 8
+    assert (G * bits) % 8 == 0 and raw.numel() % per_unit == 0, (bits, G, raw.numel())
+    dev = raw.device
+    b = ((raw.long()[:, None] >> torch.arange(8, device=dev)) & 1).reshape(-1, bits)           # one row per record
+    nw = (bits + 31) // 32
+    b = torch.nn.functional.pad(b, (0, nw * 32 - bits)).reshape(-1, nw, 32)
+    return (b << torch.arange(32, device=dev)).sum(-1)
+
+
+def rings_from_lane_words(w, bits, G=4):
+    """inverse of lane_words_from_rings: int64 [records, NW] -> uint8 ring streams [records / G, G * bits / 8]"""
+    dev = w.device
+    b = ((w[:, :, None] >> torch.arange(32, device=dev)) & 1).reshape(w.shape[0], -1)[:, :bits]
+    b = b.reshape(-1, G * bits // 8, 8)
+    return (b << torch.arange(8, device=dev)).sum(-1).to(torch.uint8)
+
+
 _MBN = None
 
 

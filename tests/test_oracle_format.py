@@ -207,3 +207,30 @@ def test_mailbox_state_machine():
     assert O.mailbox_apply(table, stage, seq, applied) == 1
     assert np.array_equal(table[1], stage[1]) and not table[[0, 2, 3]].any() and np.array_equal(applied, seq)
     assert O.mailbox_apply(table, stage, seq, applied) == 0
+
+
+@pytest.mark.parametrize("code", [0, 1, 3, 7, 9])
+def test_ring_streams_to_lane_words(code):
+    """the loader's repack step (ring byte streams -> lane records) against a window walk done directly on the byte streams:
+    state p of a ring = the 16 bits at step_off(p) of its tail-biting stream, LSB-first bytes"""
+    import torch
+    from nestquant_amd import format as F
+    rng = np.random.default_rng(300 + code)
+    bits = O.rbits(code); ka, mask = O.RKP[code]
+    nrings = 24
+    raw = rng.integers(0, 256, (nrings, 4 * bits // 8), dtype=np.uint8)
+    w = F.lane_words_from_rings(torch.from_numpy(raw.reshape(-1)), bits)
+    assert w.shape == (nrings * 4, (bits + 31) // 32) and int(w.max()) < 2**32
+    if bits % 32:
+        assert int(w[:, -1].max()) < 1 << (bits % 32)
+    assert np.array_equal(F.rings_from_lane_words(w, bits).numpy(), raw)
+    # direct walk over the bytes, no lane view involved
+    L = 4 * bits
+    stream = np.unpackbits(raw, axis=1, bitorder="little").astype(np.int64)          # [rings, L]
+    off = np.asarray(O.step_off(np.arange(256), ka, mask))
+    idx = (off[:, None] + np.arange(16)) % L
+    states = (stream[:, idx] << np.arange(16)).sum(-1)                                 # [rings, 256]
+    assert np.array_equal(O.ring_states(w.numpy().astype(np.uint32), code), states)
+    assert np.array_equal(O.lane_sums(w.numpy().astype(np.uint32), code).reshape(nrings, 256), O.hash_sum(states))
+    # and through the packer: pack_words -> unpack_words gives the records back
+    assert torch.equal(F.unpack_words(F.pack_words(w, bits), nrings * 4, bits), w)
