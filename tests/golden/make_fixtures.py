@@ -43,6 +43,18 @@ def base_code(R):
                             W2=W2.numpy().view(np.uint16), W4=W4.numpy().view(np.uint16))
 
 
+def rings_of_two(R):
+    """8. the same planes read as rings of G = 2 lanes (the reference kernel's second variant, sm120/nqmoe.cu:223-228):
+    the reference's dense decode with G = 2 at levels 2 and 4"""
+    for rk in (0, 7):
+        seed = 4000 + rk
+        gen = torch.Generator().manual_seed(seed)
+        p = R.Proj(32, 256, gen, None, rk, ("exh", 500 * rk + 9))
+        np.savez_compressed(os.path.join(OUT, f"proj_g2_rk{rk}.npz"), seed=seed, N=32, K=256, rk=rk, mbn_offset=500 * rk + 9,
+                            W2=R.dense_W(p, 2, 2, torch.float16).numpy().view(np.uint16),
+                            W4=R.dense_W(p, 4, 2, torch.float16).numpy().view(np.uint16))
+
+
 def main():
     R, SP = load_reference()
 
@@ -149,11 +161,14 @@ def main():
         np.savez_compressed(os.path.join(OUT, f"mask_rk{rk}.npz"), seed=2000 + rk, N=256, K=384, nm=1, rk=rk, mbn_offset=900 * rk + 5,
                             var=int(var), flags=p.flags.numpy(), W4=W4.numpy().view(np.uint16))
     base_code(R)
+    rings_of_two(R)
     print("fixtures written to", OUT)
 
 
 if __name__ == "__main__":
     if sys.argv[1:] == ["base_code"]:            # only the fixtures of section 7
         base_code(load_reference()[0])
+    elif sys.argv[1:] == ["rings_of_two"]:       # only the fixtures of section 8
+        rings_of_two(load_reference()[0])
     else:
         main()

@@ -199,3 +199,14 @@ def test_base_code_1_matches_reference(path):
     assert np.array_equal(O.lane_sums(op.base, 1), O.hash_sum(O.ring_states(op.base, 1)).reshape(-1, 64))
     wrong = O.Plane(N, K, np.concatenate([op.base, op.base], 0)[: op.base.shape[0]], rk=rk, res=op.res, d4=op.d4, var=op.var, bk=0)
     assert same_f16(O.dense_W(wrong, 2), z["W2"].view(np.float16)) > 1000
+
+
+@pytest.mark.parametrize("rk", [0, 7])
+def test_rings_of_two_lanes_match_reference(rk):
+    """the same planes read as rings of G = 2 records: the reference's dense_W(p, level, G=2) at levels 2 and 4"""
+    z = np.load(os.path.join(GOLD, f"proj_g2_rk{rk}.npz"))
+    gen = torch.Generator().manual_seed(int(z["seed"]))
+    p = oracle_plane(F.Proj(int(z["N"]), int(z["K"]), gen, None, rk, ("exh", int(z["mbn_offset"]))))
+    assert same_f16(O.dense_W(p, 2, G=2), z["W2"].view(np.float16)) == 0
+    assert same_f16(O.dense_W(p, 4, G=2), z["W4"].view(np.float16)) == 0
+    assert same_f16(O.dense_W(p, 4), z["W4"].view(np.float16)) > 1000      # the G = 4 reading is another matrix
