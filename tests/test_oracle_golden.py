@@ -209,4 +209,5 @@ def test_rings_of_two_lanes_match_reference(rk):
     p = oracle_plane(F.Proj(int(z["N"]), int(z["K"]), gen, None, rk, ("exh", int(z["mbn_offset"]))))
     assert same_f16(O.dense_W(p, 2, G=2), z["W2"].view(np.float16)) == 0
     assert same_f16(O.dense_W(p, 4, G=2), z["W4"].view(np.float16)) == 0
-    assert same_f16(O.dense_W(p, 4), z["W4"].view(np.float16)) > 1000      # the G = 4 reading is another matrix
+    # the G = 4 reading differs where a window crosses the end of a record whose ring neighbour changed (lanes 1 and 3)
+    assert same_f16(O.dense_W(p, 4), z["W4"].view(np.float16)) > 100
