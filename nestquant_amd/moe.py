@@ -118,8 +118,9 @@ class MoELayer:
     Same constructor, attributes and call signature as the reference's MoELayer (sm120/moe.py:231-260). Differences that
     a caller can observe: acc_gu / acc_d hold per-k-slice partial sums ([NY, S, 2I] and [NY, S, H]) instead of
     atomically accumulated [S, 2I] / [S, H], so they are not zero between calls and outputs are bitwise repeatable;
-    cnt_gu / cnt_d are the arrival counters (zero on entry, zero on exit); wq, zd, cnt_h exist for attribute
-    compatibility and stay zero."""
+    cnt_gu / cnt_d / cnt_h are arrival counters (zero on entry, zero on exit; cnt_h counts the 128-column groups of a
+    512-column block when in_had_down = 512); zd carries the low-rank plane's z_d partial sums from the gate|up launch to
+    the down launch and needs no zeroing; wq exists for attribute compatibility only (no work queue here) and stays zero."""
 
     def __init__(s, E, H, I, nm_gu=0, nm_dn=0, Bmax=4, topk=8, G=4, dev="cuda", mod=None):
         if G not in (4, 2):
