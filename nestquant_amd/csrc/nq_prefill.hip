@@ -461,7 +461,7 @@ __device__ __forceinline__ void pf_chunks(const Planes& P, const LaneCtx& L, int
         // ---- TG x 8 MFMAs: tokens 16 tg + n as the N dimension (row groups beyond the tile multiply stale LDS rows whose
         // results are never stored). Two row groups are interleaved so that four different accumulators separate an MFMA
         // from the next one that depends on it.
-        constexpr int TS = TG >= 2 ? 2 : 1, NGRP = TG / TS * 4, PD = TG >= 16 ? 2 : 1;      // read-ahead depth in groups
+        constexpr int TS = TG >= 2 ? 2 : 1, NGRP = TG / TS * 4, PD = 1;      // read-ahead depth in groups
         if constexpr (PD == 0)
         {
 #pragma unroll
