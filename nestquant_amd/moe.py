@@ -245,6 +245,31 @@ def pf_tiles(segs):
     return {bm: torch.tensor(v, dtype=torch.int32) for bm, v in out.items() if v}
 
 
+_PF_SIDE = {}
+_PF_STREAM_OF = {256: 0, 128: 1, 64: 2, 32: 3, 16: 3}          # stream 0 = the caller's
+
+
+def _pf_gemms(Lb, tb, lists, variants, mode, A0, A1, Cm, E, H, I):
+    """The grouped-GEMM launches of one projection, one per tile height. The heights work on disjoint pair rows, and a launch
+    ends with the GPU partly idle while its last workgroups drain (a workgroup runs the whole K loop, ~75 us, so a launch of a
+    few dozen tiles is a handful of such rounds); the tallest height stays on the caller's stream and the others go to side
+    streams (default priority) between two events, so that the launches overlap and fill each other's tails: 7.3 -> 7.0 ms."""
+    main = torch.cuda.current_stream()
+    side = _PF_SIDE.setdefault(str(tb.device), [])
+    while len(side) < 3:
+        side.append(torch.cuda.Stream(device=tb.device))
+    streams = [main] + side
+    ready = torch.cuda.Event(); ready.record(main)
+    for st in side:
+        st.wait_event(ready)
+    for bm, t, nt in lists:
+        stp = C.c_void_p(streams[_PF_STREAM_OF[bm]].cuda_stream)
+        for v in variants:
+            _lib.check(Lb.nq_pf_gemm(tb.data_ptr(), t.data_ptr(), nt, bm, mode | v, A0, A1, Cm, E, H, I, stp))
+    for st in side:
+        done = torch.cuda.Event(); done.record(st); main.wait_event(done)
+
+
 def prefill(s, x, sel, rw, out=None, R=None, G=None, table=None):
     """T > Bmax tokens (reference sm120/moe.py:282-326): pairs sorted by expert, each routed expert decoded inside the
     grouped GEMMs at the level of its live table row, same math as the decode path (fp32 accumulation order differs).
@@ -287,16 +312,10 @@ def prefill(s, x, sel, rw, out=None, R=None, G=None, table=None):
         pts, pes = pt[c:d], pe[c:d]
         _lib.check(Lb.nq_pf_pre(x.data_ptr(), pts.data_ptr(), pes.data_ptr(), n, tb.data_ptr(), S["xg"].data_ptr(),
                                 S["xu"].data_ptr(), S["zg"].data_ptr(), E, H, I, st))
-        for bm, t, nt in lists:
-            for v in variants:
-                _lib.check(Lb.nq_pf_gemm(tb.data_ptr(), t.data_ptr(), nt, bm, v, S["xg"].data_ptr(), S["xu"].data_ptr(),
-                                         S["acc"].data_ptr(), E, H, I, st))
+        _pf_gemms(Lb, tb, lists, variants, 0, S["xg"].data_ptr(), S["xu"].data_ptr(), S["acc"].data_ptr(), E, H, I)
         _lib.check(Lb.nq_pf_mid(S["acc"].data_ptr(), pes.data_ptr(), n, tb.data_ptr(), S["h"].data_ptr(), S["zg"].data_ptr(),
                                 S["zd"].data_ptr(), E, H, I, st))
-        for bm, t, nt in lists:
-            for v in variants:
-                _lib.check(Lb.nq_pf_gemm(tb.data_ptr(), t.data_ptr(), nt, bm, 1 | v, S["h"].data_ptr(), None,
-                                         S["y"].data_ptr(), E, H, I, st))
+        _pf_gemms(Lb, tb, lists, variants, 1, S["h"].data_ptr(), None, S["y"].data_ptr(), E, H, I)
         _lib.check(Lb.nq_pf_post(S["y"].data_ptr(), pos.data_ptr(), selc.data_ptr(), rwc.data_ptr(), T, k, c, n, tb.data_ptr(),
                                  out.data_ptr(), S["zd"].data_ptr(), E, H, I, st))
     return out
