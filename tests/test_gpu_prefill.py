@@ -139,3 +139,27 @@ def test_device_tile_planner_matches_host_lists():
             assert total == n
     with pytest.raises(RuntimeError, match="cap"):
         _lib.check(_lib.lib().nq_pf_plan(cnt.to(DEV).data_ptr(), 64, 0, 1024, tiles.data_ptr(), 64, None))
+
+
+def test_prefill_on_a_side_stream_matches_the_default_stream():
+    """prefill() forks its grouped-GEMM launches onto side streams and joins them again: the result must not depend on which
+    stream the caller is on, nor on work the caller queued right before and after it"""
+    H, I, NE, T = 512, 256, 8, 200
+    ex = to_dev(experts_on_gpu(H, I, NE, 640, rk=[(3, 9)] * NE))
+    L = M.MoELayer(NE, H, I, Bmax=8, topk=4)
+    for e in range(NE):
+        L.set(e, ex[e], (4, 2, 4, 4, 2, 4, 0, 4)[e])
+    sel, rw = gumbel_topk(T, NE, 4, seed=3)
+    g = torch.Generator().manual_seed(4)
+    x = (torch.randn(T, H, generator=g) * 0.05).half().to(DEV)
+    want = L.prefill(x, sel, rw).clone()
+    torch.cuda.synchronize()
+    s2 = torch.cuda.Stream()
+    with torch.cuda.stream(s2):
+        x2 = x * 1.0                                                # produced on the side stream just before the call
+        got = L.prefill(x2, sel, rw)
+        got2 = got * 2.0                                            # consumed on it right after
+    s2.synchronize()
+    assert torch.equal(got, want) and torch.equal(got2, want * 2.0)
+    for _ in range(3):                                              # back to back: the scratch is reused, nothing overtakes
+        assert torch.equal(L.prefill(x, sel, rw), want)
