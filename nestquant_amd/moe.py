@@ -274,7 +274,8 @@ def prefill(s, x, sel, rw, out=None, R=None, G=None, table=None):
     """T > Bmax tokens (reference sm120/moe.py:282-326): pairs sorted by expert, each routed expert decoded inside the
     grouped GEMMs at the level of its live table row, same math as the decode path (fp32 accumulation order differs).
     No host synchronisation (the reference's prefill reads the expert counts back; here the tile lists are built on the
-    device by nq_pf_plan). Exports routing hits like the decode kernel."""
+    device by nq_pf_plan). Exports routing hits like the decode kernel. Calls on one device share the scratch of pf_scratch()
+    (as the reference's do, sm120/moe.py:262-274) and the side streams of _pf_gemms, so they must be ordered on one stream."""
     if s.G != 4:
         raise NotImplementedError("prefill decodes rings of G = 4 lanes only (as the reference's pf_decode)")
     assert x.dtype == torch.float16 and rw.dtype == torch.float16 and sel.dtype == torch.int64, (x.dtype, rw.dtype, sel.dtype)
