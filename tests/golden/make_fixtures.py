@@ -55,6 +55,28 @@ def rings_of_two(R):
                             W4=R.dense_W(p, 4, 2, torch.float16).numpy().view(np.uint16))
 
 
+def shard_loader():
+    """9. the production shard loader (sm120/nqload.py: group_art + kernel_expert on the CPU): synthetic shards of
+    tests/shards.py (seeded, so the fixture stores the outputs only), the group of rank 1 of 4 (shards 2, 3)"""
+    sys.path.insert(0, os.path.dirname(os.path.dirname(OUT)))
+    from tests.shards import synth_layer
+    import nqload as NL          # imports the reference's nq_decode (torch only at import) and moe (stubbed build)
+    cases = {"a": dict(seed=5101, H=128, res_K=2.25, base_K=2, var=True, rg=2, rd=1),
+             "b": dict(seed=5102, H=128, res_K=2.5625, base_K=1.75, var=True, rg=0, rd=0)}
+    for name, kw in cases.items():
+        man, parts = synth_layer(**kw)
+        ex = NL.kernel_expert(NL.group_art(parts, man, 0, [2, 3]), dev="cpu")[0]
+        out = dict(I=ex.I, **{k: np.array(v) for k, v in kw.items()})
+        for pn, p in (("gu", ex.gu), ("dn", ex.dn)):
+            out.update({f"{pn}_base": p.base.numpy(), f"{pn}_p4": p.p4.numpy(), f"{pn}_d4": p.d4.numpy(), f"{pn}_var": p.var.numpy(),
+                        f"{pn}_rk": p.rk, f"{pn}_bk": p.bk})
+        out.update(sc2=ex.sc[2].numpy().view(np.uint16), sc4=ex.sc[4].numpy().view(np.uint16))
+        if ex.lr is not None:
+            out.update(lr=ex.lr.numpy().view(np.uint16), lr4=ex.lr4.numpy().view(np.uint16))
+        out["p4_bytes"] = NL.p4_bytes(ex)
+        np.savez_compressed(os.path.join(OUT, f"shards_{name}.npz"), **out)
+
+
 def main():
     R, SP = load_reference()
 
@@ -162,6 +184,7 @@ def main():
                             var=int(var), flags=p.flags.numpy(), W4=W4.numpy().view(np.uint16))
     base_code(R)
     rings_of_two(R)
+    shard_loader()
     print("fixtures written to", OUT)
 
 
@@ -170,5 +193,7 @@ if __name__ == "__main__":
         base_code(load_reference()[0])
     elif sys.argv[1:] == ["rings_of_two"]:       # only the fixtures of section 8
         rings_of_two(load_reference()[0])
+    elif sys.argv[1:] == ["shard_loader"]:       # only the fixtures of section 9
+        load_reference(); shard_loader()
     else:
         main()

@@ -2,11 +2,14 @@
 gives bitwise the outputs of the same experts set into a layer directly, in the decode path and in prefill."""
 import types
 
+import numpy as np
 import pytest
 import torch
 
-from nestquant_amd import format as F, moe as M, p4rec, resident
+from nestquant_amd import format as F, moe as M, nqload, p4rec, resident
+from tests.shards import synth_layer, write_layer
 from tests.test_formats import _lr_expert, _rank_layer
+from tests.util import O, oracle_plane, rel_err
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
@@ -71,3 +74,56 @@ def test_layer_from_resident_file_and_record_slots(tmp_path):
     st = torch.stack([torch.randperm(E, generator=g)[:topk] for _ in range(T)]).to(DEV)
     wt = torch.softmax(torch.randn(T, topk, generator=g), -1).half().to(DEV)
     assert torch.equal(served.prefill(xt, st, wt), direct.prefill(xt, st, wt))
+
+
+@pytest.mark.parametrize("base_K,res_K,container", [(2, 2.25, "safetensors"), (1.75, 2.5625, "pt")])
+def test_layer_from_production_shards_matches_the_oracle(tmp_path, base_K, res_K, container):
+    """shard files -> nqload.RankLayer (rank 1 of 4) -> table rows -> decode path and prefill, against the oracle's layer over
+    the oracle's dense decode of the loaded planes, with the low-rank factors taken from the shards themselves"""
+    Hh, topk, B = 256, 2, 3
+    ids = (4, 9, 17)
+    man, parts = synth_layer(seed=71, H=Hh, res_K=res_K, base_K=base_K, var=True, rg=2, rd=1, experts=ids, had_dn=512)
+    write_layer(str(tmp_path), 3, man, parts, container)
+    RL = nqload.RankLayer(str(tmp_path), 3, rank=1, tp=4, dev=DEV)
+    H, I = RL.H, RL.I
+    assert (H, I, RL.had_dn) == (Hh, 512, 512)
+    levels = [2, 4, 4]
+    layer = M.MoELayer(len(ids), H, I, Bmax=B, topk=topk)
+    for e, E in enumerate(ids):
+        row = M.entry(RL.ex[E], levels[e])
+        if levels[e] == 4:
+            row[9] = RL.ex[E].sc[4].data_ptr()
+        M.validate_row(row, H, I)
+        layer.table[e].copy_(row.to(DEV))
+    layer.rare_rows = base_K != 2
+    # dequant of a loaded projection is bit-exact against the oracle's decode of the same planes
+    for e, E in enumerate(ids):
+        for proj, p in ((0, RL.ex[E].gu), (1, RL.ex[E].dn)):
+            got = M.dequant(layer.table[e], proj, H, I, levels[e]).cpu().numpy()
+            assert np.array_equal(got.view(np.uint16), O.dense_W(oracle_plane(p), levels[e]).astype(np.float16).view(np.uint16))
+
+    def lr_of(e):
+        a = RL.art(ids[e])
+        f = lambda t: t.numpy().astype(np.float16)
+        return dict(Vg=f(a["gate"]["base"]["lr"]["V"]), U2g=f(a["gate"]["base"]["lr"]["U2"]), U2u=f(a["up"]["base"]["lr"]["U2"]),
+                    U4g=f(a["gate"]["p4"]["lr"]["U4"]), U4u=f(a["up"]["p4"]["lr"]["U4"]), Vd=f(a["down"]["base"]["lr"]["V"]),
+                    U2d=f(a["down"]["base"]["lr"]["U2"]), U4d=f(a["down"]["p4"]["lr"]["U4"]))
+
+    dense = lambda e: (O.dense_W(oracle_plane(RL.ex[ids[e]].gu), levels[e]).astype(np.float32),
+                       O.dense_W(oracle_plane(RL.ex[ids[e]].dn), levels[e]).astype(np.float32))
+    signs = lambda e: RL.ex[ids[e]].sc[levels[e]].cpu().numpy()
+    g = torch.Generator().manual_seed(5)
+    x = (torch.randn(B, H, generator=g) * 0.5).half()
+    sel = torch.stack([torch.randperm(len(ids), generator=g)[:topk] for _ in range(B)])
+    rw = torch.softmax(torch.randn(B, topk, generator=g), -1).half()
+    want = O.moe_forward(dense, levels, signs, x.numpy(), sel.numpy(), rw.numpy(), dtype=np.float64, had_dn=512, lr=lr_of)
+    y = layer(x.to(DEV), sel.to(DEV), rw.to(DEV)).cpu().numpy()
+    assert np.isfinite(y).all() and rel_err(y, want) < 1e-3
+    no_lr = O.moe_forward(dense, levels, signs, x.numpy(), sel.numpy(), rw.numpy(), dtype=np.float64, had_dn=512)
+    assert rel_err(no_lr, want) > 1e-2                  # the low-rank plane matters in this layer
+    T = 24
+    xt = (torch.randn(T, H, generator=g) * 0.5).half()
+    st = torch.stack([torch.randperm(len(ids), generator=g)[:topk] for _ in range(T)])
+    wt = torch.softmax(torch.randn(T, topk, generator=g), -1).half()
+    want = O.moe_forward(dense, levels, signs, xt.numpy(), st.numpy(), wt.numpy(), dtype=np.float64, had_dn=512, lr=lr_of)
+    assert rel_err(layer.prefill(xt.to(DEV), st.to(DEV), wt.to(DEV)).cpu().numpy(), want) < 1e-3

@@ -23,7 +23,7 @@ def oracle_plane(p):
     nrec = p.z["S"] * p.z["C"] * 32
     res = O.unpack_words(p.p4.cpu().numpy(), p.z["nrec_r"], O.rbits(p.rk))
     kw = {}
-    if p.nested:
+    if getattr(p, "nested", False):
         kw = dict(p3=O.unpack_words(p.p3.cpu().numpy(), nrec, 64), d3=u32(p.d3),
                   p4n=O.unpack_words(p.p4n.cpu().numpy(), nrec, 64), d4n=u32(p.d4n))
     bk = int(getattr(p, "bk", 0) or 0)
