@@ -1,12 +1,14 @@
 """A layer served from the on-disk formats (resident file + level-4 records in a slot pool, promoted through the mailbox)
 gives bitwise the outputs of the same experts set into a layer directly, in the decode path and in prefill."""
+import json
+import os
 import types
 
 import numpy as np
 import pytest
 import torch
 
-from nestquant_amd import format as F, moe as M, nqload, p4rec, resident
+from nestquant_amd import format as F, moe as M, nqload, p4rec, repack, resident
 from tests.shards import synth_layer, write_layer
 from tests.test_formats import _lr_expert, _rank_layer
 from tests.util import O, oracle_plane, rel_err
@@ -127,3 +129,58 @@ def test_layer_from_production_shards_matches_the_oracle(tmp_path, base_K, res_K
     wt = torch.softmax(torch.randn(T, topk, generator=g), -1).half()
     want = O.moe_forward(dense, levels, signs, xt.numpy(), st.numpy(), wt.numpy(), dtype=np.float64, had_dn=512, lr=lr_of)
     assert rel_err(layer.prefill(xt.to(DEV), st.to(DEV), wt.to(DEV)).cpu().numpy(), want) < 1e-3
+
+
+def test_layer_served_from_repacked_files_equals_the_shards_served_directly(tmp_path):
+    """shards -> repack -> (resident file, record file, index) -> level-2 rows + records read into pinned staging, copied into
+    slots on a side stream and promoted through the mailbox: bitwise the layer whose rows point at the loaded planes"""
+    root, out = str(tmp_path / "fit"), str(tmp_path / "out")
+    ids, L, rank, tp, topk, B = (0, 3, 4, 6), 7, 2, 4, 2, 4
+    man, parts = synth_layer(seed=91, H=256, res_K=2.3125, var=True, rg=1, rd=2, experts=ids, had_dn=512)
+    write_layer(root, L, man, parts, "safetensors")
+    assert repack.repack(root, out, tp=tp, layers=[L], dev=DEV, ne=8, log=lambda s: None) == [(L, r) for r in range(tp)]
+    RL = nqload.RankLayer(root, L, rank, tp, dev=DEV)
+    H, I = RL.H, RL.I
+    levels = {0: 4, 3: 2, 4: 4, 6: 4}
+    direct = M.MoELayer(8, H, I, Bmax=B, topk=topk)
+    for E in ids:
+        row = M.entry(RL.ex[E], levels[E])
+        if levels[E] == 4:
+            row[9] = RL.ex[E].sc[4].data_ptr()
+        M.validate_row(row, H, I)
+        direct.table[E].copy_(row.to(DEV))
+
+    with open(f"{out}/rank{rank}.json") as f:
+        idx = json.load(f)
+    lay = dict(seg={k: tuple(v) for k, v in idx["seg"].items()}, rec_bytes=idx["rec_bytes"])
+    got, h, i = resident.load(f"{out}/res/rank{rank}/L{L}.pt", DEV)
+    assert (h, i) == (H, I) and got[0].had_dn == 512
+    served = M.MoELayer(8, H, I, Bmax=B, topk=topk)
+    for E in ids:
+        served.set(E, got[E], 2)
+    mb = M.Mailbox(served)
+    up = [E for E in ids if levels[E] == 4]
+    pool = torch.zeros(len(up), idx["rec_bytes"], dtype=torch.uint8, device=DEV)
+    stage = torch.empty(len(up), idx["rec_bytes"], dtype=torch.uint8).pin_memory()
+    side = torch.cuda.Stream()
+    fd = os.open(f"{out}/rank{rank}.bin", os.O_RDONLY)
+    try:
+        for slot, E in enumerate(up):
+            repack.read_record(fd, idx, L, E, stage[slot])
+            with torch.cuda.stream(side):
+                pool[slot].copy_(stage[slot], non_blocking=True)
+            mb.post(E, p4rec.row(got[E], lay, pool[slot].data_ptr(), M.entry), side)
+    finally:
+        os.close(fd)
+    side.synchronize()
+    g = torch.Generator().manual_seed(3)
+    x = (torch.randn(B, H, generator=g) * 0.5).half().to(DEV)
+    sel = torch.stack([torch.tensor(ids)[torch.randperm(len(ids), generator=g)[:topk]] for _ in range(B)]).to(DEV)
+    rw = torch.softmax(torch.randn(B, topk, generator=g), -1).half().to(DEV)
+    mb.apply()
+    y = served(x, sel, rw).clone()
+    want = direct(x, sel, rw).clone()
+    torch.cuda.synchronize()
+    assert [int(served.table[E, 0]) for E in ids] == [levels[E] for E in ids]
+    assert torch.isfinite(want).all() and want.abs().max() > 0 and torch.equal(y, want)
+    assert not torch.equal(served(x, sel, rw, force_level=2), want)
