@@ -125,6 +125,15 @@ int nq_sal(const void* x, int x_dtype, int64_t x_row_stride, const void* w, int 
 int nq_pf_pre(const void* x_f16, const int32_t* pt, const int32_t* pe, int np, const int64_t* table, void* xg_f16,
               void* xu_f16, float* zg, int E, int H, int I, void* stream);
 
+/* nq_pf_pre for the pair rows of some tile heights only: tiles / cap are the lists nq_pf_plan wrote for the same rows,
+ * heights a bit mask (bit k = height 16 << k); a row is worked on when the tile that holds it has one of these heights, the
+ * other rows of xg, xu and zg are left alone. With this and nq_pf_mid_rows the kernels of one tile height (pre, gate|up
+ * GEMM, mid, down GEMM) form a chain of their own, so the heights can run on concurrent streams between nq_pf_plan and
+ * nq_pf_post. The reference's pf_pre has no such restriction (its grouped GEMMs run one after the other,
+ * sm120/moe.py:303-324). */
+int nq_pf_pre_rows(const void* x_f16, const int32_t* pt, const int32_t* pe, int np, const int64_t* table, void* xg_f16,
+                   void* xu_f16, float* zg, int E, int H, int I, const int32_t* tiles, int cap, int heights, void* stream);
+
 /* Grouped GEMM with the weights decoded from the trellis planes inside the kernel (level and planes from the live table
  * row): for every tile t = tiles[t] = {expert, first pair row, rows, 0} (device int32[ntiles][4], rows <= bm,
  * bm in {16, 32, 64, 128, 256}):  C[row][n] = sum_k A[row][k] * W_expert[n][k]  with fp32 accumulation and output.
@@ -141,6 +150,11 @@ int nq_pf_gemm(const int64_t* table, const int32_t* tiles, int ntiles, int bm, i
  * V_dn^T, fp32 [np][4] (zg, zd may be NULL). Replaces pf_mid (reference sm120/nqmoe.cu:1119-1203,1268-1277). */
 int nq_pf_mid(const float* acc_gu, const int32_t* pe, int np, const int64_t* table, void* h_f16, const float* zg, float* zd,
               int E, int H, int I, void* stream);
+
+/* nq_pf_mid for the pair rows of some tile heights only (tiles, cap, heights as in nq_pf_pre_rows); the other rows of h and
+ * zd are left alone. The reference's pf_mid has no such restriction. */
+int nq_pf_mid_rows(const float* acc_gu, const int32_t* pe, int np, const int64_t* table, void* h_f16, const float* zg, float* zd,
+                   int E, int H, int I, const int32_t* tiles, int cap, int heights, void* stream);
 
 /* For every token t < T: out[t] += sum over its picks k whose pair row pos[t][k] lies in [row_lo, row_lo + nrows) of
  * rw[t][k] * sv_o (.) Hadamard(y[pos[t][k] - row_lo]). pos int32 [T][topk] = row of pair (t, k) in the expert-sorted

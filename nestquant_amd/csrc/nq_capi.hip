@@ -148,7 +148,19 @@ extern "C" int nq_pf_pre(const void* x, const int32_t* pt, const int32_t* pe, in
     NQ_REQUIRE(x && pt && pe && table && xg && xu, "nq_pf_pre: null pointer");
     NQ_REQUIRE(E >= 1 && shape_ok(H, I), "nq_pf_pre: E=%d H=%d I=%d (H, I positive multiples of 128)", E, H, I);
     NQ_REQUIRE(aligned16(x) && aligned16(xg) && aligned16(xu), "nq_pf_pre: x, xg and xu must be 16-byte aligned");
-    return launch_pf_pre(x, pt, pe, np, table, xg, xu, zg, E, H, I, (hipStream_t)stream);
+    return launch_pf_pre(x, pt, pe, np, table, xg, xu, zg, E, H, I, nullptr, 0, 0, (hipStream_t)stream);
+}
+
+extern "C" int nq_pf_pre_rows(const void* x, const int32_t* pt, const int32_t* pe, int np, const int64_t* table, void* xg, void* xu,
+                              float* zg, int E, int H, int I, const int32_t* tiles, int cap, int heights, void* stream)
+{
+    NQ_REQUIRE(np >= 0, "nq_pf_pre_rows: np=%d", np);
+    if (np == 0 || (heights & 31) == 0) return 0;
+    NQ_REQUIRE(x && pt && pe && table && xg && xu && tiles, "nq_pf_pre_rows: null pointer");
+    NQ_REQUIRE(E >= 1 && shape_ok(H, I), "nq_pf_pre_rows: E=%d H=%d I=%d (H, I positive multiples of 128)", E, H, I);
+    NQ_REQUIRE(aligned16(x) && aligned16(xg) && aligned16(xu) && aligned16(tiles), "nq_pf_pre_rows: x, xg, xu and tiles must be 16-byte aligned");
+    NQ_REQUIRE(cap >= E && (heights & ~31) == 0, "nq_pf_pre_rows: cap=%d below E=%d, or heights=0x%x outside the five tile heights", cap, E, heights);
+    return launch_pf_pre(x, pt, pe, np, table, xg, xu, zg, E, H, I, tiles, cap, heights, (hipStream_t)stream);
 }
 
 extern "C" int nq_pf_gemm(const int64_t* table, const int32_t* tiles, int ntiles, int bm, int mode, const void* A0, const void* A1,
@@ -173,7 +185,19 @@ extern "C" int nq_pf_mid(const float* acc_gu, const int32_t* pe, int np, const i
     NQ_REQUIRE(acc_gu && pe && table && h, "nq_pf_mid: null pointer");
     NQ_REQUIRE(E >= 1 && shape_ok(H, I), "nq_pf_mid: E=%d H=%d I=%d (H, I positive multiples of 128)", E, H, I);
     NQ_REQUIRE(aligned16(acc_gu) && aligned16(h), "nq_pf_mid: acc_gu and h must be 16-byte aligned");
-    return launch_pf_mid(acc_gu, pe, np, table, h, zg, zd, E, H, I, (hipStream_t)stream);
+    return launch_pf_mid(acc_gu, pe, np, table, h, zg, zd, E, H, I, nullptr, 0, 0, (hipStream_t)stream);
+}
+
+extern "C" int nq_pf_mid_rows(const float* acc_gu, const int32_t* pe, int np, const int64_t* table, void* h, const float* zg, float* zd,
+                              int E, int H, int I, const int32_t* tiles, int cap, int heights, void* stream)
+{
+    NQ_REQUIRE(np >= 0, "nq_pf_mid_rows: np=%d", np);
+    if (np == 0 || (heights & 31) == 0) return 0;
+    NQ_REQUIRE(acc_gu && pe && table && h && tiles, "nq_pf_mid_rows: null pointer");
+    NQ_REQUIRE(E >= 1 && shape_ok(H, I), "nq_pf_mid_rows: E=%d H=%d I=%d (H, I positive multiples of 128)", E, H, I);
+    NQ_REQUIRE(aligned16(acc_gu) && aligned16(h) && aligned16(tiles), "nq_pf_mid_rows: acc_gu, h and tiles must be 16-byte aligned");
+    NQ_REQUIRE(cap >= E && (heights & ~31) == 0, "nq_pf_mid_rows: cap=%d below E=%d, or heights=0x%x outside the five tile heights", cap, E, heights);
+    return launch_pf_mid(acc_gu, pe, np, table, h, zg, zd, E, H, I, tiles, cap, heights, (hipStream_t)stream);
 }
 
 extern "C" int nq_pf_post(const float* y, const int32_t* pos, const int64_t* sel, const void* rw, int T, int topk, int row_lo, int nrows,

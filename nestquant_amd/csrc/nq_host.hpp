@@ -40,8 +40,10 @@ int launch_moe(const MoeArgs& a, const int* cfg_gu, const int* cfg_dn, int which
 int launch_mailbox(int64_t* table, const int64_t* stage, const int32_t* seq, int32_t* applied, int32_t* applied_host, int E, hipStream_t st);
 int launch_dequant(const int64_t* row, int proj, int level, int H, int I, void* out, hipStream_t st);
 int launch_pf_decode(const int64_t* table, const int32_t* experts, int G, void* Wgu, void* Wdn, int H, int I, hipStream_t st);
-int launch_pf_pre(const void* x, const int32_t* pt, const int32_t* pe, int np, const int64_t* table, void* xg, void* xu, float* zg, int E, int H, int I, hipStream_t st);
-int launch_pf_mid(const float* acc_gu, const int32_t* pe, int np, const int64_t* table, void* h, const float* zg, float* zd, int E, int H, int I, hipStream_t st);
+int launch_pf_pre(const void* x, const int32_t* pt, const int32_t* pe, int np, const int64_t* table, void* xg, void* xu, float* zg, int E, int H, int I,
+                  const int32_t* tiles, int cap, int heights, hipStream_t st);
+int launch_pf_mid(const float* acc_gu, const int32_t* pe, int np, const int64_t* table, void* h, const float* zg, float* zd, int E, int H, int I,
+                  const int32_t* tiles, int cap, int heights, hipStream_t st);
 int launch_pf_post(const float* y, const int32_t* pos, const int64_t* sel, const void* rw, int T, int topk, int row_lo, int nrows,
                    const int64_t* table, float* out, const float* zd, int E, int H, int I, hipStream_t st);
 int launch_sal(const void* x, int x_dtype, int64_t sx, const void* w, int w_dtype, const void* ids, int ids_dtype, int T, int H, int K,

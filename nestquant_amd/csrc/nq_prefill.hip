@@ -38,13 +38,32 @@ __device__ __forceinline__ void wave_sync()
     __builtin_amdgcn_wave_barrier();
 }
 
-// grid (npairs), block 256: wave w handles the 512-column segments w, w + 4, ... of the pair's row, gate and up together
+// Is pair row p (of expert e) held by a tile of one of the heights in the bit mask `heights` (bit k = 16 << k)? tiles / cap:
+// the lists of nq_pf_plan_k. The remainder tile of expert e sits at index e of the list of its height and starts at its
+// first row; the rows before it belong to the expert's full 256-row tiles. Rows of no valid expert count as height 256.
+__device__ __forceinline__ bool row_in_heights(const int32_t* __restrict__ tiles, int cap, int heights, int p, int e, int E)
+{
+    int k = 4;
+    if (e >= 0 && e < E)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+        {
+            const int4 t = ((const int4*)tiles)[(size_t)q * cap + e];
+            if (t.x == e && p >= t.y) k = q;
+        }
+    return (heights >> k) & 1;
+}
+
+// grid (npairs), block 256: wave w handles the 512-column segments w, w + 4, ... of the pair's row, gate and up together.
+// tiles (optional): work only on the rows of the tile heights in `heights`
 __global__ void __launch_bounds__(256) nq_pf_pre_k(const _Float16* __restrict__ x, const int32_t* __restrict__ pt, const int32_t* __restrict__ pe,
-                                                    const int64_t* __restrict__ table, _Float16* xg, _Float16* xu, float* zg, int E, int H, int I)
+                                                    const int64_t* __restrict__ table, _Float16* xg, _Float16* xu, float* zg, int E, int H, int I,
+                                                    const int32_t* __restrict__ tiles, int cap, int heights)
 {
     __shared__ float zsh[4][4];
     const int p = blockIdx.x, lane = threadIdx.x & 63, warp = threadIdx.x >> 6;
     const int e = pe[p];
+    if (tiles && !row_in_heights(tiles, cap, heights, p, e, E)) return;       // block-uniform
     const int ng = H / 128;
     const bool live = e >= 0 && e < E && table[(size_t)e * TBL_W] > 0;
     const _Float16* signs = live ? (const _Float16*)table[(size_t)e * TBL_W + 9] : nullptr;
@@ -138,13 +157,16 @@ __global__ void __launch_bounds__(256) nq_pf_pre_k(const _Float16* __restrict__ 
 // grid (npairs), block 256: acc_gu [P][2I] fp32 (gate | up) -> h [P][I] fp16 in B-operand order. With in_had_down = 512
 // (table word 18) the four wavefronts hold the four 128-column groups of a 512-column block and combine their WHT_128
 // results through LDS with the Sylvester H_4 / 2 before the single rounding to fp16.
+// tiles (optional): work only on the rows of the tile heights in `heights`, as nq_pf_pre_k
 __global__ void __launch_bounds__(256) nq_pf_mid_k(const float* __restrict__ acc_gu, const int32_t* __restrict__ pe,
-                                                    const int64_t* __restrict__ table, _Float16* h, const float* zg, float* zd, int E, int H, int I)
+                                                    const int64_t* __restrict__ table, _Float16* h, const float* zg, float* zd, int E, int H, int I,
+                                                    const int32_t* __restrict__ tiles, int cap, int heights)
 {
     __shared__ float wsh[4][128];
     __shared__ float zsh[4][4];
     const int p = blockIdx.x, lane = threadIdx.x & 63, warp = threadIdx.x >> 6;
     const int e = pe[p];
+    if (tiles && !row_in_heights(tiles, cap, heights, p, e, E)) return;       // block-uniform
     const bool live = e >= 0 && e < E && table[(size_t)e * TBL_W] > 0;
     const _Float16* signs = live ? (const _Float16*)table[(size_t)e * TBL_W + 9] : nullptr;
     const bool wide = live && table[(size_t)e * TBL_W + 18] == 512;      // block-uniform
@@ -568,17 +590,19 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) n
     }
 }
 
-int launch_pf_pre(const void* x, const int32_t* pt, const int32_t* pe, int np, const int64_t* table, void* xg, void* xu, float* zg, int E, int H, int I, hipStream_t st)
+int launch_pf_pre(const void* x, const int32_t* pt, const int32_t* pe, int np, const int64_t* table, void* xg, void* xu, float* zg, int E, int H, int I,
+                  const int32_t* tiles, int cap, int heights, hipStream_t st)
 {
     if (!np) return 0;
-    nq_pf_pre_k<<<np, 256, 0, st>>>((const _Float16*)x, pt, pe, table, (_Float16*)xg, (_Float16*)xu, zg, E, H, I);
+    nq_pf_pre_k<<<np, 256, 0, st>>>((const _Float16*)x, pt, pe, table, (_Float16*)xg, (_Float16*)xu, zg, E, H, I, tiles, cap, heights);
     NQ_LAUNCH_CHECK("nq_pf_pre");
     return 0;
 }
-int launch_pf_mid(const float* acc_gu, const int32_t* pe, int np, const int64_t* table, void* h, const float* zg, float* zd, int E, int H, int I, hipStream_t st)
+int launch_pf_mid(const float* acc_gu, const int32_t* pe, int np, const int64_t* table, void* h, const float* zg, float* zd, int E, int H, int I,
+                  const int32_t* tiles, int cap, int heights, hipStream_t st)
 {
     if (!np) return 0;
-    nq_pf_mid_k<<<np, 256, 0, st>>>(acc_gu, pe, table, (_Float16*)h, zg, zd, E, H, I);
+    nq_pf_mid_k<<<np, 256, 0, st>>>(acc_gu, pe, table, (_Float16*)h, zg, zd, E, H, I, tiles, cap, heights);
     NQ_LAUNCH_CHECK("nq_pf_mid");
     return 0;
 }

@@ -249,11 +249,13 @@ _PF_SIDE = {}
 _PF_STREAM_OF = {256: 0, 128: 1, 64: 2, 32: 3, 16: 3}          # stream 0 = the caller's
 
 
-def _pf_gemms(Lb, tb, lists, variants, mode, A0, A1, Cm, E, H, I):
-    """The grouped-GEMM launches of one projection, one per tile height. The heights work on disjoint pair rows, and a launch
-    ends with the GPU partly idle while its last workgroups drain (a workgroup runs the whole K loop, ~75 us, so a launch of a
-    few dozen tiles is a handful of such rounds); the tallest height stays on the caller's stream and the others go to side
-    streams (default priority) between two events, so that the launches overlap and fill each other's tails: 7.3 -> 7.0 ms."""
+def _pf_chains(Lb, tb, lists, variants, S, x, pts, pes, n, tiles, cap, E, H, I):
+    """Everything between the tile plan and the post kernel of one row chunk: rotation of the activations, gate|up GEMM, SwiGLU
+    kernel and down GEMM of every tile height. The heights work on disjoint pair rows, so each is a chain of its own. A GEMM
+    launch ends with the GPU partly idle while its last workgroups drain (a workgroup runs the whole K loop, ~75 us, so a
+    launch of a few dozen tiles is a handful of such rounds); the tallest height stays on the caller's stream and the others
+    go to side streams (default priority) between two events, so that the chains overlap, fill each other's tails and the
+    memory-bound kernels of one height run under the GEMMs of another."""
     main = torch.cuda.current_stream()
     side = _PF_SIDE.setdefault(str(tb.device), [])
     while len(side) < 3:
@@ -262,10 +264,23 @@ def _pf_gemms(Lb, tb, lists, variants, mode, A0, A1, Cm, E, H, I):
     ready = torch.cuda.Event(); ready.record(main)
     for st in side:
         st.wait_event(ready)
-    for bm, t, nt in lists:
-        stp = C.c_void_p(streams[_PF_STREAM_OF[bm]].cuda_stream)
-        for v in variants:
-            _lib.check(Lb.nq_pf_gemm(tb.data_ptr(), t.data_ptr(), nt, bm, mode | v, A0, A1, Cm, E, H, I, stp))
+    xg, xu, acc, h, y, zg, zd = (S[k].data_ptr() for k in ("xg", "xu", "acc", "h", "y", "zg", "zd"))
+
+    def gemms(mode, A0, A1, Cm):
+        for bm, t, nt in lists:
+            stp = C.c_void_p(streams[_PF_STREAM_OF[bm]].cuda_stream)
+            for v in variants:
+                _lib.check(Lb.nq_pf_gemm(tb.data_ptr(), t.data_ptr(), nt, bm, mode | v, A0, A1, Cm, E, H, I, stp))
+
+    masks = [sum(bm // 16 for bm, _, _ in lists if _PF_STREAM_OF[bm] == i) for i in range(len(streams))]    # bit k = height 16 << k
+    for st, heights in zip(streams, masks):
+        _lib.check(Lb.nq_pf_pre_rows(x.data_ptr(), pts.data_ptr(), pes.data_ptr(), n, tb.data_ptr(), xg, xu, zg, E, H, I,
+                                     tiles.data_ptr(), cap, heights, C.c_void_p(st.cuda_stream)))
+    gemms(0, xg, xu, acc)
+    for st, heights in zip(streams, masks):
+        _lib.check(Lb.nq_pf_mid_rows(acc, pes.data_ptr(), n, tb.data_ptr(), h, zg, zd, E, H, I, tiles.data_ptr(), cap, heights,
+                                     C.c_void_p(st.cuda_stream)))
+    gemms(1, h, None, y)
     for st in side:
         done = torch.cuda.Event(); done.record(st); main.wait_event(done)
 
@@ -275,7 +290,7 @@ def prefill(s, x, sel, rw, out=None, R=None, G=None, table=None):
     grouped GEMMs at the level of its live table row, same math as the decode path (fp32 accumulation order differs).
     No host synchronisation (the reference's prefill reads the expert counts back; here the tile lists are built on the
     device by nq_pf_plan). Exports routing hits like the decode kernel. Calls on one device share the scratch of pf_scratch()
-    (as the reference's do, sm120/moe.py:262-274) and the side streams of _pf_gemms, so they must be ordered on one stream."""
+    (as the reference's do, sm120/moe.py:262-274) and the side streams of _pf_chains, so they must be ordered on one stream."""
     if s.G != 4:
         raise NotImplementedError("prefill decodes rings of G = 4 lanes only (as the reference's pf_decode)")
     assert x.dtype == torch.float16 and rw.dtype == torch.float16 and sel.dtype == torch.int64, (x.dtype, rw.dtype, sel.dtype)
@@ -311,12 +326,7 @@ def prefill(s, x, sel, rw, out=None, R=None, G=None, table=None):
         _lib.check(Lb.nq_pf_plan(cnt.data_ptr(), E, c, n, tiles.data_ptr(), cap, st))
         lists = [(16 << i, tiles[i], E if i < 4 else cap) for i in (4, 3, 2, 1, 0)]          # tallest first
         pts, pes = pt[c:d], pe[c:d]
-        _lib.check(Lb.nq_pf_pre(x.data_ptr(), pts.data_ptr(), pes.data_ptr(), n, tb.data_ptr(), S["xg"].data_ptr(),
-                                S["xu"].data_ptr(), S["zg"].data_ptr(), E, H, I, st))
-        _pf_gemms(Lb, tb, lists, variants, 0, S["xg"].data_ptr(), S["xu"].data_ptr(), S["acc"].data_ptr(), E, H, I)
-        _lib.check(Lb.nq_pf_mid(S["acc"].data_ptr(), pes.data_ptr(), n, tb.data_ptr(), S["h"].data_ptr(), S["zg"].data_ptr(),
-                                S["zd"].data_ptr(), E, H, I, st))
-        _pf_gemms(Lb, tb, lists, variants, 1, S["h"].data_ptr(), None, S["y"].data_ptr(), E, H, I)
+        _pf_chains(Lb, tb, lists, variants, S, x, pts, pes, n, tiles, cap, E, H, I)
         _lib.check(Lb.nq_pf_post(S["y"].data_ptr(), pos.data_ptr(), selc.data_ptr(), rwc.data_ptr(), T, k, c, n, tb.data_ptr(),
                                  out.data_ptr(), S["zd"].data_ptr(), E, H, I, st))
     return out
