@@ -154,12 +154,12 @@ extern "C" int nq_pf_pre(const void* x, const int32_t* pt, const int32_t* pe, in
 extern "C" int nq_pf_pre_rows(const void* x, const int32_t* pt, const int32_t* pe, int np, const int64_t* table, void* xg, void* xu,
                               float* zg, int E, int H, int I, const int32_t* tiles, int cap, int heights, void* stream)
 {
-    NQ_REQUIRE(np >= 0, "nq_pf_pre_rows: np=%d", np);
-    if (np == 0 || (heights & 31) == 0) return 0;
+    NQ_REQUIRE(np >= 0 && (heights & ~31) == 0, "nq_pf_pre_rows: np=%d, heights=0x%x (a mask of the five tile heights)", np, heights);
+    if (np == 0 || heights == 0) return 0;
     NQ_REQUIRE(x && pt && pe && table && xg && xu && tiles, "nq_pf_pre_rows: null pointer");
     NQ_REQUIRE(E >= 1 && shape_ok(H, I), "nq_pf_pre_rows: E=%d H=%d I=%d (H, I positive multiples of 128)", E, H, I);
     NQ_REQUIRE(aligned16(x) && aligned16(xg) && aligned16(xu) && aligned16(tiles), "nq_pf_pre_rows: x, xg, xu and tiles must be 16-byte aligned");
-    NQ_REQUIRE(cap >= E && (heights & ~31) == 0, "nq_pf_pre_rows: cap=%d below E=%d, or heights=0x%x outside the five tile heights", cap, E, heights);
+    NQ_REQUIRE(cap >= E, "nq_pf_pre_rows: cap=%d below E=%d", cap, E);
     return launch_pf_pre(x, pt, pe, np, table, xg, xu, zg, E, H, I, tiles, cap, heights, (hipStream_t)stream);
 }
 
@@ -191,12 +191,12 @@ extern "C" int nq_pf_mid(const float* acc_gu, const int32_t* pe, int np, const i
 extern "C" int nq_pf_mid_rows(const float* acc_gu, const int32_t* pe, int np, const int64_t* table, void* h, const float* zg, float* zd,
                               int E, int H, int I, const int32_t* tiles, int cap, int heights, void* stream)
 {
-    NQ_REQUIRE(np >= 0, "nq_pf_mid_rows: np=%d", np);
-    if (np == 0 || (heights & 31) == 0) return 0;
+    NQ_REQUIRE(np >= 0 && (heights & ~31) == 0, "nq_pf_mid_rows: np=%d, heights=0x%x (a mask of the five tile heights)", np, heights);
+    if (np == 0 || heights == 0) return 0;
     NQ_REQUIRE(acc_gu && pe && table && h && tiles, "nq_pf_mid_rows: null pointer");
     NQ_REQUIRE(E >= 1 && shape_ok(H, I), "nq_pf_mid_rows: E=%d H=%d I=%d (H, I positive multiples of 128)", E, H, I);
     NQ_REQUIRE(aligned16(acc_gu) && aligned16(h) && aligned16(tiles), "nq_pf_mid_rows: acc_gu, h and tiles must be 16-byte aligned");
-    NQ_REQUIRE(cap >= E && (heights & ~31) == 0, "nq_pf_mid_rows: cap=%d below E=%d, or heights=0x%x outside the five tile heights", cap, E, heights);
+    NQ_REQUIRE(cap >= E, "nq_pf_mid_rows: cap=%d below E=%d", cap, E);
     return launch_pf_mid(acc_gu, pe, np, table, h, zg, zd, E, H, I, tiles, cap, heights, (hipStream_t)stream);
 }
 

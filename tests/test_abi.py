@@ -107,6 +107,11 @@ def test_argument_checks_run_before_any_device_work():
     assert L.nq_pf_gemm(base, base, 1, 48, 0, base, base, base, 4, 256, 256, None) != 0 and "tile height" in err()
     assert L.nq_pf_gemm(base, base, 1, 16, 0, base + 8, base, base, 4, 256, 256, None) != 0 and "aligned" in err()
     assert L.nq_pf_pre(base + 2, base, base, 1, base, base, base, None, 4, 256, 256, None) != 0 and "aligned" in err()
+    assert L.nq_pf_pre_rows(base, base, base, 1, base, base, base, None, 4, 256, 256, base, 3, 1, None) != 0 and "cap" in err()
+    assert L.nq_pf_pre_rows(base, base, base, 1, base, base, base, None, 4, 256, 256, base, 4, 32, None) != 0 and "heights" in err()
+    assert L.nq_pf_pre_rows(base, base, base, 1, base, base, base, None, 4, 256, 256, base, 4, 0, None) == 0          # no height: nothing to do
+    assert L.nq_pf_mid_rows(base, base, 1, base, base, None, None, 4, 256, 256, None, 4, 1, None) != 0 and "null" in err()
+    assert L.nq_pf_mid_rows(base, base, 1, base, base, None, None, 4, 256, 256, base + 8, 4, 1, None) != 0 and "aligned" in err()
     assert L.nq_sal(base, 0, 64, base, 0, base, 0, 9, 64, 8, 16, 1.0, base, base, None) != 0 and "at most 8" in err()
     assert L.nq_dequant(base, 2, 0, 256, 256, base, None) != 0 and "proj" in err()
     assert L.nq_mailbox(None, base, base, base, None, 4, None) != 0 and "null" in err()

@@ -163,3 +163,58 @@ def test_prefill_on_a_side_stream_matches_the_default_stream():
     assert torch.equal(got, want) and torch.equal(got2, want * 2.0)
     for _ in range(3):                                              # back to back: the scratch is reused, nothing overtakes
         assert torch.equal(L.prefill(x, sel, rw), want)
+
+
+def test_row_restricted_pre_and_mid_cover_the_rows_of_their_heights_exactly():
+    """nq_pf_pre_rows / nq_pf_mid_rows over the five single-height masks write, together, bitwise what nq_pf_pre / nq_pf_mid
+    write, each launch only the rows of tiles of its height (everything else keeps the fill value), with the height of a row
+    taken from the host construction of the tile lists"""
+    from nestquant_amd import _lib
+    Lb = _lib.lib()
+    H, I, E = 256, 512, 12
+    ex = to_dev(experts_on_gpu(H, I, E, 900, rk=[(0, 3)] * E))
+    L = M.MoELayer(E, H, I, Bmax=8, topk=2)
+    for e in range(E):
+        L.set(e, ex[e], 4 if e % 3 else 2)
+    g = torch.Generator().manual_seed(77)
+    cnt = torch.tensor([0, 5, 16, 17, 40, 64, 100, 129, 256, 300, 513, 31])
+    pe = torch.repeat_interleave(torch.arange(E), cnt).int()
+    pe[3] = -1; pe[40] = E + 2                                   # rows of no valid expert: height 256 by convention
+    n = int(cnt.sum())
+    T = 50
+    pt = torch.randint(0, T, (n,), generator=g).int()
+    x = (torch.randn(T, H, generator=g) * 0.3).half().to(DEV)
+    acc = torch.randn(n, 2 * I, generator=g).to(DEV)
+    pe_d, pt_d = pe.to(DEV), pt.to(DEV)
+    cap = E + n // 256 + 1
+    tiles = torch.empty(5, cap, 4, dtype=torch.int32, device=DEV)
+    _lib.check(Lb.nq_pf_plan(cnt.int().to(DEV).data_ptr(), E, 0, n, tiles.data_ptr(), cap, None))
+    # height class of every row from the host lists
+    start = torch.cumsum(cnt, 0) - cnt
+    cls = torch.full((n,), 4)
+    for bm, t in M.pf_tiles([(e, int(start[e]), int(cnt[e])) for e in range(E) if cnt[e]]).items():
+        for e, r0, rows, _ in t.tolist():
+            cls[r0:r0 + rows] = bm.bit_length() - 5
+    cls[3] = cls[40] = 4
+    assert sorted(set(cls.tolist())) == [0, 1, 2, 3, 4]
+
+    def pre(rows_mask):
+        xg = torch.full((n, H), 7.0, dtype=torch.float16, device=DEV); xu = torch.full_like(xg, 7.0)
+        a = (x.data_ptr(), pt_d.data_ptr(), pe_d.data_ptr(), n, L.table.data_ptr(), xg.data_ptr(), xu.data_ptr(), None, E, H, I)
+        _lib.check(Lb.nq_pf_pre(*a, None) if rows_mask is None else Lb.nq_pf_pre_rows(*a, tiles.data_ptr(), cap, rows_mask, None))
+        return xg.cpu(), xu.cpu()
+
+    def mid(rows_mask):
+        h = torch.full((n, I), 7.0, dtype=torch.float16, device=DEV)
+        a = (acc.data_ptr(), pe_d.data_ptr(), n, L.table.data_ptr(), h.data_ptr(), None, None, E, H, I)
+        _lib.check(Lb.nq_pf_mid(*a, None) if rows_mask is None else Lb.nq_pf_mid_rows(*a, tiles.data_ptr(), cap, rows_mask, None))
+        return (h.cpu(),)
+
+    for fn in (pre, mid):
+        whole = fn(None)
+        for k in range(5):
+            part = fn(1 << k)
+            for w, q in zip(whole, part):
+                mine = cls == k
+                assert torch.equal(q[mine], w[mine]) and bool((q[~mine] == 7.0).all()), (fn.__name__, k)
+        assert all(torch.equal(a, b) for a, b in zip(fn(31), whole))
