@@ -344,3 +344,48 @@ def test_rings_of_two_lanes():
         L2.set(0, to_dev(experts_on_gpu(H, I, 1, 950, var_ids=(0,)))[0], 2)
     with pytest.raises(NotImplementedError):
         M.MoELayer(NE, H, I, G=1)
+
+
+@pytest.mark.parametrize("H,I,NE,topk,seed", [(128, 128, 3, 1, 1), (128, 384, 5, 3, 2), (384, 128, 4, 4, 3), (640, 896, 6, 5, 4),
+                                              (256, 1024, 9, 8, 5), (896, 512, 7, 2, 6), (1152, 640, 5, 6, 7)])
+def test_odd_shapes_decode_and_prefill_vs_full_oracle(H, I, NE, topk, seed):
+    """shapes whose chunk and strip counts are odd, prime or minimal (1 to 9 chunks, k-slices that do not divide evenly by the
+    default tilings' wishes), random codes, sign planes, nested and wide level 4, level 0 rows, every B from 1 to 8, repeated
+    and zero-weight picks; the 512-wide rotation where I allows it: decode path and prefill against the oracle's decode and
+    float64 layer"""
+    rng = random.Random(seed)
+    g = torch.Generator().manual_seed(100 + seed)
+    codes = list(range(10))
+    rk = [(rng.choice(codes), rng.choice(codes)) for _ in range(NE)]
+    nested = tuple(i for i in range(NE) if rng.random() < 0.3)
+    var_ids = tuple(i for i in range(NE) if i not in nested and rng.random() < 0.5)
+    ex = experts_on_gpu(H, I, NE, 7000 + 10 * seed, nested_ids=nested, rk=rk, var_ids=var_ids)
+    levels = [rng.choice((2, 4, 4, 3) if i in nested else (2, 4, 4, 0)) for i in range(NE)]
+    if all(lv == 0 for lv in levels):
+        levels[0] = 2
+    had = 512 if I % 512 == 0 and seed % 2 else 128
+    for e in ex:
+        e.had_dn = had
+    planes = [(oracle_plane(e.gu), oracle_plane(e.dn), e.nested) for e in ex]
+    signs = [e.signs.numpy() for e in ex]
+    to_dev(ex)
+    L = M.MoELayer(NE, H, I, Bmax=8, topk=topk)
+    for e in range(NE):
+        L.set(e, ex[e], levels[e])
+    for B in range(1, 9):
+        sel = torch.stack([torch.randint(0, NE, (topk,), generator=g) for _ in range(B)])       # repeats allowed
+        rw = torch.softmax(torch.randn(B, topk, generator=g), -1).half()
+        if B % 3 == 0:
+            rw[B - 1, topk - 1] = 0
+        x = (torch.randn(B, H, generator=g) * 0.05).half()
+        want = oracle_layer(planes, levels, signs, x, sel, rw, had_dn=had)
+        y = L(x.to(DEV), sel.to(DEV), rw.to(DEV)).cpu().numpy()
+        assert rel_err(y, want) < 5e-5 or np.abs(want).max() == 0, (B, rel_err(y, want))
+    T = 37 + 8 * seed
+    sel = torch.stack([torch.randperm(NE, generator=g)[:topk] if topk <= NE else torch.randint(0, NE, (topk,), generator=g) for _ in range(T)])
+    rw = torch.softmax(torch.randn(T, topk, generator=g), -1).half()
+    x = (torch.randn(T, H, generator=g) * 0.05).half()
+    want = oracle_layer(planes, levels, signs, x, sel, rw, had_dn=had)
+    for R in (None, 48):
+        y = L.prefill(x.to(DEV), sel.to(DEV), rw.to(DEV), R=R).cpu().numpy()
+        assert rel_err(y, want) < 5e-5, (R, rel_err(y, want))
