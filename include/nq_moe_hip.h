@@ -6,11 +6,11 @@
  * reference raises TORCH_CHECK -> RuntimeError at the same points, sm120/nqmoe.cu:871-878,887,897).
  *
  * Table row = int64[NQ_TBL_W] per expert (reference sm120/moe.py:216-229, sm120/nqmoe.cu:26-45):
- *   [0] level 0/2/3/4   [1..4] gate|up: base, residual plane, block words, flags(must be 0)   [5..8] down: same
+ *   [0] level 0/2/3/4   [1..4] gate|up: base, residual plane, block words, mask-mode flags (0 = none)   [5..8] down: same
  *   [9] fp16 sign/scale vector [H su_g | I sv_g | I sv_u | I su_d | H sv_o | H su_u]
  *   [10],[11] residual window code of gate|up, down (0..9 as the reference; 10 = nested K=1 plane P3; 11 = nested
  *   P3 || P4: uint2 sub-array of P3 followed by uint2 sub-array of P4)   [12],[13] sign-variant planes (0 = none)
- *   [14..17] low-rank plane (must be 0)   [18] in_had_down (must be 0 or 128)   [19] base codes (must be 0)
+ *   [14..17] low-rank plane: U/V buffers and ranks 0..4   [18] in_had_down 0 / 128 / 512   [19] base codes: 0 or 1 per projection
  */
 #ifndef NQ_MOE_HIP_H
 #define NQ_MOE_HIP_H
@@ -33,7 +33,7 @@ int nq_codes(uint32_t out[4]);
 
 /* Validate one table row held in HOST memory [host]: level, window codes, mask-mode flags (level 2, or level 4 with a wide
  * residual plane), low-rank plane (both buffers, ranks 0..4), in_had_down (0, 128, or 512 dividing I), and that the base
- * codes, which this library does not implement, are 0. Replaces the asserts of MoELayer.set (reference
+ * codes are 0 or 1 (the others are not implemented). Replaces the asserts of MoELayer.set (reference
  * sm120/moe.py:243-252); an unsupported field is an error, never silently ignored. */
 int nq_validate_row(const int64_t* row_host, int H, int I);
 
@@ -175,6 +175,70 @@ int nq_pf_plan(const int32_t* counts, int E, int row_lo, int nrows, int32_t* til
 
 /* hits[e] += counts[e] (hits may be host-mapped). Replaces pf_hits (reference sm120/nqmoe.cu:1241-1245,1288-1293). */
 int nq_pf_hits(const int32_t* counts, int32_t* hits, int E, void* stream);
+
+/* ---- Refinement-record upgrade engine (host threads + one side stream; replaces the class Engine of the reference's
+ * streaming/nqstream.cu:51-277 and its Python surface, :8-26). One engine per record file (one rank) and GPU. Unlike the
+ * entry points above, an engine owns memory for its lifetime: n_host pinned host entries of rec_bytes each (bounce
+ * buffers of the reads and a least-recently-used cache of records), pinned staging of rows and sequence numbers, an
+ * optional pinned RAM tier, one non-blocking stream of default priority, qd (+ qd_alt) reader threads and one director
+ * thread. It launches no kernel: its device work is hipMemcpyAsync host -> device. ---- */
+typedef struct NqStream NqStream;
+
+/* one finished op, as the tuples of the reference's Engine.poll() (streaming/nqstream.cu:110-113): hit = the record came
+ * from the host cache or the RAM tier; a failed read has t_read < 0 (the negated errno, or -1 for a short read) and
+ * t_e2e = -1 and has written neither row nor seq; a cancelled op has cancelled = 1 and both times = -1e9 */
+typedef struct NqStreamDone { int64_t tag; int32_t hit; int32_t cancelled; double t_read; double t_e2e; } NqStreamDone;
+
+/* counters of Engine.stats() (streaming/nqstream.cu:114-128); drive_direct = the file was opened with O_DIRECT (0 = the
+ * file system refused it and reads are buffered); failed = a HIP call of the engine failed (nq_last_error has its text) */
+typedef struct NqStreamStats
+{
+    int64_t upgrades, posts, host_hits, bytes_read, fault_injected, queued, reading, copying;
+    int64_t drives, n_host, drive_qd[2], drive_inflight[2], drive_reads[2], drive_bytes[2], drive_direct[2];
+    double drive_read_s[2];
+    int64_t tier_state, tier_recs, tier_hits, tier_bytes, cancelled, waiting, failed;
+    double now;
+} NqStreamStats;
+
+/* Open the record file `path` [host] (records of rec_bytes each, rec_bytes % 4096 == 0) for device `device`; alt_path
+ * (NULL or "" = none) is an identical copy on a second drive with its own queue depth qd_alt (0 = qd): each read goes to
+ * the drive with fewer reads in flight. n_host >= qd + qd_alt. The environment variables NQ_FAULT_READ_MS and
+ * NQ_FAULT_FAIL_PPM set the fault injection of nq_stream_set_fault at open. NULL on failure (nq_last_error).
+ * Reference: Engine(path, rec_bytes, n_host, qd, device, alt_path, qd_alt), streaming/nqstream.cu:72-93. */
+NqStream* nq_stream_open(const char* path, const char* alt_path, int64_t rec_bytes, int n_host, int qd, int qd_alt, int device);
+
+/* Queue an upgrade and return: record `rec` of the file -> device address slot (rec_bytes), then row_host [host]
+ * int64[NQ_TBL_W] -> stage_row (device), then seq -> seq_ptr (device int32), in this order on the engine's stream.
+ * Reference: Engine.upgrade, streaming/nqstream.cu:97-100. */
+int nq_stream_upgrade(NqStream* s, int64_t tag, int64_t rec, void* slot, void* stage_row, const int64_t* row_host, void* seq_ptr, int32_t seq);
+
+/* Queue a row-only op (a downgrade): row, then seq. Reference: Engine.post, streaming/nqstream.cu:101-104. */
+int nq_stream_post(NqStream* s, int64_t tag, void* stage_row, const int64_t* row_host, void* seq_ptr, int32_t seq);
+
+/* Best effort: an op that has started neither a read nor a device write is dropped and reported by nq_stream_poll as
+ * cancelled; one that has started completes normally. Reference: Engine.cancel, streaming/nqstream.cu:95,200-210. */
+int nq_stream_cancel(NqStream* s, int64_t tag);
+
+/* Move up to max finished ops into out [host]; returns their number. The device writes of a reported op are complete, so
+ * the next nq_mailbox may apply its row. Reference: Engine.poll, streaming/nqstream.cu:110-113. */
+int nq_stream_poll(NqStream* s, NqStreamDone* out, int max);
+
+/* Pinned RAM tier: read the n records recs [host] once, in the caller's thread, into one pinned buffer; an upgrade of
+ * one of them then skips the drive. Returns n, or -1. nq_stream_tier_drop releases the tier once no copy reads from it.
+ * Reference: Engine.tier_load / tier_drop, streaming/nqstream.cu:130-155,218-220. */
+int64_t nq_stream_tier_load(NqStream* s, const int64_t* recs, int64_t n);
+int nq_stream_tier_drop(NqStream* s);
+
+/* Fault injection for tests of the failure paths: read_ms = minimum spacing between the starts of drive reads (a slow
+ * drive), fail_ppm = share of completed reads reported as failed (a failing drive). Reference: the environment
+ * variables NQ_FAULT_READ_MS / NQ_FAULT_FAIL_PPM read by the constructor, streaming/nqstream.cu:68-70,92-93,264-269. */
+int nq_stream_set_fault(NqStream* s, double read_ms, int64_t fail_ppm);
+
+int nq_stream_stats(NqStream* s, NqStreamStats* out);
+
+/* Stop the threads, wait for the stream, free everything; ops not yet finished are dropped without a report.
+ * Reference: Engine.close, streaming/nqstream.cu:83-93. */
+void nq_stream_close(NqStream* s);
 
 #ifdef __cplusplus
 }

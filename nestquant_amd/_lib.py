@@ -44,6 +44,17 @@ SIGNATURES = {
     "nq_pf_post": (C.c_int, [_vp, _i32p, _i64p, _vp, _i, _i, _i, _i, _i64p, _vp, _vp, _i, _i, _i, _vp]),
     "nq_pf_plan": (C.c_int, [_i32p, _i, _i, _i, _i32p, _i, _vp]),
     "nq_pf_hits": (C.c_int, [_i32p, _i32p, _i, _vp]),
+    # record upgrade engine (host threads; structures mirrored in stream_engine.py)
+    "nq_stream_open": (C.c_void_p, [C.c_char_p, C.c_char_p, C.c_int64, _i, _i, _i, _i]),
+    "nq_stream_upgrade": (C.c_int, [_vp, C.c_int64, C.c_int64, _vp, _vp, C.POINTER(C.c_int64), _vp, C.c_int32]),
+    "nq_stream_post": (C.c_int, [_vp, C.c_int64, _vp, C.POINTER(C.c_int64), _vp, C.c_int32]),
+    "nq_stream_cancel": (C.c_int, [_vp, C.c_int64]),
+    "nq_stream_poll": (C.c_int, [_vp, _vp, _i]),
+    "nq_stream_tier_load": (C.c_int64, [_vp, C.POINTER(C.c_int64), C.c_int64]),
+    "nq_stream_tier_drop": (C.c_int, [_vp]),
+    "nq_stream_set_fault": (C.c_int, [_vp, C.c_double, C.c_int64]),
+    "nq_stream_stats": (C.c_int, [_vp, _vp]),
+    "nq_stream_close": (None, [_vp]),
 }
 
 

@@ -115,3 +115,19 @@ def test_argument_checks_run_before_any_device_work():
     assert L.nq_sal(base, 0, 64, base, 0, base, 0, 9, 64, 8, 16, 1.0, base, base, None) != 0 and "at most 8" in err()
     assert L.nq_dequant(base, 2, 0, 256, 256, base, None) != 0 and "proj" in err()
     assert L.nq_mailbox(None, base, base, base, None, 4, None) != 0 and "null" in err()
+
+
+def test_stream_engine_refuses_bad_arguments_before_touching_the_gpu(tmp_path):
+    """the checks of the reference's Engine constructor (streaming/nqstream.cu:76,77,81): record size a multiple of 4 KiB,
+    at least as many host entries as reads in flight, the record file must exist"""
+    from nestquant_amd.stream_engine import Engine
+    f = tmp_path / "r.bin"
+    f.write_bytes(b"\0" * 8192)
+    with pytest.raises(RuntimeError, match="4096"):
+        Engine(str(f), 4095, 8, 2, 0)
+    with pytest.raises(RuntimeError, match="n_host"):
+        Engine(str(f), 4096, 3, 4, 0)
+    with pytest.raises(RuntimeError, match="n_host"):
+        Engine(str(f), 4096, 4, 3, 0, alt_path=str(f), qd_alt=2)
+    with pytest.raises(RuntimeError, match="open .*missing.bin"):
+        Engine(str(tmp_path / "missing.bin"), 4096, 4, 2, 0)
