@@ -287,6 +287,68 @@ def churn_leg(L, MB, ex, levels, routes, xs, dev, steps=64, ops_per_step=8):
     return res
 
 
+def stream_leg(dev, nrec=48, nslot=32, nup=192, n_host=16, qd=8):
+    """The record upgrade engine at the full-shape record size (p4rec layout for H=6144, I=2048, residual K=2): `nup` upgrades
+    of records picked at random from a file of `nrec` records written here to the box's temporary directory (the engine drops a
+    record's cached pages after reading it, so repeated picks go back to the drive unless a host entry still holds them), then
+    the same from the pinned RAM tier (pure host -> device copies); rows and sequence numbers go to a scratch mailbox."""
+    import tempfile
+    from nestquant_amd import p4rec
+    from nestquant_amd.stream_engine import Engine
+    rb = p4rec.layout_of(p4rec.seg_bytes(6144, 2048))["rec_bytes"]
+    rng = np.random.default_rng(7)
+    slots = torch.empty(nslot, rb, dtype=torch.uint8, device=dev)
+    stage = torch.zeros(nslot, 20, dtype=torch.int64, device=dev)
+    seq = torch.zeros(nslot, dtype=torch.int32, device=dev)
+    row = torch.zeros(20, dtype=torch.int64)
+    with tempfile.TemporaryDirectory() as d:
+        path = os.path.join(d, "rank0.bin")
+        block = rng.integers(0, 256, rb, dtype=np.uint8)
+        with open(path, "wb") as f:
+            for r in range(nrec):
+                block[:8] = r
+                f.write(block.tobytes())
+        picks = [int(r) for r in rng.integers(0, nrec, nup)]
+
+        def run(eng):
+            t0 = time.perf_counter(); n = 0; lat = []
+            for i, r in enumerate(picks):
+                eng.upgrade(i, r, slots[i % nslot].data_ptr(), stage[i % nslot].data_ptr(), row, seq.data_ptr() + 4 * (i % nslot), i + 1)
+            while n < nup and time.perf_counter() - t0 < 60:
+                for tag, hit, trd, te2e in eng.poll():
+                    assert trd >= 0, f"read failed ({trd})"
+                    n += 1; lat.append(te2e)
+                time.sleep(2e-4)
+            dt = time.perf_counter() - t0
+            assert n == nup
+            torch.cuda.synchronize()
+            return dt, eng.stats()
+
+        eng = Engine(path, rb, n_host, qd, torch.cuda.current_device())
+        try:
+            dt_file, st = run(eng)
+            eng.upgrade(nup, 5, slots[0].data_ptr(), stage[0].data_ptr(), row, seq.data_ptr(), nup + 1)
+            while not eng.poll():
+                time.sleep(2e-4)
+            torch.cuda.synchronize()
+            block[:8] = 5
+            assert torch.equal(slots[0].cpu(), torch.from_numpy(block)), "slot bytes differ from the record"
+        finally:
+            eng.close()
+        eng = Engine(path, rb, n_host, qd, torch.cuda.current_device())
+        try:
+            t0 = time.perf_counter(); eng.tier_load(list(range(nrec))); dt_load = time.perf_counter() - t0
+            dt_tier, st_t = run(eng)
+            assert st_t["tier_hits"] == nup and st_t["bytes_read"] == 0
+        finally:
+            eng.close()
+    return dict(workload=f"{nup} upgrades of {rb} B records (H=6144, I=2048) from a {nrec}-record file in the temporary directory into {nslot} slots, "
+                         f"n_host {n_host}, qd {qd}; then from the pinned RAM tier",
+                rec_bytes=rb, file_GBps=round(nup * rb / dt_file / 1e9, 2), host_hit_share=round(st["host_hits"] / nup, 3),
+                o_direct=bool(st["drive_direct"][0]), read_ms_mean=round(st["drive_read_s"][0] / max(st["drive_reads"][0], 1) * 1e3, 3),
+                tier_GBps=round(nup * rb / dt_tier / 1e9, 2), tier_load_GBps=round(nrec * rb / dt_load / 1e9, 2))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -296,6 +358,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill (4096 tokens) leg")
     ap.add_argument("--no-churn", action="store_true", help="skip the plane-churn leg")
+    ap.add_argument("--no-stream", action="store_true", help="skip the record upgrade engine leg (file -> pinned -> slot)")
     ap.add_argument("--no-caller", action="store_true", help="skip the caller-dtype leg (bf16 / fp32 / int32 tensors)")
     ap.add_argument("--calib", action="store_true", help="also run one 256 MiB device copy (reads 256 MiB, writes 256 MiB): "
                     "the known-size kernel that scales rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
@@ -395,6 +458,7 @@ def main():
     prefill = None if a.no_prefill else prefill_leg(L, ex, dev)
     caller = None if a.no_caller else caller_leg(L, MB, routes, xs, dev)
     churn = None if a.no_churn else churn_leg(L, MB, ex, levels, routes[:16], xs, dev)
+    stream = None if a.no_stream else stream_leg(dev)
     print(json.dumps({
         "metric": "MoE layer us + HBM GB/s (decode bs1 top-8); prefill grouped-GEMM TFLOP/s",
         "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": W,
@@ -403,7 +467,7 @@ def main():
         "config": {"workload": f"decode MoE layer: E=256 top-8 B={B}, H=6144 I=2048, levels 2/3/4 = "
                                f"{lv_counts[2]}/{lv_counts[3]}/{lv_counts[4]} experts, seeded softmax routing avoiding the previous step",
                    "code_MB_per_step": round(nbytes / K / 1e6, 2), "hbm_frac_layer": round(gbs / HBM_PEAK_GBS, 4)},
-        "roofline": roofline, "cpu_baseline": cpu, "prefill": prefill, "caller_dtypes": caller, "churn": churn}))
+        "roofline": roofline, "cpu_baseline": cpu, "prefill": prefill, "caller_dtypes": caller, "churn": churn, "stream": stream}))
 
 
 if __name__ == "__main__":

@@ -379,6 +379,7 @@ struct Engine
             (e = hipHostMalloc((void**)&rows, (size_t)nring * ROW_W * 8, hipHostMallocPortable)) != hipSuccess ||
             (e = hipHostMalloc((void**)&seqs, (size_t)nring * 4, hipHostMallocPortable)) != hipSuccess)
             return nq::set_error("nq_stream_open: pinned memory (%zu bytes of entries): %s", (size_t)nh * rb, hipGetErrorString(e));
+        memset(host, 0, (size_t)nh * rb);                          // first touch of pinned pages is slow (2.7 GB/s against 23): pay it here
         for (int i = 0; i < nring; ++i) ring_free.push_back(i);
         ent_rec.assign(nh, -1); ent_users.assign(nh, 0); ent_stamp.assign(nh, 0);
         if (const char* v = getenv("NQ_FAULT_READ_MS")) fault_gap_us = (int64_t)(atof(v) * 1e3);
