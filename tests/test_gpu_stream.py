@@ -344,3 +344,62 @@ def test_executor_serves_a_layer_through_upgrades_and_downgrades(tmp_path):
         assert st["landed_cum"] == 3 and st["free_slots"] == 1 and st["ops_outstanding"] == 0 and st["op_p50_ms"] > 0
     finally:
         ex.close()
+
+
+def test_scheduler_executor_and_layer_in_one_serving_loop(tmp_path):
+    """the reference's serving step (sm120/serve/nq_vllm.py:546-574 with streaming/smoke_sched.py's loop): mailbox, layer
+    call with the hits export, counts -> Scheduler.step -> RankExecutor.apply, poll after the call. Routing favours two
+    experts at a time and then moves on; whenever nothing is in flight the table's levels are the scheduler's, and the layer
+    equals, bitwise, a layer set directly to those levels"""
+    from nestquant_amd.scheduler import Scheduler
+    root, out = str(tmp_path / "fit"), str(tmp_path / "out")
+    ids, L, rank, tp, topk, B = (0, 1, 3, 4, 6, 7), 5, 1, 4, 2, 1
+    man, parts = synth_layer(seed=17, H=256, res_K=2.25, experts=ids)
+    write_layer(root, L, man, parts, "safetensors")
+    repack.repack(root, out, tp=tp, layers=[L], dev=DEV, ne=8, log=lambda s: None)
+    RL = nqload.RankLayer(root, L, rank, tp, dev=DEV)
+    H, I = RL.H, RL.I
+    rf = RankFile(out, rank)
+    got, _, _ = resident.load(f"{out}/res/rank{rank}/L{L}.pt", DEV)
+    served, direct = M.MoELayer(8, H, I, Bmax=B, topk=topk), M.MoELayer(8, H, I, Bmax=B, topk=topk)
+    hits = torch.zeros(8, dtype=torch.int32).pin_memory()
+    served.hits_ptr = hits.data_ptr()
+    for E in ids:
+        served.set(E, got[E], 2)
+    mb = M.Mailbox(served)
+    ex = RankExecutor(rf, {L: (served, mb, {E: got[E] for E in ids})}, nslot=2, n_host=4, qd=2, device=0)
+    S = Scheduler([L], {L: []}, {L: []}, rf.rb, NE=8, n_float=2, half_life=16, refresh=4, cap_GBps=1e3, tok_per_s=1.0, slots=2)
+    g = torch.Generator().manual_seed(9)
+    x = (torch.randn(B, H, generator=g) * 0.5).half().to(DEV)
+    rw = torch.tensor([[0.625, 0.375]]).half().to(DEV)
+    seen_sets, checked = set(), 0
+    try:
+        for t in range(240):
+            pair = [(0, 1), (3, 4), (6, 7), (4, 0)][(t // 60) % 4]
+            sel = torch.tensor([pair], device=DEV)
+            mb.apply()
+            prev = hits.clone()
+            y = served(x, sel, rw).clone()
+            torch.cuda.synchronize()
+            ex.poll(S)
+            counts = (hits - prev).numpy().astype(np.float64)[None]
+            assert counts.sum() == topk and counts[0, list(pair)].tolist() == [1, 1]
+            if ex.quiet() and not ex.pend:
+                lv = S.level()[0]
+                assert [int(served.table[E, 0]) for E in ids] == [int(lv[E]) for E in ids]
+                assert sorted(E for (_, E) in ex.slot_of) == [E for E in ids if lv[E] == 4]
+                for E in ids:
+                    row = M.entry(RL.ex[E], int(lv[E]))
+                    row[9] = RL.ex[E].sc[int(lv[E])].data_ptr()
+                    direct.table[E].copy_(row.to(DEV))
+                want = direct(x, sel, rw).clone()
+                torch.cuda.synchronize()
+                assert torch.equal(y, want)
+                seen_sets.add(tuple(E for E in ids if lv[E] == 4)); checked += 1
+            ups, downs = S.step(counts, ntok=B)
+            ex.apply(ups, downs, S)
+            time.sleep(0.001)
+        assert checked >= 100 and {(0, 1), (3, 4), (6, 7), (0, 4)} <= seen_sets, (checked, seen_sets)
+        assert S.stats["ups"] >= 8 and S.stats["downs"] >= 6 and ex.n_failed == 0
+    finally:
+        ex.close()
