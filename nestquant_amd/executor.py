@@ -28,13 +28,17 @@ from .moe import entry, validate_row
 
 
 class RankExecutor:
-    def __init__(s, rf, layers, nslot, n_host=64, qd=8, device=None, wait_for_slot=True, shadow=False, alt_path=None, qd_alt=0, tier=None):
+    def __init__(s, rf, layers, nslot, n_host=64, qd=8, device=None, wait_for_slot=True, shadow=False, alt_path=None, qd_alt=0, tier=None,
+                 engine=None):
+        """engine: an object with the Engine interface to use instead of `rf.engine(...)` (tests of the bookkeeping pass a
+        host-only stand-in together with device="cpu"; serving code leaves it None)"""
         s.shadow, s.rf, s.lay, s.rb, s.layers = shadow, rf, rf.lay, rf.rb, layers
-        dev = torch.device("cuda", torch.cuda.current_device() if device is None else device)
+        dev = torch.device(device) if isinstance(device, (str, torch.device)) else \
+            torch.device("cuda", torch.cuda.current_device() if device is None else device)
         s.slots = torch.empty(nslot, s.rb, dtype=torch.uint8, device=dev)
         s.free = list(range(nslot))[::-1]
         s.slot_of = {}
-        s.eng = rf.engine(n_host, qd, dev.index, alt_path=alt_path or "", qd_alt=qd_alt)
+        s.eng = engine if engine is not None else rf.engine(n_host, qd, dev.index, alt_path=alt_path or "", qd_alt=qd_alt)
         s.tag, s.ops = 0, {}                                  # tag -> (L, E, level, seq)
         s.up_tag, s.wait_apply, s.pend = {}, {}, []           # wait_apply: device writes done, not yet applied by the mailbox
         s.n_cancel = s.n_landed = s.n_refused = s.n_failed = s.n_waited = 0
