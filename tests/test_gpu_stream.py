@@ -237,6 +237,27 @@ def test_two_drives_share_the_reads(tmp_path):
         Engine(path, RB, 16, 2, 0, alt_path=short)
 
 
+def test_close_with_ops_still_queued_returns_and_later_calls_raise(tmp_path):
+    path, data = record_file(tmp_path, 16)
+    b = Bench(16)
+    eng = Engine(path, RB, 4, 2, 0)
+    eng.set_fault(read_ms=200.0)                                      # at most two reads start before close()
+    for i in range(16):
+        b.upgrade(eng, i, i)
+    time.sleep(0.01)
+    t0 = time.time()
+    eng.close()
+    assert time.time() - t0 < 5.0
+    eng.close()                                                       # a second close is a no-op
+    torch.cuda.synchronize()
+    sq = b.seq.cpu()
+    landed = [i for i in range(16) if int(sq[i])]
+    assert len(landed) <= 2 and all(int(sq[i]) == i + 1 and torch.equal(b.slots[i].cpu(), data[i]) for i in landed)
+    for call in (eng.poll, eng.stats, lambda: eng.cancel(1), lambda: b.upgrade(eng, 0, 0)):
+        with pytest.raises(RuntimeError, match="closed"):
+            call()
+
+
 class Sched:
     """records the executor's callbacks"""
 
