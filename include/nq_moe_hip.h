@@ -31,6 +31,12 @@ const char* nq_last_error(void);
  * {gate|up, down}; replaces rk_codes() / bk_codes() (reference sm120/nqmoe.cu:938-940, sm120/moe.py:246-252). */
 int nq_codes(uint32_t out[4]);
 
+/* Occupancy of a decode kernel (mode 0 = gate|up, 1 = down; any_rows as NqMoeArgs.common_rows != 1) launched with sb
+ * wavefronts per workgroup and shm bytes of dynamic LDS: out[0] = resident workgroups per CU, out[1] = registers per lane,
+ * out[2] = spill bytes per lane. Replaces occ(mode, G, cpw, sb, shm) (reference sm120/nqmoe.cu:930-937, which packs the
+ * three figures into one integer; G and cpw select no separate kernel here). Needs a GPU. */
+int nq_occ(int mode, int any_rows, int sb, int shm, int out[3]);
+
 /* Validate one table row held in HOST memory [host]: level, window codes, mask-mode flags (level 2, or level 4 with a wide
  * residual plane), low-rank plane (both buffers, ranks 0..4), in_had_down (0, 128, or 512 dividing I), and that the base
  * codes are 0 or 1 (the others are not implemented). Replaces the asserts of MoELayer.set (reference

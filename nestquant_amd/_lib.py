@@ -30,6 +30,7 @@ SIGNATURES = {
     "nq_abi_version": (C.c_int, []),
     "nq_last_error": (C.c_char_p, []),
     "nq_codes": (C.c_int, [C.POINTER(C.c_uint32)]),
+    "nq_occ": (C.c_int, [_i, _i, _i, _i, C.POINTER(C.c_int)]),
     "nq_validate_row": (C.c_int, [C.POINTER(C.c_int64), _i, _i]),
     "nq_dequant": (C.c_int, [_i64p, _i, _i, _i, _i, _vp, _vp]),
     "nq_pf_decode": (C.c_int, [_i64p, _i32p, _i, _vp, _vp, _i, _i, _vp]),

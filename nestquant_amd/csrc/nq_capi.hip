@@ -29,6 +29,12 @@ extern "C" int nq_codes(uint32_t out[4])
     return 0;
 }
 
+extern "C" int nq_occ(int mode, int any_rows, int sb, int shm, int out[3])
+{
+    NQ_REQUIRE(out && (mode == 0 || mode == 1) && sb >= 1 && sb <= 16 && shm >= 0, "nq_occ: mode 0 / 1, 1..16 wavefronts per workgroup, an output array");
+    return query_occ(mode, any_rows, sb, shm, out);
+}
+
 extern "C" int nq_validate_row(const int64_t* r, int H, int I)
 {
     NQ_REQUIRE(r, "nq_validate_row: null row");

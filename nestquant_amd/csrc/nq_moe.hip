@@ -555,6 +555,22 @@ int launch_moe(const MoeArgs& a, const int* cfg_gu, const int* cfg_dn, int which
     return 0;
 }
 
+// resident workgroups per CU, registers and spill bytes of a decode kernel for a launch shape
+int query_occ(int mode, int any_rows, int sb, int shm, int* out)
+{
+    auto kern = mode == 0 ? (any_rows ? nq_gemv_k<0, true> : nq_gemv_k<0, false>) : (any_rows ? nq_gemv_k<1, true> : nq_gemv_k<1, false>);
+    hipError_t e;
+    if (shm > 48 * 1024 && (e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, shm)) != hipSuccess)
+        return set_error("nq_occ: LDS %d bytes: %s", shm, hipGetErrorString(e));
+    int nb = 0;
+    if ((e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, (const void*)kern, 64 * sb, (size_t)shm)) != hipSuccess)
+        return set_error("nq_occ: %s", hipGetErrorString(e));
+    hipFuncAttributes fa;
+    if ((e = hipFuncGetAttributes(&fa, (const void*)kern)) != hipSuccess) return set_error("nq_occ: %s", hipGetErrorString(e));
+    out[0] = nb; out[1] = fa.numRegs; out[2] = (int)fa.localSizeBytes;
+    return 0;
+}
+
 int launch_mailbox(int64_t* table, const int64_t* stage, const int32_t* seq, int32_t* applied, int32_t* applied_host, int E, hipStream_t st)
 {
     nq_mailbox_k<<<(E + 127) / 128, 128, 0, st>>>(table, stage, seq, applied, applied_host, E);

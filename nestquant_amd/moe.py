@@ -83,6 +83,14 @@ def rk_codes():
     return [int(out[0]), int(out[1])]
 
 
+def occ(mode, sb, shm, any_rows=False):
+    """(resident workgroups per CU, registers per lane, spill bytes per lane) of the decode kernel `mode` (0 gate|up, 1 down)
+    launched with sb wavefronts per workgroup and shm bytes of dynamic LDS; the reference's M.occ (sm120/nqmoe.cu:930-937)"""
+    out = (C.c_int * 3)()
+    _lib.check(_lib.lib().nq_occ(mode, int(any_rows), sb, shm, out))
+    return tuple(out)
+
+
 def bk_codes():
     out = (C.c_uint32 * 4)()
     _lib.check(_lib.lib().nq_codes(out))
