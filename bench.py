@@ -217,19 +217,28 @@ def caller_leg(L, MB, routes, xs, dev, reps=4):
             "results": "bitwise equal"}
 
 
-def churn_leg(L, MB, ex, levels, routes, xs, dev, steps=64, ops_per_step=8):
-    """config 5: B=1 layer steps with 8 promote/demote ops per step issued on a side stream (pinned host -> slot copies)"""
+def churn_leg(L, MB, ex, levels, routes, xs, dev, steps=64, ops_per_step=8, native=True):
+    """config 5: B=1 layer steps with 8 promote/demote ops per step issued on a side stream (pinned host -> slot copies);
+    native: the ops go through the upgrade engine's upload() (its own thread and stream), else through torch copies"""
     from nestquant_amd import churn as CH
     lv4 = [e for e in range(E) if levels[e] >= 3]
-    X = CH.ChurnExecutor(L, MB, {e: ex[e] for e in range(E)}, nslots=len(lv4) + 4 * ops_per_step)
+    X = CH.ChurnExecutor(L, MB, {e: ex[e] for e in range(E)}, nslots=len(lv4) + 4 * ops_per_step, native=native)
     saved = L.table.clone()
     for e in range(E):
         L.table[e].copy_(X.row(e, 2))
+
+    def settle():
+        for _ in range(4000):
+            MB.apply(); torch.cuda.synchronize()
+            X.poll()
+            if not X.pend:
+                return
+            time.sleep(5e-4)
+        raise RuntimeError("churn ops did not land")
+
     for e in lv4:                                                # bring the pool to the config-3 state (levels 3 become 4)
         X.promote(e, 4)
-    torch.cuda.synchronize()                                     # the side-stream copies and rows have landed
-    MB.apply(); torch.cuda.synchronize(); X.poll()
-    assert not X.pend
+    settle()
     X.bytes_copied = 0
     s = torch.cuda.Stream()
     graphs = []
@@ -265,25 +274,25 @@ def churn_leg(L, MB, ex, levels, routes, xs, dev, steps=64, ops_per_step=8):
             lat.append(e0.elapsed_time(e1) * 1e3)
             for e in X.poll():
                 lags.append(st - issued.pop(e, st))
+        if churn:
+            settle()                                             # the H2D rate is over issue -> last copy landed and applied
         wall = time.perf_counter() - t0
         return sorted(lat)[len(lat) // 2], lags, wall
 
     idle_us, _, _ = run(False)
     churn_us, lags, wall = run(True)
     torch.cuda.synchronize()
-    for _ in range(64):                                          # drain outstanding ops, then check the books
-        MB.apply(); torch.cuda.synchronize()
-        X.poll()
-        if not X.pend:
-            break
+    settle()                                                     # drain outstanding ops, then check the books
     X.check_invariants()
     res = dict(workload=f"plane churn: {steps} B=1 layer steps, {ops_per_step} promote(2->4)/demote(4->2) ops per step on a side "
                         f"stream, {X.lay.bytes} B per promotion from pinned host memory",
                step_us_idle=round(idle_us, 2), step_us_churn=round(churn_us, 2), ops=X.n_ops - len(lv4), refused=X.n_refused,
                h2d_GBps=round(X.bytes_copied / wall / 1e9, 2), h2d_MB=round(X.bytes_copied / 1e6, 1),
                lag_steps_median=(sorted(lags)[len(lags) // 2] if lags else None), lag_steps_max=(max(lags) if lags else None),
-               invariants="B,T,O,K hold after the run")
+               invariants="B,T,O,K hold after the run", issued_by="upgrade engine (upload)" if native else "torch copies")
+    X.close()
     L.table.copy_(saved)
+    MB.apply(); torch.cuda.synchronize()
     return res
 
 
@@ -457,7 +466,11 @@ def main():
     lv_counts = {lv: levels.count(lv) for lv in (2, 3, 4)}
     prefill = None if a.no_prefill else prefill_leg(L, ex, dev)
     caller = None if a.no_caller else caller_leg(L, MB, routes, xs, dev)
-    churn = None if a.no_churn else churn_leg(L, MB, ex, levels, routes[:16], xs, dev)
+    churn = None
+    if not a.no_churn:
+        churn = churn_leg(L, MB, ex, levels, routes[:16], xs, dev, native=True)
+        t = churn_leg(L, MB, ex, levels, routes[:16], xs, dev, native=False)
+        churn["torch_copies"] = {k: t[k] for k in ("step_us_churn", "ops", "refused", "h2d_GBps", "lag_steps_median", "lag_steps_max")}
     stream = None if a.no_stream else stream_leg(dev)
     print(json.dumps({
         "metric": "MoE layer us + HBM GB/s (decode bs1 top-8); prefill grouped-GEMM TFLOP/s",

@@ -204,6 +204,7 @@ typedef struct NqStreamStats
     double drive_read_s[2];
     int64_t tier_state, tier_recs, tier_hits, tier_bytes, cancelled, waiting, failed;
     double now;
+    int64_t uploads, upload_bytes;
 } NqStreamStats;
 
 /* Open the record file `path` [host] (records of rec_bytes each, rec_bytes % 4096 == 0) for device `device`; alt_path
@@ -220,6 +221,17 @@ int nq_stream_upgrade(NqStream* s, int64_t tag, int64_t rec, void* slot, void* s
 
 /* Queue a row-only op (a downgrade): row, then seq. Reference: Engine.post, streaming/nqstream.cu:101-104. */
 int nq_stream_post(NqStream* s, int64_t tag, void* stage_row, const int64_t* row_host, void* seq_ptr, int32_t seq);
+
+/* Queue an upload from the caller's pinned host memory and return: nspans (1..NQ_STREAM_MAX_SPANS) copies src_host[i] ->
+ * dst[i] (device) of nbytes[i], then the row, then seq, in this order on the engine's stream. The source must stay valid
+ * and unchanged until nq_stream_poll reports the op. This is the promotion of a resident-in-RAM expert (several spans: the
+ * planes a nested level adds); an engine opened with path NULL or "" serves only uploads and row-only ops and owns no
+ * host entries. The reference has no such call: its serving engine reads every record from the file or its RAM tier
+ * (streaming/nqstream.cu:183-191); its level-switch script copies from pinned tensors with torch
+ * (sm120/levelswitch_mbox.py:33-65), which this replaces. */
+#define NQ_STREAM_MAX_SPANS 8
+int nq_stream_upload(NqStream* s, int64_t tag, int nspans, const void* const* src_host, void* const* dst, const int64_t* nbytes,
+                     void* stage_row, const int64_t* row_host, void* seq_ptr, int32_t seq);
 
 /* Best effort: an op that has started neither a read nor a device write is dropped and reported by nq_stream_poll as
  * cancelled; one that has started completes normally. Reference: Engine.cancel, streaming/nqstream.cu:95,200-210. */

@@ -49,6 +49,8 @@ SIGNATURES = {
     "nq_stream_open": (C.c_void_p, [C.c_char_p, C.c_char_p, C.c_int64, _i, _i, _i, _i]),
     "nq_stream_upgrade": (C.c_int, [_vp, C.c_int64, C.c_int64, _vp, _vp, C.POINTER(C.c_int64), _vp, C.c_int32]),
     "nq_stream_post": (C.c_int, [_vp, C.c_int64, _vp, C.POINTER(C.c_int64), _vp, C.c_int32]),
+    "nq_stream_upload": (C.c_int, [_vp, C.c_int64, _i, C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.POINTER(C.c_int64), _vp,
+                                   C.POINTER(C.c_int64), _vp, C.c_int32]),
     "nq_stream_cancel": (C.c_int, [_vp, C.c_int64]),
     "nq_stream_poll": (C.c_int, [_vp, _vp, _i]),
     "nq_stream_tier_load": (C.c_int64, [_vp, C.POINTER(C.c_int64), C.c_int64]),

@@ -22,7 +22,7 @@ One outstanding op per expert; a slot is reused only after the level-2 row that 
 import torch
 
 from .format import CODE_L3, CODE_L4N
-from .moe import entry
+from .moe import entry, validate_row
 
 ALIGN = 256
 
@@ -75,9 +75,16 @@ class ChurnExecutor:
     layer / mailbox: nestquant_amd.moe.MoELayer / Mailbox; experts: {e: nested Expert whose base planes and sign vector
     are resident on the device}; nslots device slots are allocated here. Every expert starts at level 2."""
 
-    def __init__(s, layer, mailbox, experts, nslots, side_stream=None):
+    def __init__(s, layer, mailbox, experts, nslots, side_stream=None, native=False):
+        """native=True: copies, rows and sequence numbers are issued by the upgrade engine (stream_engine.Engine without a
+        record file: its own thread and side stream, `upload` from the pinned images) instead of torch copies on
+        `side_stream`; the books and the protocol are the same"""
         s.L, s.MB, s.ex = layer, mailbox, experts
         dev = layer.table.device
+        s.eng, s.tag, s.lat = None, 0, []
+        if native:
+            from .stream_engine import Engine
+            s.eng = Engine("", 0, 0, 8, dev.index if dev.index is not None else torch.cuda.current_device())
         s.lay = SlotLayout(layer.H, layer.I)
         s.slots = torch.zeros(nslots, s.lay.bytes, dtype=torch.uint8, device=dev)
         s.host = {e: s.lay.image(x) for e, x in experts.items()}
@@ -112,11 +119,15 @@ class ChurnExecutor:
             return False
         slot = s.slot_of[e] if cur >= 3 else s.free.pop()
         s.slot_of[e] = slot
-        with torch.cuda.stream(s.side):
-            for o, n in s.lay.spans(cur, level):
-                s.slots[slot, o:o + n].copy_(s.host[e][o:o + n], non_blocking=True)
-                s.bytes_copied += n
-        s.MB.post(e, s.row(e, level, slot), s.side)               # row, then seq, after the copies, same stream
+        spans = s.lay.spans(cur, level)
+        s.bytes_copied += sum(n for _, n in spans)
+        if s.eng is not None:
+            s._issue(e, s.row(e, level, slot), [(s.host[e].data_ptr() + o, s.slots[slot].data_ptr() + o, n) for o, n in spans])
+        else:
+            with torch.cuda.stream(s.side):
+                for o, n in spans:
+                    s.slots[slot, o:o + n].copy_(s.host[e][o:o + n], non_blocking=True)
+            s.MB.post(e, s.row(e, level, slot), s.side)           # row, then seq, after the copies, same stream
         s.pend[e] = (level, None)
         s.n_ops += 1
         return True
@@ -129,13 +140,37 @@ class ChurnExecutor:
             s.n_refused += 1
             return False
         slot = s.slot_of[e]
-        s.MB.post(e, s.row(e, level, slot if level == 3 else None), s.side)
+        row = s.row(e, level, slot if level == 3 else None)
+        if s.eng is not None:
+            s._issue(e, row, None)
+        else:
+            s.MB.post(e, row, s.side)
         s.pend[e] = (level, slot if level == 2 else None)
         s.n_ops += 1
         return True
 
+    def _issue(s, e, row, spans):
+        """one op through the engine: what Mailbox.post does on the host (row check, sequence number), then upload / post"""
+        assert s.MB.done(e), "one outstanding op per expert"
+        validate_row(row, s.L.H, s.L.I)
+        s.L.rare_rows |= bool(row[4] or row[8] or row[19])
+        s.MB.hseq[e] += 1
+        s.tag += 1
+        stage, seq = s.MB.stage.data_ptr() + s.MB.stage.stride(0) * 8 * e, s.MB.seq.data_ptr() + 4 * e
+        if spans:
+            s.eng.upload(s.tag, spans, stage, row, seq, s.MB.hseq[e])
+        else:
+            s.eng.post(s.tag, stage, row, seq, s.MB.hseq[e])
+
+    def close(s):
+        if s.eng is not None:
+            s.eng.close()
+            s.eng = None
+
     def poll(s):
         """after a layer call finished: ops the mailbox applied take effect on the host books; returns the experts landed"""
+        if s.eng is not None:
+            s.lat += [t for _, _, _, t in s.eng.poll()]
         landed = []
         for e in list(s.pend):
             if s.MB.done(e):

@@ -47,7 +47,9 @@ double now()
 struct Op
 {
     int64_t tag = 0, rec = -1;
-    bool read = false;                   // upgrade (record bytes + row + seq) or row-only op
+    bool read = false;                   // upgrade from the record file (record bytes + row + seq); otherwise row-only or upload
+    int nspans = 0;                      // upload: spans of the caller's pinned memory copied before the row (no file, no entry)
+    const void* sp_src[NQ_STREAM_MAX_SPANS]; void* sp_dst[NQ_STREAM_MAX_SPANS]; int64_t sp_n[NQ_STREAM_MAX_SPANS];
     void* slot = nullptr; void* stage = nullptr; void* seqp = nullptr;
     int32_t seq = 0;
     int64_t row[ROW_W];
@@ -101,7 +103,7 @@ struct Engine
     std::vector<Op*> copying;
     std::atomic<int> infl[2] = {{0}, {0}}, n_reading{0}, n_copying{0};   // written by the director, read by stats()
     // counters (under mu)
-    int64_t n_up = 0, n_post = 0, n_hit = 0, bytes = 0, n_cancel = 0, n_fault = 0, n_tier_hit = 0, tier_bytes = 0, n_wait = 0;
+    int64_t n_up = 0, n_post = 0, n_hit = 0, bytes = 0, n_cancel = 0, n_fault = 0, n_tier_hit = 0, tier_bytes = 0, n_wait = 0, n_upload = 0, upload_bytes = 0;
     int64_t d_reads[2] = {0, 0}, d_bytes[2] = {0, 0}; double d_rdt[2] = {0, 0};
     // fault injection (streaming/nqstream.cu:68-70): minimum spacing between drive reads; share of reads reported as failed
     std::atomic<int64_t> fault_gap_us{0}, fault_ppm{0};
@@ -174,6 +176,8 @@ struct Engine
         memcpy(r, o->row, sizeof o->row);
         seqs[o->ring] = o->seq;
         bool ok = true;
+        for (int i = 0; i < o->nspans && ok; ++i)
+            ok = hip_ok(hipMemcpyAsync(o->sp_dst[i], o->sp_src[i], (size_t)o->sp_n[i], hipMemcpyHostToDevice, st), "hipMemcpyAsync(span)");
         if (o->read)
         {
             const void* src = o->tier_src ? (const void*)o->tier_src : (const void*)(host + (size_t)o->entry * rb);
@@ -212,7 +216,11 @@ struct Engine
             if (!o->read)
             {
                 waiting.pop_front(); o->t_rd = o->t0;
-                { std::lock_guard<std::mutex> g(mu); n_post++; }
+                {
+                    std::lock_guard<std::mutex> g(mu);
+                    if (o->nspans) { n_upload++; for (int i = 0; i < o->nspans; ++i) upload_bytes += o->sp_n[i]; }
+                    else n_post++;
+                }
                 issue_copies(o);
                 continue;
             }
@@ -375,11 +383,11 @@ struct Engine
         if ((e = hipSetDevice(dev)) != hipSuccess) return nq::set_error("nq_stream_open: hipSetDevice(%d): %s", dev, hipGetErrorString(e));
         if ((e = hipStreamCreateWithFlags(&st, hipStreamNonBlocking)) != hipSuccess) return nq::set_error("nq_stream_open: stream: %s", hipGetErrorString(e));
         nring = (qd[0] + qd[1]) * 4;
-        if ((e = hipHostMalloc((void**)&host, (size_t)nh * rb, hipHostMallocPortable)) != hipSuccess ||
+        if ((nh && (e = hipHostMalloc((void**)&host, (size_t)nh * rb, hipHostMallocPortable)) != hipSuccess) ||
             (e = hipHostMalloc((void**)&rows, (size_t)nring * ROW_W * 8, hipHostMallocPortable)) != hipSuccess ||
             (e = hipHostMalloc((void**)&seqs, (size_t)nring * 4, hipHostMallocPortable)) != hipSuccess)
             return nq::set_error("nq_stream_open: pinned memory (%zu bytes of entries): %s", (size_t)nh * rb, hipGetErrorString(e));
-        memset(host, 0, (size_t)nh * rb);                          // first touch of pinned pages is slow (2.7 GB/s against 23): pay it here
+        if (nh) memset(host, 0, (size_t)nh * rb);                          // first touch of pinned pages is slow (2.7 GB/s against 23): pay it here
         for (int i = 0; i < nring; ++i) ring_free.push_back(i);
         ent_rec.assign(nh, -1); ent_users.assign(nh, 0); ent_stamp.assign(nh, 0);
         if (const char* v = getenv("NQ_FAULT_READ_MS")) fault_gap_us = (int64_t)(atof(v) * 1e3);
@@ -437,7 +445,17 @@ NqStream* nq_stream_open(const char* path, const char* alt_path, int64_t rec_byt
 {
     const bool two = alt_path && alt_path[0];
     const int q1 = two ? (qd_alt > 0 ? qd_alt : qd) : 0;
-    if (!path || rec_bytes <= 0 || rec_bytes % 4096 != 0 || qd < 1 || n_host < qd + q1)
+    const bool no_file = !path || !path[0];                      // uploads and row-only ops only: no drive, no host entries
+    if (no_file)
+    {
+        if (two) { nq::set_error("nq_stream_open: alt_path without path"); return nullptr; }
+        NqStream* s = new NqStream;
+        Engine& e = s->e;
+        e.dev = device; e.nh = 0; e.rb = 0; e.nd = 0; e.qd[0] = qd > 0 ? qd : 8; e.qd[1] = 0;
+        if (e.start()) { delete s; return nullptr; }
+        return s;
+    }
+    if (rec_bytes <= 0 || rec_bytes % 4096 != 0 || qd < 1 || n_host < qd + q1)
     {
         nq::set_error("nq_stream_open: need rec_bytes %% 4096 == 0 and n_host >= qd (+ qd_alt) >= 1 (rec_bytes %lld, n_host %d, qd %d, qd_alt %d)",
                       (long long)rec_bytes, n_host, qd, q1);
@@ -453,6 +471,7 @@ NqStream* nq_stream_open(const char* path, const char* alt_path, int64_t rec_byt
 int nq_stream_upgrade(NqStream* s, int64_t tag, int64_t rec, void* slot, void* stage_row, const int64_t* row_host, void* seq_ptr, int32_t seq)
 {
     NQ_REQUIRE(s && !s->e.closed, "nq_stream_upgrade: engine is closed");
+    NQ_REQUIRE(s->e.nd > 0, "nq_stream_upgrade: this engine was opened without a record file");
     NQ_REQUIRE(rec >= 0 && slot && stage_row && row_host && seq_ptr, "nq_stream_upgrade: null pointer or negative record index");
     Op* o = new Op; o->tag = tag; o->rec = rec; o->read = true; o->slot = slot; o->stage = stage_row; o->seqp = seq_ptr; o->seq = seq;
     return s->e.enqueue(o, row_host);
@@ -463,6 +482,21 @@ int nq_stream_post(NqStream* s, int64_t tag, void* stage_row, const int64_t* row
     NQ_REQUIRE(s && !s->e.closed, "nq_stream_post: engine is closed");
     NQ_REQUIRE(stage_row && row_host && seq_ptr, "nq_stream_post: null pointer");
     Op* o = new Op; o->tag = tag; o->stage = stage_row; o->seqp = seq_ptr; o->seq = seq;
+    return s->e.enqueue(o, row_host);
+}
+
+int nq_stream_upload(NqStream* s, int64_t tag, int nspans, const void* const* src_host, void* const* dst, const int64_t* nbytes,
+                     void* stage_row, const int64_t* row_host, void* seq_ptr, int32_t seq)
+{
+    NQ_REQUIRE(s && !s->e.closed, "nq_stream_upload: engine is closed");
+    NQ_REQUIRE(nspans >= 1 && nspans <= NQ_STREAM_MAX_SPANS && src_host && dst && nbytes, "nq_stream_upload: 1..%d spans", NQ_STREAM_MAX_SPANS);
+    NQ_REQUIRE(stage_row && row_host && seq_ptr, "nq_stream_upload: null pointer");
+    Op* o = new Op; o->tag = tag; o->stage = stage_row; o->seqp = seq_ptr; o->seq = seq; o->nspans = nspans;
+    for (int i = 0; i < nspans; ++i)
+    {
+        if (!src_host[i] || !dst[i] || nbytes[i] <= 0) { delete o; return nq::set_error("nq_stream_upload: span %d is empty or null", i); }
+        o->sp_src[i] = src_host[i]; o->sp_dst[i] = dst[i]; o->sp_n[i] = nbytes[i];
+    }
     return s->e.enqueue(o, row_host);
 }
 
@@ -552,6 +586,7 @@ int nq_stream_stats(NqStream* s, NqStreamStats* out)
     }
     out->tier_state = e.tier_state.load(); out->tier_recs = (int64_t)e.tier_n; out->tier_hits = e.n_tier_hit;
     out->tier_bytes = e.tier_bytes; out->cancelled = e.n_cancel; out->waiting = e.n_wait; out->now = now();
+    out->uploads = e.n_upload; out->upload_bytes = e.upload_bytes;
     out->failed = e.fail.empty() ? 0 : 1;
     if (!e.fail.empty()) nq::set_error("nq_stream: %s", e.fail.c_str());
     return 0;

@@ -11,6 +11,7 @@ there is no Python fallback.
     e.poll() -> [(tag, hit, t_read_s, t_e2e_s)]     ops whose device writes are complete
     e.cancel(tag) / e.tier_load(recs) / e.tier_drop() / e.stats() / e.close()
     e.set_fault(read_ms, fail_ppm)                  # what the reference reads from NQ_FAULT_READ_MS / NQ_FAULT_FAIL_PPM
+    e.upload(tag, [(host_ptr, dev_ptr, bytes)], stage_ptr, row, seq_ptr, seq)     # from the caller's pinned memory (no file)
 """
 import ctypes as C
 import json
@@ -33,7 +34,7 @@ class NqStreamStats(C.Structure):
                 + [(k, C.c_int64 * 2) for k in ("drive_qd", "drive_inflight", "drive_reads", "drive_bytes", "drive_direct")]
                 + [("drive_read_s", C.c_double * 2)]
                 + [(k, C.c_int64) for k in ("tier_state", "tier_recs", "tier_hits", "tier_bytes", "cancelled", "waiting", "failed")]
-                + [("now", C.c_double)])
+                + [("now", C.c_double), ("uploads", C.c_int64), ("upload_bytes", C.c_int64)])
 
 
 _POLL_MAX = 256
@@ -54,8 +55,9 @@ def _row_array(row):
 
 class Engine:
     def __init__(s, path, rec_bytes, n_host, qd, device, alt_path="", qd_alt=0):
+        """path "" (or None): an engine without a record file, for upload() and post() only"""
         s.M = _lib.lib()
-        s.h = s.M.nq_stream_open(str(path).encode(), (alt_path or "").encode(), int(rec_bytes), int(n_host), int(qd), int(qd_alt), int(device))
+        s.h = s.M.nq_stream_open(str(path or "").encode(), (alt_path or "").encode(), int(rec_bytes), int(n_host), int(qd), int(qd_alt), int(device))
         if not s.h:
             raise RuntimeError(s.M.nq_last_error().decode())
         s._buf = (NqStreamDone * _POLL_MAX)()
@@ -70,6 +72,15 @@ class Engine:
 
     def post(s, tag, stage, row, seqp, seq):
         _lib.check(s.M.nq_stream_post(s._handle(), int(tag), int(stage), _row_array(row), int(seqp), int(seq)))
+
+    def upload(s, tag, spans, stage, row, seqp, seq):
+        """spans: [(pinned host address, device address, bytes)], copied in order before the row and seq; the host memory
+        must stay valid until poll() reports the tag"""
+        n = len(spans)
+        src = (C.c_void_p * n)(*[int(a) for a, _, _ in spans])
+        dst = (C.c_void_p * n)(*[int(b) for _, b, _ in spans])
+        nb = (C.c_int64 * n)(*[int(c) for _, _, c in spans])
+        _lib.check(s.M.nq_stream_upload(s._handle(), int(tag), n, src, dst, nb, int(stage), _row_array(row), int(seqp), int(seq)))
 
     def cancel(s, tag):
         _lib.check(s.M.nq_stream_cancel(s._handle(), int(tag)))
@@ -102,7 +113,8 @@ class Engine:
             raise RuntimeError(s.M.nq_last_error().decode())
         nd = st.drives
         d = {k: getattr(st, k) for k in ("upgrades", "posts", "host_hits", "bytes_read", "fault_injected", "queued", "reading", "copying",
-                                         "drives", "n_host", "tier_state", "tier_recs", "tier_hits", "tier_bytes", "cancelled", "waiting", "now")}
+                                         "drives", "n_host", "tier_state", "tier_recs", "tier_hits", "tier_bytes", "cancelled", "waiting", "now",
+                                         "uploads", "upload_bytes")}
         for k in ("drive_qd", "drive_inflight", "drive_reads", "drive_bytes", "drive_read_s", "drive_direct"):
             d[k] = list(getattr(st, k))[:nd]
         return d

@@ -25,7 +25,8 @@ def test_slot_layout_and_rows():
     assert lay.spans(2, 4) == [(0, lay.bytes)] and lay.bytes >= 2 * (4718592 + 73728)
 
 
-def test_churn_racing_graph_replays():
+@pytest.mark.parametrize("native", [False, True], ids=["torch_copies", "engine_uploads"])
+def test_churn_racing_graph_replays(native):
     H, I, NE, NSLOT, B, K = 512, 256, 8, 3, 4, 4
     ex = {e: F.Expert(H, I, seed=70 + e, dev="cpu", nested=True, var=(e == 2)) for e in range(NE)}
     planes = {e: (oracle_plane(x.gu), oracle_plane(x.dn)) for e, x in ex.items()}
@@ -35,7 +36,7 @@ def test_churn_racing_graph_replays():
         x.gu.slot = x.gu.nested_plane(); x.dn.slot = x.dn.nested_plane()
     L = M.MoELayer(NE, H, I, Bmax=B, topk=K)
     MB = M.Mailbox(L)
-    X = CH.ChurnExecutor(L, MB, ex, NSLOT)
+    X = CH.ChurnExecutor(L, MB, ex, NSLOT, native=native)
     for e in range(NE):
         L.table[e].copy_(X.row(e, 2))
     g = torch.Generator().manual_seed(0)
@@ -92,6 +93,8 @@ def test_churn_racing_graph_replays():
         for sl in set(X.free) - free_before:                     # released slots are scribbled at once: stale use would show
             with torch.cuda.stream(X.side):
                 X.slots[sl].copy_(junk, non_blocking=True)
+            if native:
+                X.side.synchronize()                             # the engine's uploads run on its own stream, not X.side
         err = rel_err(out, ref(X.level))
         worst = max(worst, err)
         assert err < 5e-5, (st, err, X.level)
@@ -102,7 +105,12 @@ def test_churn_racing_graph_replays():
             X.check_invariants()
     torch.cuda.synchronize()
     X.check_invariants()
-    assert nops > 30 and changed > 10 and X.bytes_copied > 0
+    # the engine's ops land a thread hop later than copies issued from this thread, so fewer experts are idle when picked
+    assert nops > (20 if native else 30) and changed > (5 if native else 10) and X.bytes_copied > 0
+    if native:
+        st_ = X.eng.stats()
+        assert st_["upload_bytes"] == X.bytes_copied and st_["uploads"] + st_["posts"] == nops and len(X.lat) == nops
+    X.close()
     print(f"ops {nops}, refused {X.n_refused}, state changes seen {changed}, worst rel err {worst:.2e}")
 
 
