@@ -258,6 +258,36 @@ def test_close_with_ops_still_queued_returns_and_later_calls_raise(tmp_path):
             call()
 
 
+def test_uploads_from_pinned_memory_on_an_engine_without_a_file():
+    src = torch.randint(0, 256, (3, RB), dtype=torch.uint8).pin_memory()
+    b = Bench(2)
+    eng = Engine("", 0, 0, 4, 0)
+    try:
+        row = torch.full((20,), 7, dtype=torch.int64)
+        # three spans into one slot, out of order and of different sizes, then row and seq
+        spans = [(src[0].data_ptr(), b.slots[0].data_ptr() + 4096, 8192), (src[1].data_ptr() + 512, b.slots[0].data_ptr(), 4096),
+                 (src[2].data_ptr(), b.slots[0].data_ptr() + 32768, RB - 32768)]
+        eng.upload(1, spans, b.stage[0].data_ptr(), row, b.seq.data_ptr(), 5)
+        eng.post(2, b.stage[1].data_ptr(), row * 2, b.seq.data_ptr() + 4, 9)
+        done = drain(eng, 2)
+        assert not done[1][0] and done[1][1] == 0.0 and done[1][2] >= 0
+        torch.cuda.synchronize()
+        got = b.slots[0].cpu()
+        assert torch.equal(got[4096:12288], src[0][:8192]) and torch.equal(got[:4096], src[1][512:4608])
+        assert torch.equal(got[32768:], src[2][:RB - 32768]) and not got[12288:32768].any()
+        assert b.seq.tolist() == [5, 9] and b.stage[0].tolist() == [7] * 20 and b.stage[1].tolist() == [14] * 20
+        st = eng.stats()
+        assert (st["uploads"], st["upload_bytes"], st["posts"], st["upgrades"], st["drives"]) == (1, 8192 + 4096 + RB - 32768, 1, 0, 0)
+        with pytest.raises(RuntimeError, match="without a record file"):
+            b.upgrade(eng, 0, 0)
+        with pytest.raises(RuntimeError, match="spans"):
+            eng.upload(3, [(src.data_ptr(), b.slots[0].data_ptr(), 16)] * 9, b.stage[0].data_ptr(), row, b.seq.data_ptr(), 6)
+        with pytest.raises(RuntimeError, match="span 0"):
+            eng.upload(3, [(src.data_ptr(), b.slots[0].data_ptr(), 0)], b.stage[0].data_ptr(), row, b.seq.data_ptr(), 6)
+    finally:
+        eng.close()
+
+
 class Sched:
     """records the executor's callbacks"""
 
