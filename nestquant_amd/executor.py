@@ -192,6 +192,46 @@ class RankExecutor:
                        cp_p50_ms=float(np.percentile(a[:, 1], 50)), cp_p99_ms=float(np.percentile(a[:, 1], 99)))
         return out
 
+    def check_invariants(s, sched=None, max_bytes=None):
+        """Slot-integrity probe after the reference's sm120/serve/nq_slotcheck.py:11-21; synchronises the device and
+        reads records from the rank's file. Keys (L, E) in transit (an op in flight or a row not yet applied) are skipped.
+          B  slot bytes == the expert's record in the file          T  table row == the level-4 row built for the slot
+          O  a level-4 row points into the pool at the slot its key owns (level-2 rows equal the level-2 row)
+          K  slot_of injective, no owned slot in the free list, the free list without duplicates
+          S  (with sched) scheduler state UP <=> key resident and not in transit
+        max_bytes: compare at most this many leading bytes of each record (None = all). Raises AssertionError."""
+        torch.cuda.synchronize(s.slots.device)
+        transit = {(o[0], o[1]) for o in s.ops.values()} | set(s.wait_apply) | set(s.pend)
+        owned = list(s.slot_of.values())
+        assert len(set(owned)) == len(owned), "K: two keys own one slot"
+        assert not set(owned) & set(s.free), "K: an owned slot is in the free list"
+        assert len(set(s.free)) == len(s.free), "K: a slot is twice in the free list"
+        lo, hi = s.slot0, s.slot0 + s.nslot * s.rb
+        n = s.rb if max_bytes is None else min(s.rb, max_bytes)
+        with open(s.rf.path, "rb") as f:
+            for L, (M, _, exs) in s.layers.items():
+                table = M.table.cpu().numpy()
+                for E in exs:
+                    k = (L, E)
+                    if k in transit:
+                        continue
+                    r2, z, m = s.rc[k]
+                    sl = s.slot_of.get(k)
+                    if sl is None or s.shadow:
+                        assert (table[E] == r2).all(), f"T: row of {k} is not its level-2 row"
+                    else:
+                        assert (table[E] == z + m * s.addr(sl)).all(), f"T: row of {k} is not the level-4 row of slot {sl}"
+                        for w in np.nonzero(m)[0]:
+                            a = int(table[E][w])
+                            assert lo <= a < hi and (a - lo) // s.rb == sl, f"O: word {w} of the row of {k} leaves slot {sl}"
+                    if sl is not None:
+                        f.seek(s.rf.rec(L, E) * s.rb)
+                        rec = np.frombuffer(f.read(n), np.uint8)
+                        assert (s.slots[sl, :n].cpu().numpy() == rec).all(), f"B: slot {sl} differs from the record of {k}"
+                    if sched is not None:
+                        up = int(sched.state[sched.li[L], E]) == 2
+                        assert up == (sl is not None), f"S: scheduler state of {k} is {int(sched.state[sched.li[L], E])}, slot {sl}"
+
     def busy(s):
         return bool(s.ops or s.wait_apply or s.pend)
 

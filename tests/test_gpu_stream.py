@@ -362,6 +362,7 @@ def test_executor_serves_a_layer_through_upgrades_and_downgrades(tmp_path):
         torch.cuda.synchronize()
         assert [int(served.table[E, 0]) for E in ids] == [levels[E] for E in ids]
         assert torch.isfinite(want).all() and torch.equal(y, want)
+        ex.check_invariants()
 
     try:
         check()
@@ -391,6 +392,18 @@ def test_executor_serves_a_layer_through_upgrades_and_downgrades(tmp_path):
         assert len(ex.free) == 1 and ex.n_failed == 1 and (L, 3) not in ex.slot_of
         ex.eng.set_fault()
         check()
+        # the probe has teeth: a flipped slot byte and a foreign table row are both found
+        sl6 = ex.slot_of[L, 6]
+        ex.slots[sl6, 100] ^= 1
+        with pytest.raises(AssertionError, match="B: slot"):
+            ex.check_invariants()
+        ex.slots[sl6, 100] ^= 1
+        keep = served.table[6].clone()
+        served.table[6, 2] += ex.rb
+        with pytest.raises(AssertionError, match="T: row"):
+            ex.check_invariants()
+        served.table[6].copy_(keep)
+        ex.check_invariants()
         st = ex.io_stats()
         assert st["landed_cum"] == 3 and st["free_slots"] == 1 and st["ops_outstanding"] == 0 and st["op_p50_ms"] > 0
     finally:
@@ -447,6 +460,8 @@ def test_scheduler_executor_and_layer_in_one_serving_loop(tmp_path):
                 torch.cuda.synchronize()
                 assert torch.equal(y, want)
                 seen_sets.add(tuple(E for E in ids if lv[E] == 4)); checked += 1
+                if checked % 16 == 0:
+                    ex.check_invariants(S)
             ups, downs = S.step(counts, ntok=B)
             ex.apply(ups, downs, S)
             time.sleep(0.001)
