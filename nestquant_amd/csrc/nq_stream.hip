@@ -55,7 +55,7 @@ struct Op
     int64_t row[ROW_W];
     double t0 = 0, t_rd = 0, t_sub = 0;
     int entry = -1, ring = -1, drive = -1;
-    bool hit = false;
+    bool hit = false, copy_failed = false;   // copy_failed: a HIP call of this op's copies failed (seq was not written)
     const uint8_t* tier_src = nullptr;
     int64_t got = 0;                     // bytes the read returned, or -errno
     hipEvent_t ev = nullptr;
@@ -185,6 +185,7 @@ struct Engine
         }
         ok = ok && hip_ok(hipMemcpyAsync(o->stage, r, ROW_W * 8, hipMemcpyHostToDevice, st), "hipMemcpyAsync(row)");
         ok = ok && hip_ok(hipMemcpyAsync(o->seqp, seqs + o->ring, 4, hipMemcpyHostToDevice, st), "hipMemcpyAsync(seq)");
+        o->copy_failed = !ok;                                    // the chain stops at the first failure, so seq is never written after one
         o->ev = get_event();
         if (o->ev) hip_ok(hipEventRecord(o->ev, st), "hipEventRecord");
         copying.push_back(o); n_copying++;
@@ -199,7 +200,8 @@ struct Engine
             ring_free.push_back(o->ring);
             if (o->tier_src) tier_users--;
             else if (o->read) ent_users[o->entry]--;
-            report(o->tag, o->hit, o->t_rd - o->t0, now() - o->t0);
+            if (o->copy_failed) report(o->tag, false, -(double)EIO, -1.0);   // as a failed read: the row was never committed
+            else report(o->tag, o->hit, o->t_rd - o->t0, now() - o->t0);
             delete o;
             copying[i] = copying.back(); copying.pop_back(); n_copying--;
         }
