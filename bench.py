@@ -296,6 +296,54 @@ def churn_leg(L, MB, ex, levels, routes, xs, dev, steps=64, ops_per_step=8, nati
     return res
 
 
+def config2_leg(L, ex, levels, dev, R=64, reps=4):
+    """config 2: one expert's fused gate|up projection (6144 -> 2 x 2048, decode + GEMV without the layer around it) at each
+    level for 1 / 4 / 8 tokens: a graph of R launches over R different experts (cold weights), event-timed; GB/s of the code
+    bytes the launch reads at that level"""
+    saved = L.table.clone()
+    g = torch.Generator().manual_seed(2)
+    s = torch.cuda.Stream()
+    picks = [(37 * i) % E for i in range(R)]
+    out = {}
+    for lv in (2, 3, 4):
+        for e in picks:
+            L.set(e, ex[e], lv)
+        nbytes = sum(code_bytes(ex, [lv] * E, [e], which="gu") for e in picks) / R
+        for B in (1, 4, 8):
+            if B > L.out.shape[0]:
+                continue
+            x = (torch.randn(B, H, generator=g) * 0.05).half().to(dev)
+            rw = torch.ones(B, 1, dtype=torch.float16, device=dev)
+            sels = [torch.full((B, 1), e, dtype=torch.int64, device=dev) for e in picks]
+            best = None
+            for nst in (12, 6, 3, 2):                            # k-slice in chunks: a lone expert fills the GPU only when cut finer
+                cfg = [1, L.cfg_gu[1], nst]
+                with torch.cuda.stream(s):
+                    for q in sels:
+                        L(x, q, rw, which=1, cfg_gu=cfg)
+                torch.cuda.synchronize()
+                gr = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(gr, stream=s):
+                    for q in sels:
+                        L(x, q, rw, which=1, cfg_gu=cfg)
+                with torch.cuda.stream(s):
+                    gr.replay()
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record(s)
+                    for _ in range(reps):
+                        gr.replay()
+                    e1.record(s)
+                torch.cuda.synchronize()
+                us = e0.elapsed_time(e1) * 1e3 / (reps * R)
+                if best is None or us < best[0]:
+                    best = (us, nst)
+            out[f"L{lv}_B{B}"] = dict(us=round(best[0], 2), GBps=round(nbytes / best[0] / 1e3, 1), k_slice_chunks=best[1])
+    L.table.copy_(saved)
+    out["workload"] = ("one expert's gate|up projection per launch (N=4096, K=6144), 64 experts in turn, best k-slice of 12 / 6 / 3 / 2 chunks; "
+                       "code bytes per launch: " + ", ".join(f"L{lv} {int(sum(code_bytes(ex, [lv] * E, [e], which='gu') for e in picks) / R)}" for lv in (2, 3, 4)))
+    return out
+
+
 def stream_leg(dev, nrec=48, nslot=32, nup=192, n_host=16, qd=8):
     """The record upgrade engine at the full-shape record size (p4rec layout for H=6144, I=2048, residual K=2): `nup` upgrades
     of records picked at random from a file of `nrec` records written here to the box's temporary directory (the engine drops a
@@ -367,6 +415,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill (4096 tokens) leg")
     ap.add_argument("--no-churn", action="store_true", help="skip the plane-churn leg")
+    ap.add_argument("--no-config2", action="store_true", help="skip the single-projection leg (per-level GB/s at 1 / 4 / 8 tokens)")
     ap.add_argument("--no-stream", action="store_true", help="skip the record upgrade engine leg (file -> pinned -> slot)")
     ap.add_argument("--no-caller", action="store_true", help="skip the caller-dtype leg (bf16 / fp32 / int32 tensors)")
     ap.add_argument("--calib", action="store_true", help="also run one 256 MiB device copy (reads 256 MiB, writes 256 MiB): "
@@ -383,7 +432,7 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    L, MB, ex, levels = build_layer(dev, Bmax=max(4, B))
+    L, MB, ex, levels = build_layer(dev, Bmax=max(8, B))
     R = 64
     routes = make_routings(B, R, dev)
     g = torch.Generator().manual_seed(1)
@@ -482,6 +531,7 @@ def main():
         t = churn_leg(L, MB, ex, levels, routes[:16], xs, dev, native=False)
         churn["torch_copies"] = {k: t[k] for k in ("step_us_churn", "ops", "refused", "h2d_GBps", "lag_steps_median", "lag_steps_max")}
     stream = None if a.no_stream else stream_leg(dev)
+    config2 = None if a.no_config2 else config2_leg(L, ex, levels, dev)
     print(json.dumps({
         "metric": "MoE layer us + HBM GB/s (decode bs1 top-8); prefill grouped-GEMM TFLOP/s",
         "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": W,
@@ -491,7 +541,7 @@ def main():
         "config": {"workload": f"decode MoE layer: E=256 top-8 B={B}, H=6144 I=2048, levels 2/3/4 = "
                                f"{lv_counts[2]}/{lv_counts[3]}/{lv_counts[4]} experts, seeded softmax routing avoiding the previous step",
                    "code_MB_per_step": round(nbytes / K / 1e6, 2), "hbm_frac_layer": round(gbs / HBM_PEAK_GBS, 4)},
-        "roofline": roofline, "cpu_baseline": cpu, "prefill": prefill, "caller_dtypes": caller, "churn": churn, "stream": stream}))
+        "roofline": roofline, "cpu_baseline": cpu, "prefill": prefill, "caller_dtypes": caller, "churn": churn, "stream": stream, "config2": config2}))
 
 
 if __name__ == "__main__":
