@@ -139,6 +139,7 @@ class MoELayer:
         S = Bmax * topk
         f32, i32 = torch.float32, torch.int32
         s.cfg_gu, s.cfg_dn = s.default_cfg(H, I)
+        s._tuned = True                               # cfg_for may pick the tuned k-slice lengths; set_cfg switches that off
         s.h = torch.zeros(S, I, dtype=torch.float16, device=dev)
         s.cnt_gu = torch.zeros(S * (I // 128), dtype=i32, device=dev); s.cnt_d = torch.zeros(H // 128, dtype=i32, device=dev)
         s.wq = torch.zeros(4, dtype=i32, device=dev)
@@ -151,6 +152,19 @@ class MoELayer:
                                                       # that writes such rows into the table itself must set it, else the tokens
                                                       # that pick them come out NaN
         s._alloc_partials()
+
+    # k-slice lengths (chunks) per token count 1..8 at the full shape H = 6144, I = 2048, top-8 over 256 experts, measured on
+    # an MI355X with the routing of the layer benchmark; the reference keeps such tables for its GPUs
+    # (sm120/serve/nq_vllm.py:32-33). Index = tokens of the call; other shapes use default_cfg for every count.
+    TUNED_NST = {(6144, 2048): ([12, 12, 24, 12, 24, 12, 24, 24, 24], [8, 8, 16, 16, 8, 16, 16, 16, 16])}
+
+    def cfg_for(s, T):
+        """(cfg_gu, cfg_dn) for a decode call of T tokens: the layer's defaults, with the tuned k-slice length for T where this
+        shape has a table and set_cfg has not replaced the defaults"""
+        t = s.TUNED_NST.get((s.H, s.I)) if s._tuned else None
+        if t is None or T >= len(t[0]):
+            return s.cfg_gu, s.cfg_dn
+        return [s.cfg_gu[0], s.cfg_gu[1], t[0][T]], [s.cfg_dn[0], s.cfg_dn[1], t[1][T]]
 
     @staticmethod
     def default_cfg(H, I):
@@ -175,6 +189,7 @@ class MoELayer:
     def set_cfg(s, cfg_gu=None, cfg_dn=None):
         """change the default tilings (re-sizes the partial-sum workspaces; not graph-safe)"""
         s.cfg_gu, s.cfg_dn = list(cfg_gu or s.cfg_gu), list(cfg_dn or s.cfg_dn)
+        s._tuned = False
         s._alloc_partials()
 
     def set(s, e, ex, level):
@@ -197,7 +212,8 @@ class MoELayer:
         out = s.out[:B] if out is None else out
         assert out.dtype in _DT_OUT and out.is_contiguous(), out.dtype
         tb = s.table if table is None else table
-        cg, cd = list(cfg_gu or s.cfg_gu), list(cfg_dn or s.cfg_dn)
+        tg, td = s.cfg_for(B)
+        cg, cd = list(cfg_gu or tg), list(cfg_dn or td)
         s._alloc_partials(cg, cd)                    # grows only when a call brings a finer k-split than any before
         a = _lib.NqMoeArgs()
         a.x, a.sel, a.rw, a.table, a.out = x.data_ptr(), sel.data_ptr(), rw.data_ptr(), tb.data_ptr(), out.data_ptr()

@@ -143,7 +143,16 @@ def test_full_shape_layer_like_reference_check():
                 worst = max(worst, err)
                 assert err < 5e-5, (B, mode, cg, cd, err)
                 assert rel_err(y.cpu().numpy(), pure) < 1e-3, (B, mode, cg, cd)
+            # no tiling given: the k-slice lengths tuned for this shape and token count (the default ones at B = 1 and 3)
+            tg, td = L.cfg_for(B)
+            assert (tg[2], td[2]) == {1: (12, 8), 2: (24, 16), 3: (12, 16), 4: (24, 8)}[B] and tg[:2] == L.cfg_gu[:2]
+            y = L(x, sel, rw)
+            torch.cuda.synchronize()
+            assert rel_err(y.cpu().numpy(), want) < 5e-5 and torch.equal(y, L(x, sel, rw, cfg_gu=tg, cfg_dn=td))
     assert not L.cnt_gu.any() and not L.cnt_d.any()              # workspace counters are clean after the calls
+    L.set_cfg([1, 4, 6], None)                                   # explicit defaults win over the table
+    assert L.cfg_for(2) == ([1, 4, 6], L.cfg_dn)
+    assert M.MoELayer(4, 256, 128).cfg_for(2) == tuple(M.MoELayer.default_cfg(256, 128))     # no table for other shapes
     print("worst rel err vs the float64 oracle", worst)
 
 
