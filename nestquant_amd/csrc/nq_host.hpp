@@ -33,6 +33,9 @@ struct MoeArgs
     int* cnt_h;                       // arrival counters of the 512-column blocks (in_had_down = 512) [S * I/128]; may be null
     int G;                            // lanes per ring: 4, or 2 (the same planes read as rings of two records)
     int common_rows;                  // 1 = every row that can be picked has base window code 0 and no mask-mode flags; 0 = unknown
+    int fuse;                         // both launches belong to this call: for runs whose row has neither a low-rank plane nor the
+                                      // 512-wide rotation the down launch's staging does the gate|up finisher (set by launch_moe)
+    int ny_gu;                        // k-slices of the gate|up launch (the down launch's fused staging sums that many partials)
 };
 
 // kernel launchers defined next to their kernels

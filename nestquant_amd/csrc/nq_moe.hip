@@ -270,6 +270,10 @@ __device__ __forceinline__ void finish_gu(const MoeArgs& a, RunInfo& R, int z, i
         }
         float v0 = sw0 * (float)sud.x, v1 = sw1 * (float)sud.y;
         wht128(v0, v1, lane);
+        // h = fp16 of the fp32 rotation result (two roundings, as the reference's kernel and its torch restatement). Left alone,
+        // the compiler merges the rotation's last multiply into the conversion (v_fma_mixlo_f16: one rounding) at some call
+        // sites and not at others; this one and the down launch's staging must give the same bits.
+        asm volatile("" : "+v"(v0), "+v"(v1));
         if (wide) st_dev2(a.part_gu + (size_t)s * 2 * a.I + col, make_float2(v0, v1));
         else
         {
@@ -467,6 +471,39 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
             }
         }
     }
+    else if (a.fuse && R.had != 512 && R.lr == nullptr)
+    {
+        // The gate|up finisher, done here for this k-slice's columns of the run's tokens: g = WHT(sum of gate partials) * sv_g,
+        // u likewise, h = fp16(WHT(silu(g) * u * su_d)), written straight into the B-operand rows (same operations in the same
+        // order as finish_gu, so the same bits). Every column block of the run repeats it; in exchange the gate|up launch ends
+        // with its last partial sum and h makes no round trip through memory. Runs whose row has a low-rank plane or the
+        // 512-wide rotation keep the finisher in the gate|up launch: both launches read the same row, so they agree.
+        const _Float16 *sv_g = signs + a.H, *sv_u = sv_g + a.I, *su_d = sv_u + a.I;
+        const int Sgu = a.B * a.topk;
+        for (int task = warp; task < ntok * NC; task += SB)
+        {
+            const int j = task / NC, c = task - j * NC, col = k0 + c * 128 + 2 * lane;
+            const float* p = a.part_gu + (size_t)R.slot[j] * 2 * a.I + col;
+            const float* const rows2[2] = {p, p + a.I};
+            const half2_t svg = *(const half2_t*)(sv_g + col), svu = *(const half2_t*)(sv_u + col), sud = *(const half2_t*)(su_d + col);
+            float2 pq[2];
+            sum_partials<2>(rows2, (size_t)Sgu * 2 * a.I, a.ny_gu, pq);
+            float g0 = pq[0].x, g1 = pq[0].y, u0 = pq[1].x, u1 = pq[1].y;
+            wht128(g0, g1, lane); wht128(u0, u1, lane);
+            g0 *= (float)svg.x; g1 *= (float)svg.y; u0 *= (float)svu.x; u1 *= (float)svu.y;
+            const float sw0 = g0 / (1.f + __expf(-g0)) * u0, sw1 = g1 / (1.f + __expf(-g1)) * u1;
+            float v0 = sw0 * (float)sud.x, v1 = sw1 * (float)sud.y;
+            wht128(v0, v1, lane);
+            asm volatile("" : "+v"(v0), "+v"(v1));            // as in finish_gu: the scaled fp32 value is rounded to fp16, in two steps
+            _Float16* dst = (_Float16*)(smem + j * rowstride + c * 256);
+            dst[bop_index(2 * lane)] = (_Float16)v0; dst[bop_index(2 * lane + 1)] = (_Float16)v1;
+            if (blockIdx.x == 0)                                 // h stays inspectable, as the gate|up finisher leaves it
+            {
+                half2_t hv; hv.x = (_Float16)v0; hv.y = (_Float16)v1;
+                *(half2_t*)(a.h + (size_t)R.slot[j] * a.I + col) = hv;
+            }
+        }
+    }
     else
     {
         for (int i = threadIdx.x; i < ntok * NC * 64; i += blockDim.x)
@@ -507,6 +544,9 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
         st_dev4(part + row, acc[0]);
         st_dev4(part + row + 8, acc[1]);
     }
+
+    // fused finisher: the down launch's staging forms h from these partial sums itself (no arrival counter, no finisher here)
+    if (MODE == 0 && a.fuse && R.had != 512 && R.lr == nullptr) return;   // block-uniform (a property of the run's row)
 
     // ---- arrival counter of the 128-row group this block belongs to; the last block to arrive finishes the group
     const int rows0 = blockIdx.x * SB * 32;
@@ -551,13 +591,16 @@ int launch_moe(const MoeArgs& a, const int* cfg_gu, const int* cfg_dn, int which
         const int NX = N / 32 / SB, NY = C / NC;
         const int shm = std::max(a.B * (NC * 256 + 16) + 256, SB * 512);
         const bool any = a.common_rows != 1;
+        MoeArgs b = a;
+        b.fuse = which == 3;                                      // both launches belong to this call
+        b.ny_gu = (a.H / 128) / (cfg_gu[0] * cfg_gu[2]);
         auto kern = mode == 0 ? (any ? nq_gemv_k<0, true> : nq_gemv_k<0, false>) : (any ? nq_gemv_k<1, true> : nq_gemv_k<1, false>);
         if (shm > 48 * 1024)
         {
             hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, shm);
             if (e != hipSuccess) return set_error("moe_forward: LDS %d bytes: %s", shm, hipGetErrorString(e));
         }
-        kern<<<dim3(NX, NY, S), 64 * SB, shm, st>>>(a, NC);
+        kern<<<dim3(NX, NY, S), 64 * SB, shm, st>>>(b, NC);
         NQ_LAUNCH_CHECK("moe_forward");
     }
     return 0;

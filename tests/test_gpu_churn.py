@@ -2,6 +2,7 @@
 equal the float64 oracle of the level state it actually applied, every swapped expert must dequantise bit-exactly, and the
 slot / table invariants must hold (reference sm120/levelswitch_mbox.py, sm120/serve/nq_slotcheck.py)."""
 import random
+import time
 
 import numpy as np
 import pytest
@@ -108,6 +109,11 @@ def test_churn_racing_graph_replays(native):
     # the engine's ops land a thread hop later than copies issued from this thread, so fewer experts are idle when picked
     assert nops > (20 if native else 30) and changed > (5 if native else 10) and X.bytes_copied > 0
     if native:
+        for _ in range(2000):                                    # the engine reports an op a moment after its copies completed
+            X.poll()
+            if len(X.lat) == nops:
+                break
+            time.sleep(0.001)
         st_ = X.eng.stats()
         assert st_["upload_bytes"] == X.bytes_copied and st_["uploads"] + st_["posts"] == nops and len(X.lat) == nops
     X.close()

@@ -413,3 +413,46 @@ def test_occupancy_query_matches_the_launch_shape_the_layer_uses():
     assert M.occ(0, 4, 4096, any_rows=True)[0] >= 1
     with pytest.raises(RuntimeError, match="nq_occ"):
         M.occ(2, 4, 0)
+
+
+def test_finisher_in_the_down_launch_gives_the_same_bits(golden_dir):
+    """One call with both launches (which = 3) lets the down launch's staging form h from the gate|up partial sums for runs
+    whose row has neither a low-rank plane nor the 512-wide rotation; those runs keep the finisher in the gate|up launch.
+    The same layer call issued as two calls (which = 1, then which = 2) always runs the finisher in the gate|up launch.
+    Both must give the same bits: rows of both kinds in one call, 1-4 tokens, several tilings, and at the full shape."""
+    z, L, ex, x, sel, rw = _optional_feature_layer(golden_dir, 128, False)
+    H, I = int(z["H"]), int(z["I"])
+    from tests.test_oracle_golden import LR_NAMES
+    ex[1].set_lr(*[torch.from_numpy(z[f"lr1_{n}"].view(np.float16).copy()) for n in LR_NAMES])   # expert 1: low-rank plane
+    ex[2].had_dn = 512                                                                             # expert 2: 512-wide rotation
+    for e in range(3):
+        L.set(e, ex[e], int(z["levels"][e]))                                                       # expert 0 stays plain
+    g = torch.Generator().manual_seed(5)
+    for B in (1, 2):
+        xb = (torch.randn(B, H, generator=g) * 0.3).half().to(DEV)
+        sb = torch.stack([torch.randperm(3, generator=g) for _ in range(B)]).to(DEV)
+        wb = (torch.rand(B, 3, generator=g) + 0.1).half().to(DEV)
+        for cg, cd in (([1, 4, 2], [1, 4, 4]), ([1, 4, 1], [1, 2, 1]), ([1, 2, 2], [1, 1, 2])):
+            L.h.fill_(float("nan"))                              # h of the plain run is not needed by the one-call form
+            y3 = L(xb, sb, wb, cfg_gu=cg, cfg_dn=cd).clone()
+            L(xb, sb, wb, which=1, cfg_gu=cg, cfg_dn=cd)
+            y12 = L(xb, sb, wb, which=2, cfg_gu=cg, cfg_dn=cd).clone()
+            torch.cuda.synchronize()
+            assert torch.isfinite(y3).all() and torch.equal(y3, y12), (B, cg, cd)
+            assert not L.cnt_gu.any() and not L.cnt_d.any() and not L.cnt_h.any()
+    # full shape, plain rows at levels 2 / 3 / 4, 1-4 tokens, the tuned tilings
+    H, I, NE = 6144, 2048, 10
+    levels = [2, 4, 3, 2, 4, 2, 3, 4, 2, 2]
+    exs = to_dev(experts_on_gpu(H, I, NE, 300, nested_ids=tuple(range(NE))))
+    L = M.MoELayer(NE, H, I, Bmax=4)
+    for e in range(NE):
+        L.set(e, exs[e], levels[e])
+    for B in (1, 2, 3, 4):
+        xb = (torch.randn(B, H, generator=g) * 0.05).half().to(DEV)
+        sb = torch.stack([torch.randperm(NE, generator=g)[:8] for _ in range(B)]).to(DEV)
+        wb = torch.softmax(torch.randn(B, 8, generator=g), -1).half().to(DEV)
+        y3 = L(xb, sb, wb).clone()
+        L(xb, sb, wb, which=1)
+        y12 = L(xb, sb, wb, which=2).clone()
+        torch.cuda.synchronize()
+        assert torch.isfinite(y3).all() and y3.abs().max() > 0 and torch.equal(y3, y12), B
