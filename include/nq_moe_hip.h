@@ -76,7 +76,10 @@ typedef struct NqMoeArgs
     const int64_t* table;     /* int64 [E][NQ_TBL_W] */
     void* out;                /* [B][H], out_dtype */
     void* acc_gu;             /* fp32 workspace */
-    void* h;                  /* fp16 workspace */
+    void* h;                  /* fp16 [B*topk, I]: rotated SwiGLU output of every pick, input of the down launch. Written by the
+                                 gate|up launch (which = 1, and runs whose row has a low-rank plane or in_had_down = 512) or,
+                                 when both launches belong to the call (which = 3), by the down launch, which then forms it from
+                                 the gate|up partial sums itself; same bits either way */
     void* acc_d;              /* fp32 workspace */
     int32_t* cnt_gu;          /* int32 workspace, zero on entry */
     int32_t* cnt_d;           /* int32 workspace, zero on entry */
