@@ -135,3 +135,25 @@ def test_shadow_posts_level_2_rows_and_io_stats_reports_intervals():
     assert st["landed_cum"] == 1 and st["ops_outstanding"] == 0 and st["free_slots"] == 1 and st["slot_wait"] == 0
     assert abs(st["op_p50_ms"] - 6.0) < 1e-6 and abs(st["rd_p50_ms"] - 4.0) < 1e-6 and abs(st["cp_p50_ms"] - 2.0) < 1e-6
     assert st["delivered_GBps"] > 0 and ex.io_stats()["delivered_GBps"] == 0       # second call: nothing since the first
+
+
+def test_rank_file_index_and_row_arguments(tmp_path):
+    import json
+    import numpy as np
+    from nestquant_amd import stream_engine as SE
+    idx = dict(format="nq-p4rec-v1", tp=4, rank=2, L0=3, NE=256, rec_bytes=8192, seg={"gu.p4": [0, 4096], "gu.d4": [4096, 256]}, layers={})
+    (tmp_path / "rank2.json").write_text(json.dumps(idx))
+    rf = SE.RankFile(str(tmp_path), 2)
+    assert rf.path == f"{tmp_path}/rank2.bin" and rf.rb == 8192 and rf.lay == dict(seg=idx["seg"], rec_bytes=8192)
+    assert rf.rec(3, 0) == 0 and rf.rec(5, 17) == 2 * 256 + 17                     # ((L - L0) * NE + E), streaming/stream_engine.py:21
+    assert SE.mod().Engine is SE.Engine
+    # a row is int64[20] from a CPU tensor, a numpy array or a list; anything else is refused as the reference's binding does
+    for row in (torch.arange(20), np.arange(20, dtype=np.int64), list(range(20))):
+        assert list(SE._row_array(row)) == list(range(20))
+    for bad in (torch.arange(19), torch.arange(20, dtype=torch.int32), list(range(21))):
+        try:
+            SE._row_array(bad)
+        except RuntimeError as e:
+            assert "int64 cpu [20]" in str(e)
+        else:
+            raise AssertionError("accepted a malformed row")
