@@ -110,6 +110,20 @@ typedef struct NqMoeArgs
 } NqMoeArgs;
 int nq_moe_forward(const NqMoeArgs* args, void* stream);
 
+/* nq_moe_forward for callers that cannot allocate device memory or keep workspaces of their own (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc). It has no counterpart in the reference, whose MoELayer
+ * always owns its workspaces (sm120/moe.py:231-241). Same arguments, kernels and results as nq_moe_forward, except that the
+ * workspace fields of *args (acc_gu, h, acc_d, cnt_gu, cnt_d, cnt_h, zd and their capacities) are not looked at: partial
+ * sums, h, z_d and the arrival counters live in one array of NQ_STATIC_SCRATCH_BYTES that is part of the library's device
+ * image (every GPU the library runs on holds its own copy until the process ends). The call allocates and frees nothing; it
+ * clears the counters with a small kernel, then makes the two launches. A call whose shape and k-slices need more than the
+ * array holds is refused with an error (full shape H=6144, I=2048, B*topk=64 picks with the default k-slices: about 7.3 MiB).
+ * All calls on one GPU share the array: calls that overlap on one GPU (different streams) race; order them on one stream.
+ * The first call on a device looks up the array's address (hipGetSymbolAddress) and so must not be made under stream
+ * capture; later calls may be. */
+#define NQ_STATIC_SCRATCH_BYTES (16u << 20)
+int nq_moe_forward_static(const NqMoeArgs* args, void* stream);
+
 /* table[e] <- stage[e] for every e with seq[e] != applied[e]; then applied[e] <- seq[e], mirrored to applied_host
  * [host-mapped, optional]. Replaces mailbox (reference sm120/nqmoe.cu:908-929). */
 int nq_mailbox(int64_t* table, const int64_t* stage, const int32_t* seq, int32_t* applied, int32_t* applied_host, int E,

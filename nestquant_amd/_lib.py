@@ -35,6 +35,7 @@ SIGNATURES = {
     "nq_dequant": (C.c_int, [_i64p, _i, _i, _i, _i, _vp, _vp]),
     "nq_pf_decode": (C.c_int, [_i64p, _i32p, _i, _vp, _vp, _i, _i, _vp]),
     "nq_moe_forward": (C.c_int, [C.POINTER(NqMoeArgs), _vp]),
+    "nq_moe_forward_static": (C.c_int, [C.POINTER(NqMoeArgs), _vp]),
     "nq_sal": (C.c_int, [_vp, _i, C.c_int64, _vp, _i, _vp, _i, _i, _i, _i, _i, C.c_double, _vp, _vp, _vp]),
     "nq_mailbox": (C.c_int, [_i64p, _i64p, _i32p, _i32p, _i32p, _i, _vp]),
     "nq_pf_pre": (C.c_int, [_vp, _i32p, _i32p, _i, _i64p, _vp, _vp, _vp, _i, _i, _i, _vp]),

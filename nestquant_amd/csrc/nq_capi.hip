@@ -95,19 +95,22 @@ extern "C" int nq_sal(const void* x, int x_dtype, int64_t x_row_stride, const vo
     return launch_sal(x, x_dtype, x_row_stride, w, w_dtype, ids, ids_dtype, T, H, K, E, (float)rsf, acc, host, (hipStream_t)stream);
 }
 
-extern "C" int nq_moe_forward(const NqMoeArgs* p, void* stream)
+// checks shared by the two decode entry points; own_ws: the caller brings the workspaces (nq_moe_forward), else they are
+// carved from the library's built-in scratch (nq_moe_forward_static) and the workspace fields of *p are not looked at
+static int moe_args(const char* who, const NqMoeArgs* p, bool own_ws, MoeArgs& a)
 {
-    NQ_REQUIRE(p, "nq_moe_forward: null args");
-    NQ_REQUIRE(p->x && p->sel && p->rw && p->table && p->out && p->acc_gu && p->h && p->acc_d && p->cnt_gu && p->cnt_d, "nq_moe_forward: null pointer");
-    NQ_REQUIRE(p->B >= 1 && p->B <= 8 && p->topk >= 1 && p->B * p->topk <= 64, "nq_moe_forward: B=%d topk=%d (B <= 8, B*topk <= 64)", p->B, p->topk);
-    NQ_REQUIRE(p->E >= 1, "nq_moe_forward: E=%d", p->E);
-    NQ_REQUIRE(shape_ok(p->H, p->I), "nq_moe_forward: H=%d I=%d must be positive multiples of 128", p->H, p->I);
-    NQ_REQUIRE((p->which & ~3) == 0, "nq_moe_forward: which=%d", p->which);
-    NQ_REQUIRE(p->force_level == 0 || p->force_level == 2 || p->force_level == 3 || p->force_level == 4, "nq_moe_forward: force_level=%d", p->force_level);
+    NQ_REQUIRE(p, "%s: null args", who);
+    NQ_REQUIRE(p->x && p->sel && p->rw && p->table && p->out, "%s: null pointer", who);
+    NQ_REQUIRE(!own_ws || (p->acc_gu && p->h && p->acc_d && p->cnt_gu && p->cnt_d), "%s: null workspace pointer", who);
+    NQ_REQUIRE(p->B >= 1 && p->B <= 8 && p->topk >= 1 && p->B * p->topk <= 64, "%s: B=%d topk=%d (B <= 8, B*topk <= 64)", who, p->B, p->topk);
+    NQ_REQUIRE(p->E >= 1, "%s: E=%d", who, p->E);
+    NQ_REQUIRE(shape_ok(p->H, p->I), "%s: H=%d I=%d must be positive multiples of 128", who, p->H, p->I);
+    NQ_REQUIRE((p->which & ~3) == 0, "%s: which=%d", who, p->which);
+    NQ_REQUIRE(p->force_level == 0 || p->force_level == 2 || p->force_level == 3 || p->force_level == 4, "%s: force_level=%d", who, p->force_level);
     NQ_REQUIRE(p->x_dtype >= 0 && p->x_dtype <= 2 && p->rw_dtype >= 0 && p->rw_dtype <= 2 && p->sel_dtype >= 0 && p->sel_dtype <= 1 && p->out_dtype >= 0 && p->out_dtype <= 2,
-               "nq_moe_forward: dtype codes x=%d sel=%d rw=%d out=%d", p->x_dtype, p->sel_dtype, p->rw_dtype, p->out_dtype);
-    NQ_REQUIRE(aligned16(p->x) && aligned16(p->out) && aligned16(p->acc_gu) && aligned16(p->acc_d) && aligned16(p->h),
-               "nq_moe_forward: x, out, acc_gu, acc_d and h must be 16-byte aligned");
+               "%s: dtype codes x=%d sel=%d rw=%d out=%d", who, p->x_dtype, p->sel_dtype, p->rw_dtype, p->out_dtype);
+    NQ_REQUIRE(aligned16(p->x) && aligned16(p->out), "%s: x and out must be 16-byte aligned", who);
+    NQ_REQUIRE(!own_ws || (aligned16(p->acc_gu) && aligned16(p->acc_d) && aligned16(p->h)), "%s: acc_gu, acc_d and h must be 16-byte aligned", who);
     const int64_t S = (int64_t)p->B * p->topk;
     for (int mode = 0; mode < 2; ++mode)
     {
@@ -118,25 +121,42 @@ extern "C" int nq_moe_forward(const NqMoeArgs* p, void* stream)
         NQ_REQUIRE(C % NC == 0 && (SB == 1 || SB == 2 || SB == 4) && NC <= 48,
                    "bad cfg: k-slice %d chunks of %d, %d wavefronts per block for N=%d (sb must be 1, 2 or 4)", NC, C, SB, N);
         const int64_t need = (int64_t)(C / NC) * S * N, have = mode == 0 ? p->acc_gu_elems : p->acc_d_elems;
-        NQ_REQUIRE(have >= need, "workspace too small: %s holds %lld floats, needs %lld", mode == 0 ? "acc_gu" : "acc_d", (long long)have, (long long)need);
+        NQ_REQUIRE(!own_ws || have >= need, "workspace too small: %s holds %lld floats, needs %lld", mode == 0 ? "acc_gu" : "acc_d", (long long)have, (long long)need);
     }
-    NQ_REQUIRE(p->h_elems >= S * p->I && p->out_elems >= (int64_t)p->B * p->H, "workspace too small: h or out");
-    NQ_REQUIRE(p->cnt_gu_elems >= S * (p->I / 128) && p->cnt_d_elems >= p->H / 128, "workspace too small: cnt_gu or cnt_d");
-    MoeArgs a{};
+    NQ_REQUIRE(p->out_elems >= (int64_t)p->B * p->H, "workspace too small: out");
+    a = MoeArgs{};
     a.x = p->x; a.sel = p->sel; a.rw = p->rw; a.B = p->B; a.topk = p->topk;
     a.x_dtype = p->x_dtype; a.sel_dtype = p->sel_dtype; a.rw_dtype = p->rw_dtype; a.out_dtype = p->out_dtype;
     a.table = p->table; a.E = p->E; a.H = p->H; a.I = p->I;
-    a.part_gu = (float*)p->acc_gu; a.h = (_Float16*)p->h; a.part_d = (float*)p->acc_d; a.out = p->out;
-    a.force_level = p->force_level; a.hits = p->hits; a.cnt_gu = p->cnt_gu; a.cnt_d = p->cnt_d;
-    NQ_REQUIRE(p->cnt_h && p->cnt_h_elems >= S * (p->I / 128), "workspace too small: cnt_h");
-    a.cnt_h = p->cnt_h;
-    NQ_REQUIRE(p->zd && p->zd_elems >= S * (p->I / 128) * 4, "workspace too small: zd");
-    a.zd = (float*)p->zd;
-    NQ_REQUIRE(p->common_rows == 0 || p->common_rows == 1, "nq_moe_forward: common_rows=%d (0 or 1)", p->common_rows);
+    a.out = p->out; a.force_level = p->force_level; a.hits = p->hits;
+    if (own_ws)
+    {
+        NQ_REQUIRE(p->h_elems >= S * p->I, "workspace too small: h");
+        NQ_REQUIRE(p->cnt_gu_elems >= S * (p->I / 128) && p->cnt_d_elems >= p->H / 128, "workspace too small: cnt_gu or cnt_d");
+        NQ_REQUIRE(p->cnt_h && p->cnt_h_elems >= S * (p->I / 128), "workspace too small: cnt_h");
+        NQ_REQUIRE(p->zd && p->zd_elems >= S * (p->I / 128) * 4, "workspace too small: zd");
+        a.part_gu = (float*)p->acc_gu; a.h = (_Float16*)p->h; a.part_d = (float*)p->acc_d;
+        a.cnt_gu = p->cnt_gu; a.cnt_d = p->cnt_d; a.cnt_h = p->cnt_h; a.zd = (float*)p->zd;
+    }
+    NQ_REQUIRE(p->common_rows == 0 || p->common_rows == 1, "%s: common_rows=%d (0 or 1)", who, p->common_rows);
     a.common_rows = p->common_rows;
-    NQ_REQUIRE(p->G == 0 || p->G == 4 || p->G == 2, "nq_moe_forward: G=%d (rings of 4 lanes, or 2)", p->G);
+    NQ_REQUIRE(p->G == 0 || p->G == 4 || p->G == 2, "%s: G=%d (rings of 4 lanes, or 2)", who, p->G);
     a.G = p->G == 2 ? 2 : 4;
+    return 0;
+}
+
+extern "C" int nq_moe_forward(const NqMoeArgs* p, void* stream)
+{
+    MoeArgs a;
+    if (int rc = moe_args("nq_moe_forward", p, true, a)) return rc;
     return launch_moe(a, p->cfg_gu, p->cfg_dn, p->which, (hipStream_t)stream);
+}
+
+extern "C" int nq_moe_forward_static(const NqMoeArgs* p, void* stream)
+{
+    MoeArgs a;
+    if (int rc = moe_args("nq_moe_forward_static", p, false, a)) return rc;
+    return launch_moe_static(a, p->cfg_gu, p->cfg_dn, p->which, (hipStream_t)stream);
 }
 
 extern "C" int nq_mailbox(int64_t* table, const int64_t* stage, const int32_t* seq, int32_t* applied, int32_t* applied_host, int E, void* stream)

@@ -40,6 +40,7 @@ struct MoeArgs
 
 // kernel launchers defined next to their kernels
 int launch_moe(const MoeArgs& a, const int* cfg_gu, const int* cfg_dn, int which, hipStream_t st);
+int launch_moe_static(MoeArgs a, const int* cfg_gu, const int* cfg_dn, int which, hipStream_t st);
 int query_occ(int mode, int any_rows, int sb, int shm, int* out);
 int launch_mailbox(int64_t* table, const int64_t* stage, const int32_t* seq, int32_t* applied, int32_t* applied_host, int E, hipStream_t st);
 int launch_dequant(const int64_t* row, int proj, int level, int H, int I, void* out, hipStream_t st);

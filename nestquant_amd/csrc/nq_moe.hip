@@ -19,6 +19,8 @@
 #include "nq_tile.hpp"
 #include "nq_host.hpp"
 #include <algorithm>
+#include <mutex>
+#include "../../include/nq_moe_hip.h"
 
 namespace nq {
 
@@ -604,6 +606,60 @@ int launch_moe(const MoeArgs& a, const int* cfg_gu, const int* cfg_dn, int which
         NQ_LAUNCH_CHECK("moe_forward");
     }
     return 0;
+}
+
+// ---- nq_moe_forward_static: the same two launches with every workspace carved from one built-in device array --------------
+// For callers that cannot allocate (stream capture, serving loops, harnesses that forbid hipMalloc). Each GPU holds its own
+// copy of the array at its own address; in host code the array's name is only a handle for hipGetSymbolAddress, which is
+// asked once per device, with that device current, and the address it returns is what the kernels are given. Calls on one
+// GPU share the array: two calls that overlap on one GPU (different streams) race.
+constexpr size_t STATIC_SCRATCH_BYTES = (size_t)NQ_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+constexpr int MAX_DEVICES = 64;
+static unsigned char* g_scratch_ptr[MAX_DEVICES] = {};
+static std::mutex g_scratch_mu;
+
+__global__ void nq_clear_k(int* p, int n)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+
+int launch_moe_static(MoeArgs a, const int* cfg_gu, const int* cfg_dn, int which, hipStream_t st)
+{
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return set_error("nq_moe_forward_static: current device %d: %s", dev, hipGetErrorString(e));
+    unsigned char* base;
+    {
+        std::lock_guard<std::mutex> lk(g_scratch_mu);
+        if (!g_scratch_ptr[dev])
+        {
+            void* ptr = nullptr;
+            e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+            if (e != hipSuccess || !ptr) return set_error("nq_moe_forward_static: address of the built-in scratch on device %d: %s", dev, hipGetErrorString(e));
+            g_scratch_ptr[dev] = (unsigned char*)ptr;
+        }
+        base = g_scratch_ptr[dev];
+    }
+    const size_t S = (size_t)a.B * a.topk, G128 = (size_t)a.I / 128;
+    const size_t ny_gu = (size_t)(a.H / 128) / (cfg_gu[0] * cfg_gu[2]), ny_dn = (size_t)(a.I / 128) / (cfg_dn[0] * cfg_dn[2]);
+    size_t off = 0;
+    auto take = [&](size_t bytes) { const size_t o = off; off += (bytes + 255) & ~(size_t)255; return o; };
+    const size_t o_cnt = take((2 * S * G128 + (size_t)a.H / 128) * sizeof(int));       // cnt_gu | cnt_h | cnt_d: cleared below
+    const size_t o_gu = take(ny_gu * S * 2 * a.I * sizeof(float)), o_d = take(ny_dn * S * a.H * sizeof(float));
+    const size_t o_h = take(S * a.I * sizeof(_Float16)), o_zd = take(S * G128 * 4 * sizeof(float));
+    if (off > STATIC_SCRATCH_BYTES)
+        return set_error("nq_moe_forward_static: this call needs %zu bytes of workspace (B=%d topk=%d H=%d I=%d, %zu and %zu k-slices), the built-in "
+                         "scratch holds %zu: use coarser k-slices, or nq_moe_forward with workspaces of the caller's", off, a.B, a.topk, a.H, a.I, ny_gu, ny_dn,
+                         STATIC_SCRATCH_BYTES);
+    a.cnt_gu = (int*)(base + o_cnt); a.cnt_h = a.cnt_gu + S * G128; a.cnt_d = a.cnt_h + S * G128;
+    a.part_gu = (float*)(base + o_gu); a.part_d = (float*)(base + o_d); a.h = (_Float16*)(base + o_h); a.zd = (float*)(base + o_zd);
+    // the counters must be zero on entry; a fill kernel, not hipMemsetAsync, so that the call can be recorded into a graph
+    const int ncnt = (int)(2 * S * G128 + (size_t)a.H / 128);
+    nq_clear_k<<<(ncnt + 255) / 256, 256, 0, st>>>(a.cnt_gu, ncnt);
+    NQ_LAUNCH_CHECK("nq_moe_forward_static");
+    return launch_moe(a, cfg_gu, cfg_dn, which, st);
 }
 
 // resident workgroups per CU, registers and spill bytes of a decode kernel for a launch shape

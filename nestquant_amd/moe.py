@@ -200,12 +200,14 @@ class MoELayer:
         s.rare_rows |= bool(row[4] or row[8] or row[19])
         s.table[e].copy_(row.to(s.table.device), non_blocking=False)
 
-    def __call__(s, x, sel, rw, out=None, force_level=0, which=3, cfg_gu=None, cfg_dn=None, table=None):
+    def __call__(s, x, sel, rw, out=None, force_level=0, which=3, cfg_gu=None, cfg_dn=None, table=None, static_ws=False):
         """x [B, H], sel [B, topk], rw [B, topk] -> fp32 [B, H] (s.out[:B] unless `out` is given). As in the reference x
         and rw are fp16 and sel int64; the kernels also take x / rw in bf16 or fp32, sel in int32 and `out` in fp16 or
         bf16, with the roundings of x.half(), rw.half() and out.to(dtype) (the casts the reference's caller launches as
         separate kernels, sm120/serve/nq_vllm.py:522,560).
-        table: optional [E, TBL_W] override. Everything is enqueued on torch's current stream; nothing syncs."""
+        table: optional [E, TBL_W] override. Everything is enqueued on torch's current stream; nothing syncs.
+        static_ws: go through nq_moe_forward_static, which ignores this layer's workspaces and uses the library's built-in
+        device scratch instead (for callers that must not allocate; calls on one GPU then share that scratch)."""
         assert x.dtype in _DT_IN and rw.dtype in _DT_IN and sel.dtype in _DT_SEL, (x.dtype, rw.dtype, sel.dtype)
         assert x.is_contiguous() and sel.is_contiguous() and rw.is_contiguous()
         B, topk = sel.shape
@@ -214,7 +216,8 @@ class MoELayer:
         tb = s.table if table is None else table
         tg, td = s.cfg_for(B)
         cg, cd = list(cfg_gu or tg), list(cfg_dn or td)
-        s._alloc_partials(cg, cd)                    # grows only when a call brings a finer k-split than any before
+        if not static_ws:
+            s._alloc_partials(cg, cd)                # grows only when a call brings a finer k-split than any before
         a = _lib.NqMoeArgs()
         a.x, a.sel, a.rw, a.table, a.out = x.data_ptr(), sel.data_ptr(), rw.data_ptr(), tb.data_ptr(), out.data_ptr()
         a.acc_gu, a.h, a.acc_d, a.hits = s.acc_gu.data_ptr(), s.h.data_ptr(), s.acc_d.data_ptr(), s.hits_ptr or None
@@ -229,7 +232,7 @@ class MoELayer:
         a.G = s.G
         a.common_rows = int(table is None and not s.rare_rows)     # a caller's own table: unknown
         a.x_dtype, a.sel_dtype, a.rw_dtype, a.out_dtype = _DT_IN[x.dtype], _DT_SEL[sel.dtype], _DT_IN[rw.dtype], _DT_OUT[out.dtype]
-        _lib.check(s.M.nq_moe_forward(C.byref(a), _lib.stream_ptr()))
+        _lib.check((s.M.nq_moe_forward_static if static_ws else s.M.nq_moe_forward)(C.byref(a), _lib.stream_ptr()))
         return out
 
 
