@@ -440,8 +440,7 @@ def main():
     outs = torch.zeros(R, B, H, dtype=torch.float32, device=dev)
 
     def step(i):
-        MB.apply()
-        L(xs[i], routes[i][0], routes[i][1], out=outs[i])
+        L(xs[i], routes[i][0], routes[i][1], out=outs[i], mailbox=MB)        # the mailbox is applied by the call's first launch
 
     s = torch.cuda.Stream()
     with torch.cuda.stream(s):

@@ -20,7 +20,7 @@ extern "C" {
 #endif
 
 #define NQ_TBL_W 20
-#define NQ_ABI_VERSION 1
+#define NQ_ABI_VERSION 2
 
 /* library identification; no counterpart in the reference (its module is rebuilt per process by sm120/build.py:7-12) */
 int nq_abi_version(void);
@@ -107,14 +107,28 @@ typedef struct NqMoeArgs
     int32_t G;                /* lanes per ring (reference moe_forward's G, sm120/nqmoe.cu:223-228,862): 0 or 4 = rings of four
                                  records (the format every artifact uses), 2 = the same planes read as rings of two records
                                  (the reference's test variant; not with sign-variant planes, not in prefill) */
+    void* route_ws;           /* NQ_ROUTE_WS_BYTES of device memory, 64-byte aligned, contents irrelevant on entry: the call's first
+                                 launch (one workgroup) does the routing once -- picks -> runs of distinct experts with their table
+                                 rows (reference route(), sm120/nqmoe.cu:379-449, which every block of the reference repeats) -- and
+                                 leaves it here for the two projection launches */
+    int64_t route_ws_bytes;
+    int64_t* mb_table;        /* optional mailbox, applied by the call's first launch before it reads the table: exactly
+                                 nq_mailbox(mb_table, mb_stage, mb_seq, mb_applied, mb_applied_host, E) followed by the layer call, in
+                                 one launch less (the reference's caller applies the mailbox at the top of every layer step,
+                                 sm120/serve/nq_vllm.py:546). NULL = no mailbox in this call; otherwise normally == table */
+    const int64_t* mb_stage;
+    const int32_t* mb_seq;
+    int32_t* mb_applied;
+    int32_t* mb_applied_host; /* [host-mapped], may be NULL */
 } NqMoeArgs;
+#define NQ_ROUTE_WS_BYTES 32768
 int nq_moe_forward(const NqMoeArgs* args, void* stream);
 
 /* nq_moe_forward for callers that cannot allocate device memory or keep workspaces of their own (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc). It has no counterpart in the reference, whose MoELayer
  * always owns its workspaces (sm120/moe.py:231-241). Same arguments, kernels and results as nq_moe_forward, except that the
- * workspace fields of *args (acc_gu, h, acc_d, cnt_gu, cnt_d, cnt_h, zd and their capacities) are not looked at: partial
- * sums, h, z_d and the arrival counters live in one array of NQ_STATIC_SCRATCH_BYTES that is part of the library's device
+ * workspace fields of *args (acc_gu, h, acc_d, cnt_gu, cnt_d, cnt_h, zd, route_ws and their capacities) are not looked at:
+ * partial sums, h, z_d, the routing result and the arrival counters live in one array of NQ_STATIC_SCRATCH_BYTES that is part of the library's device
  * image (every GPU the library runs on holds its own copy until the process ends). The call allocates and frees nothing; it
  * clears the counters with a small kernel, then makes the two launches. A call whose shape and k-slices need more than the
  * array holds is refused with an error (full shape H=6144, I=2048, B*topk=64 picks with the default k-slices: about 7.3 MiB).

@@ -22,7 +22,13 @@ class NqMoeArgs(C.Structure):
                 ("cfg_gu", C.c_int32 * 4), ("cfg_dn", C.c_int32 * 4), ("force_level", C.c_int32), ("which", C.c_int32),
                 ("x_dtype", C.c_int32), ("sel_dtype", C.c_int32), ("rw_dtype", C.c_int32), ("out_dtype", C.c_int32),
                 ("cnt_h", C.c_void_p), ("cnt_h_elems", C.c_int64), ("zd", C.c_void_p), ("zd_elems", C.c_int64),
-                ("common_rows", C.c_int32), ("G", C.c_int32)]
+                ("common_rows", C.c_int32), ("G", C.c_int32),
+                ("route_ws", C.c_void_p), ("route_ws_bytes", C.c_int64),
+                ("mb_table", C.c_void_p), ("mb_stage", C.c_void_p), ("mb_seq", C.c_void_p), ("mb_applied", C.c_void_p),
+                ("mb_applied_host", C.c_void_p)]
+
+
+ROUTE_WS_BYTES = 32768          # NQ_ROUTE_WS_BYTES
 
 
 # name -> (restype, argtypes); every symbol declared in include/nq_moe_hip.h

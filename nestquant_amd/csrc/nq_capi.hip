@@ -137,6 +137,14 @@ static int moe_args(const char* who, const NqMoeArgs* p, bool own_ws, MoeArgs& a
         NQ_REQUIRE(p->zd && p->zd_elems >= S * (p->I / 128) * 4, "workspace too small: zd");
         a.part_gu = (float*)p->acc_gu; a.h = (_Float16*)p->h; a.part_d = (float*)p->acc_d;
         a.cnt_gu = p->cnt_gu; a.cnt_d = p->cnt_d; a.cnt_h = p->cnt_h; a.zd = (float*)p->zd;
+        NQ_REQUIRE(p->route_ws && p->route_ws_bytes >= NQ_ROUTE_WS_BYTES && ((uintptr_t)p->route_ws & 63) == 0,
+                   "workspace too small: route_ws needs %d bytes, 64-byte aligned", NQ_ROUTE_WS_BYTES);
+        a.route = (RouteWs*)p->route_ws;
+    }
+    if (p->mb_table)
+    {
+        NQ_REQUIRE(p->mb_stage && p->mb_seq && p->mb_applied, "%s: mailbox needs stage, seq and applied", who);
+        a.mb_table = p->mb_table; a.mb_stage = p->mb_stage; a.mb_seq = p->mb_seq; a.mb_applied = p->mb_applied; a.mb_applied_host = p->mb_applied_host;
     }
     NQ_REQUIRE(p->common_rows == 0 || p->common_rows == 1, "%s: common_rows=%d (0 or 1)", who, p->common_rows);
     a.common_rows = p->common_rows;

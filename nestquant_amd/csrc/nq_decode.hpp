@@ -230,7 +230,7 @@ __device__ __forceinline__ uint32_t weight_pair(const uint32_t* wb, const uint32
 //   [18] in_had_down (0 / 128 / 512)  [19] base window codes, gate|up | down << 8 (0 or 1)
 template <int C> struct CodeTag { static constexpr int value = C; };
 typedef const NQ_GLOBAL uint64_t* gp_u64;
-struct Planes { gp_u4 base; gp_u8 res; gp_u32 dw; gp_u8 var; int code; gp_u64 flags; int bcode; };
+struct Planes { gp_u4 base; gp_u8 res; gp_u32 dw; gp_u8 var; gp_u64 flags; int code; int bcode; };
 
 // Base record of a lane: code 0 = one uint4 per record; other codes = the residual plane's sub-array layout at
 // Rec<BK>::BITS bits per record (reference sm120/NQ_RES_V2.md:38-46), at most 128 bits.

@@ -21,6 +21,7 @@ inline int set_error(const char* fmt, ...)
     if (e_ != hipSuccess) return nq::set_error("%s: %s", what, hipGetErrorString(e_)); } while (0)
 
 // arguments of one decode-path layer call (device pointers; see NqMoeArgs in include/nq_moe_hip.h)
+struct RouteWs;                       // runs and picks of one call, written by the routing launch (nq_moe.hip)
 struct MoeArgs
 {
     const void* x; const void* sel; const void* rw; int B, topk;
@@ -36,6 +37,9 @@ struct MoeArgs
     int fuse;                         // both launches belong to this call: for runs whose row has neither a low-rank plane nor the
                                       // 512-wide rotation the down launch's staging does the gate|up finisher (set by launch_moe)
     int ny_gu;                        // k-slices of the gate|up launch (the down launch's fused staging sums that many partials)
+    RouteWs* route;                   // NQ_ROUTE_WS_BYTES of device memory: what the routing launch hands to the projection launches
+    int64_t* mb_table; const int64_t* mb_stage; const int32_t* mb_seq; int32_t* mb_applied; int32_t* mb_applied_host;
+                                      // mailbox applied by the routing launch before it reads the table (mb_table == nullptr: none)
 };
 
 // kernel launchers defined next to their kernels

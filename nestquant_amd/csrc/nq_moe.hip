@@ -113,85 +113,166 @@ __device__ __forceinline__ void out2_store(const MoeArgs& a, size_t i, float v0,
 }
 
 constexpr int MAXTOK = 8;                      // tokens of one run = tokens of one call (the MFMA N dimension holds 16)
-struct RunInfo
+// What the projection launches need to know about run r, written once per call by nq_prep_k (one per projection: the plane
+// addresses differ). A run = one distinct routed expert + the tokens that picked it.
+struct alignas(64) RunHdr
 {
-    Planes P;                     // this launch's projection of the run's expert
+    Planes P;                     // this projection of the run's expert
     const _Float16* signs;        // su_g | sv_g | sv_u | su_d | sv_o | su_u
-    int level, ntok, nruns;
+    const _Float16* lr; const _Float16* lr4;      // low-rank plane of the run's expert (lr == nullptr: none)
+    int level, ntok;
     int had;                      // width of the Hadamard on the down projection's input: 128 or 512
-    const _Float16* lr; const _Float16* lr4; int rg, rd;      // low-rank plane of the run's expert (lr == nullptr: none)
-    float z[MAXTOK][4];           // gate|up finisher: x V_gu^T of the run's tokens
-    int slot[MAXTOK];
-    float pick_w[64];             // routing weight of every pick, 0 for picks that contribute nothing
-    const _Float16* pick_signs[64];
-    const _Float16* pick_lr[64]; const _Float16* pick_lr4[64]; unsigned char pick_rg[64], pick_rd[64], pick_lv[64];
+    int rg, rd;
+    unsigned char slot[MAXTOK];   // pick index (token * topk + k) of the run's tokens
+    __device__ __forceinline__ int slot_of(int j) const       // by shifts: a run-time index into slot[] would put the header into scratch memory
+    {
+        unsigned long long v;
+        __builtin_memcpy(&v, slot, 8);
+        return (int)((v >> (8 * j)) & 0xFFull);
+    }
 };
+struct PickInfo                   // per pick, for the down launch's combine
+{
+    float w[64];                  // routing weight, 0 for picks that contribute nothing
+    const _Float16* signs[64];
+    const _Float16* lr[64]; const _Float16* lr4[64]; unsigned char rg[64], rd[64], lv[64];
+};
+struct RouteWs { int nruns; int pad[15]; PickInfo picks; RunHdr run[2][64]; };
+static_assert(sizeof(RunHdr) == 128, "RunHdr is read as 32 scalar words");
+static_assert(sizeof(RouteWs) <= NQ_ROUTE_WS_BYTES, "NQ_ROUTE_WS_BYTES in include/nq_moe_hip.h is too small");
+
+// ---- mailbox rows: 20 int64 read past every cache (a copy engine may have written them while kernels ran), all in flight
+// together and waited for once (the compiler would wait after each atomic load: twenty round trips)
+__device__ __forceinline__ void ld_sys_row(const int64_t* p, int64_t* f)
+{
+#pragma unroll
+    for (int i = 0; i < TBL_W; ++i) asm volatile("global_load_dwordx2 %0, %1, off offset:%2 sc0 sc1" : "=v"(f[i]) : "v"(p), "n"(8 * i) : "memory");
+#pragma unroll
+    for (int i = 0; i < TBL_W; i += 4) asm volatile("s_waitcnt vmcnt(0)" : "+v"(f[i]), "+v"(f[i + 1]), "+v"(f[i + 2]), "+v"(f[i + 3]) :: "memory");
+}
 
 // ---- routing dedup: picks -> runs (refined experts first, then by first occurrence); slots in pick order ----------------
-// called by one full wavefront; lane s owns pick s (S <= 64). Fills run z. A run takes at most one pick per token: a token
+// One wavefront of nq_prep_k, once per call; lane s owns pick s (S <= 64). A run takes at most one pick per token: a token
 // that names the same expert twice opens a second run of that expert, so a run never has more than B tokens. Every lane
-// requests the table-row fields of its own pick together with the level, so the leader's fields cost no second round trip.
-template <int MODE>
-__device__ __forceinline__ void route(const MoeArgs& a, int z, RunInfo* R, int lane)
+// requests all fields of its own pick's table row together, so the leader's fields cost no second round trip. With a mailbox
+// in the call the lane also reads the expert's seq / applied pair: when they differ, its row is the staged one (read after
+// seq, as the mailbox does), which is what the table holds once the mailbox part of this kernel has written it; nothing
+// writes the table before every routing read is done (see nq_prep_k), so the plain loads of the row cannot be torn.
+__device__ __forceinline__ void route(const MoeArgs& a, RouteWs* W, int lane)
 {
     const int S = a.B * a.topk;
-    int e = -1, lv = 0; bool ok = false;
-    int64_t f_base = 0, f_res = 0, f_dw = 0, f_var = 0, f_code = 0, f_signs = 0, f_had = 0, f_lr = 0, f_lr4 = 0, f_rg = 0, f_rd = 0, f_flags = 0, f_bk = 0;
+    int e = -1, lv = 0; bool ok = false, inrange = false;
+    int64_t f[TBL_W];
+#pragma unroll
+    for (int i = 0; i < TBL_W; ++i) f[i] = 0;
     if (lane < S)
     {
         const long long ee = sel_at(a, lane);
         if (ee >= 0 && ee < a.E)
         {
-            e = (int)ee;
+            e = (int)ee; inrange = true;
             const int64_t* ent = a.table + (size_t)e * TBL_W;
-            constexpr int o = MODE == 0 ? 1 : 5;
-            lv = (int)ent[0];
-            f_base = ent[o]; f_res = ent[o + 1]; f_dw = ent[o + 2]; f_var = ent[MODE == 0 ? 12 : 13]; f_code = ent[10 + MODE]; f_signs = ent[9]; f_had = ent[18];
-            f_lr = ent[14]; f_lr4 = ent[15]; f_rg = ent[16]; f_rd = ent[17]; f_flags = ent[o + 3]; f_bk = ent[19];
+#pragma unroll
+            for (int i = 0; i < TBL_W; ++i) f[i] = ent[i];
+            if (a.mb_table)
+            {
+                const int32_t ap = a.mb_applied[e];
+                const int32_t sq = __hip_atomic_load(a.mb_seq + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                if (sq != ap) ld_sys_row(a.mb_stage + (size_t)e * TBL_W, f);
+            }
+            lv = (int)f[0];
             ok = rw_at(a, lane) != 0.f && lv > 0;
         }
     }
+    if (a.hits && inrange && rw_at(a, lane) != 0.f)
+        __hip_atomic_fetch_add(a.hits + e, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    const int level = a.force_level ? a.force_level : lv;
     // Runs of refined experts (level 3, 4: twice the decode work per chunk) are numbered before the level-2 ones, each group
     // by first occurrence: workgroups are dispatched in run order, so the long ones start first and spread over all CUs, and
     // the short ones fill in around them (gate|up 44.0 -> 42.6 us, down 28.4 -> 27.2 us on the benchmark's level mix).
     const unsigned long long okm = __ballot(ok);
-    const unsigned long long heavy = __ballot(ok && (a.force_level ? a.force_level : lv) > 2);
+    const unsigned long long heavy = __ballot(ok && level > 2);
     const unsigned long long below = (1ull << lane) - 1ull;
     const int tok = lane / a.topk, sh = tok * a.topk;
     const unsigned long long mytok = sh < 64 ? (a.topk >= 64 ? ~0ull : ((1ull << a.topk) - 1ull)) << sh : 0ull;
     int r = 0;
     for (int pass = 0; pass < 2; ++pass)
     {
-    unsigned long long rem = pass == 0 ? heavy : okm & ~heavy;
-    while (rem)
-    {
-        const int leader = __ffsll((long long)rem) - 1;
-        const int ev = __shfl(e, leader);
-        const unsigned long long same = __ballot(((rem >> lane) & 1ull) && e == ev);
-        const unsigned long long m = __ballot(((same >> lane) & 1ull) && (same & mytok & below) == 0ull);   // first pick per token
-        if (r == z && ((m >> lane) & 1ull))
+        unsigned long long rem = pass == 0 ? heavy : okm & ~heavy;
+        while (rem)
         {
-            const int pos = __popcll(m & below);
-            R->slot[pos] = lane;
-            if (pos == 0)
+            const int leader = __ffsll((long long)rem) - 1;
+            const int ev = __shfl(e, leader);
+            const unsigned long long same = __ballot(((rem >> lane) & 1ull) && e == ev);
+            const unsigned long long m = __ballot(((same >> lane) & 1ull) && (same & mytok & below) == 0ull);   // first pick per token
+            if ((m >> lane) & 1ull)
             {
-                Planes P;
-                P.base = (gp_u4)f_base; P.res = (gp_u8)f_res; P.dw = (gp_u32)f_dw; P.var = (gp_u8)f_var; P.code = (int)f_code; P.flags = (gp_u64)f_flags;
-                P.bcode = (int)((f_bk >> (8 * MODE)) & 0xFF);
-                R->P = P; R->signs = (const _Float16*)f_signs;
-                R->level = a.force_level ? a.force_level : lv;
-                R->had = f_had == 512 ? 512 : 128;
-                R->lr = (const _Float16*)f_lr; R->lr4 = (const _Float16*)f_lr4; R->rg = (int)f_rg; R->rd = (int)f_rd;
-                R->ntok = __popcll(m);
+                const int pos = __popcll(m & below);
+                W->run[0][r].slot[pos] = (unsigned char)lane; W->run[1][r].slot[pos] = (unsigned char)lane;
+                if (pos == 0)
+                {
+#pragma unroll
+                    for (int mode = 0; mode < 2; ++mode)
+                    {
+                        RunHdr& R = W->run[mode][r];
+                        const int o = mode == 0 ? 1 : 5;
+                        R.P.base = (gp_u4)f[o]; R.P.res = (gp_u8)f[o + 1]; R.P.dw = (gp_u32)f[o + 2]; R.P.flags = (gp_u64)f[o + 3];
+                        R.P.var = (gp_u8)f[12 + mode]; R.P.code = (int)f[10 + mode]; R.P.bcode = (int)((f[19] >> (8 * mode)) & 0xFF);
+                        R.signs = (const _Float16*)f[9];
+                        R.level = level;
+                        R.had = f[18] == 512 ? 512 : 128;
+                        R.lr = (const _Float16*)f[14]; R.lr4 = (const _Float16*)f[15]; R.rg = (int)f[16]; R.rd = (int)f[17];
+                        R.ntok = __popcll(m);
+                    }
+                }
             }
+            rem &= ~m; ++r;
         }
-        rem &= ~m; ++r;
     }
+    PickInfo& K = W->picks;
+    K.w[lane] = ok ? rw_at(a, lane) : 0.f; K.signs[lane] = (const _Float16*)f[9];
+    K.lr[lane] = (const _Float16*)f[14]; K.lr4[lane] = (const _Float16*)f[15];
+    K.rg[lane] = (unsigned char)f[16]; K.rd[lane] = (unsigned char)f[17]; K.lv[lane] = (unsigned char)level;
+    if (lane == 0) W->nruns = r;
+}
+
+// First launch of every layer call, one workgroup of five wavefronts: wavefront 0 does the routing, once for both projection
+// launches (which then read one RunHdr each instead of repeating the dependent loads sel -> table row in every one of their
+// ~1800 workgroups) and the hits export; wavefronts 1..4 are the mailbox, when the caller hands its buffers over with the call
+// (table[e] <- stage[e] where seq[e] != applied[e], then applied[e] <- seq[e], as nq_mailbox_k). Both read at the same time,
+// so the call's chain of memory round trips is sel -> row (+ the staged row of an expert whose update is pending); the
+// mailbox writes the table only after the barrier that the routing wavefront reaches when all its reads are done.
+__global__ void __launch_bounds__(320) nq_prep_k(MoeArgs a)
+{
+    const int t = (int)threadIdx.x - 64;
+    int64_t row[TBL_W];
+    int32_t sq = 0; bool pend = false;
+    if (t < 0) route(a, a.route, threadIdx.x);
+    else if (a.mb_table && t < a.E)
+    {
+        const int32_t ap = a.mb_applied[t];
+        sq = __hip_atomic_load(a.mb_seq + t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        pend = sq != ap;
+        if (pend) ld_sys_row(a.mb_stage + (size_t)t * TBL_W, row);
     }
-    R->pick_w[lane] = ok ? rw_at(a, lane) : 0.f; R->pick_signs[lane] = (const _Float16*)f_signs;
-    R->pick_lr[lane] = (const _Float16*)f_lr; R->pick_lr4[lane] = (const _Float16*)f_lr4;
-    R->pick_rg[lane] = (unsigned char)f_rg; R->pick_rd[lane] = (unsigned char)f_rd; R->pick_lv[lane] = (unsigned char)(a.force_level ? a.force_level : lv);
-    if (lane == 0) R->nruns = r;
+    if (!a.mb_table) return;                                     // block-uniform
+    __syncthreads();
+    if (t < 0) return;
+    for (int e = t; e < a.E; e += 256)
+    {
+        if (e != t)
+        {
+            sq = __hip_atomic_load(a.mb_seq + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            pend = sq != a.mb_applied[e];
+            if (pend) ld_sys_row(a.mb_stage + (size_t)e * TBL_W, row);
+        }
+        if (!pend) continue;
+#pragma unroll
+        for (int i = 0; i < TBL_W; ++i) a.mb_table[(size_t)e * TBL_W + i] = row[i];
+        __threadfence();
+        a.mb_applied[e] = sq;
+        if (a.mb_applied_host) __hip_atomic_store(a.mb_applied_host + e, sq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
 }
 
 // finisher of gate|up for (run z, 128-column group grp): h[slot] = fp16(WHT(silu(g) * u * su_d)), g = WHT(sum_y part_g) * sv_g.
@@ -199,7 +280,7 @@ __device__ __forceinline__ void route(const MoeArgs& a, int z, RunInfo* R, int l
 // WHT_512 = H_4 (x) WHT_128 / 2) the group's WHT_128 result goes, in fp32, into the gate columns of k-slice 0 that this
 // finisher has just consumed, and the last of the four groups of a 512-column block combines them with the Sylvester H_4
 // and rounds to fp16 once.
-__device__ __forceinline__ void finish_gu(const MoeArgs& a, RunInfo& R, int z, int grp, int NY, int warp, int SB, int lane, int& last)
+__device__ __forceinline__ void finish_gu(const MoeArgs& a, const RunHdr& R, float (*zl)[4], int z, int grp, int NY, int warp, int SB, int lane, int& last)
 {
     const _Float16 *sv_g = R.signs + a.H, *sv_u = sv_g + a.I, *su_d = sv_u + a.I;
     const int S = a.B * a.topk, col = grp * 128 + 2 * lane;
@@ -212,7 +293,7 @@ __device__ __forceinline__ void finish_gu(const MoeArgs& a, RunInfo& R, int z, i
     {
         for (int j = warp; j < R.ntok; j += SB)
         {
-            const int tok = R.slot[j] / a.topk;
+            const int tok = R.slot_of(j) / a.topk;
             float zz[4] = {0.f, 0.f, 0.f, 0.f};
             for (int k = 2 * lane; k < a.H; k += 128)
             {
@@ -226,7 +307,7 @@ __device__ __forceinline__ void finish_gu(const MoeArgs& a, RunInfo& R, int z, i
             {
 #pragma unroll
                 for (int m = 32; m >= 1; m >>= 1) zz[r] += __shfl_xor(zz[r], m);
-                if (lane == 0) R.z[j][r] = zz[r];
+                if (lane == 0) zl[j][r] = zz[r];
             }
         }
         __syncthreads();
@@ -235,7 +316,7 @@ __device__ __forceinline__ void finish_gu(const MoeArgs& a, RunInfo& R, int z, i
     const _Float16* U4g = R.lr4, *U4u = U4g + (size_t)rg * a.I;
     for (int j = warp; j < R.ntok; j += SB)
     {
-        const int s = R.slot[j];
+        const int s = R.slot_of(j);
         const float* p = a.part_gu + (size_t)s * 2 * a.I + col;
         const half2_t svg = *(const half2_t*)(sv_g + col), svu = *(const half2_t*)(sv_u + col), sud = *(const half2_t*)(su_d + col);
         const float* const rows2[2] = {p, p + a.I};
@@ -248,7 +329,7 @@ __device__ __forceinline__ void finish_gu(const MoeArgs& a, RunInfo& R, int z, i
         for (int r = 0; r < 4; ++r)
             if (r < rg)
             {
-                const float zr = R.z[j][r];
+                const float zr = zl[j][r];
                 half2_t ug = *(const half2_t*)(U2g + (size_t)r * a.I + col), uu = *(const half2_t*)(U2u + (size_t)r * a.I + col);
                 g0 += zr * (float)ug.x; g1 += zr * (float)ug.y; u0 += zr * (float)uu.x; u1 += zr * (float)uu.y;
                 if (R.level == 4)
@@ -293,7 +374,7 @@ __device__ __forceinline__ void finish_gu(const MoeArgs& a, RunInfo& R, int z, i
     const int c0 = (grp / 4) * 512 + 2 * lane;
     for (int j = warp; j < R.ntok; j += SB)
     {
-        const int s = R.slot[j];
+        const int s = R.slot_of(j);
         float2 w[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) w[q] = ld_dev2_issue(a.part_gu + (size_t)s * 2 * a.I + c0 + q * 128);
@@ -317,7 +398,7 @@ __device__ __forceinline__ void finish_gu(const MoeArgs& a, RunInfo& R, int z, i
 
 // combine of the down projection for output rows [grp * 128, +128): out[b] = sum_k rw[b,k] * sv_o[e] (.) WHT(sum_y part_d[slot])
 // picks of a token are spread over the block's wavefronts and reduced through LDS (red: SB * 128 floats)
-__device__ __forceinline__ void finish_dn(const MoeArgs& a, const RunInfo& R, int grp, int NY, int warp, int SB, int lane, float* red)
+__device__ __forceinline__ void finish_dn(const MoeArgs& a, const PickInfo& R, int grp, int NY, int warp, int SB, int lane, float* red)
 {
     const int S = a.B * a.topk, col = grp * 128 + 2 * lane;
     for (int b = 0; b < a.B; ++b)
@@ -333,9 +414,9 @@ __device__ __forceinline__ void finish_dn(const MoeArgs& a, const RunInfo& R, in
             for (int q = 0; q < 2; ++q)
             {
                 const int kq = k + q * SB, s = b * a.topk + kq;
-                if (kq >= a.topk || R.pick_w[s] == 0.f) continue;     // what route() saw: no second look at the table
-                w[q] = R.pick_w[s]; rows2[q] = a.part_d + (size_t)s * a.H + col;
-                sv[q] = *(const half2_t*)(R.pick_signs[s] + a.H + 3 * a.I + col);
+                if (kq >= a.topk || R.w[s] == 0.f) continue;     // what route() saw: no second look at the table
+                w[q] = R.w[s]; rows2[q] = a.part_d + (size_t)s * a.H + col;
+                sv[q] = *(const half2_t*)(R.signs[s] + a.H + 3 * a.I + col);
             }
             if (w[0] == 0.f && w[1] == 0.f) continue;
             sum_partials<2>(rows2, (size_t)S * a.H, NY, pv);
@@ -346,12 +427,12 @@ __device__ __forceinline__ void finish_dn(const MoeArgs& a, const RunInfo& R, in
                 wht128(v0, v1, lane);
                 if (w[q] == 0.f) continue;
                 v0 *= (float)sv[q].x; v1 *= (float)sv[q].y;
-                const int s = b * a.topk + k + q * SB, prd = R.pick_lr[s] ? R.pick_rd[s] : 0;
+                const int s = b * a.topk + k + q * SB, prd = R.lr[s] ? R.rd[s] : 0;
                 if (prd)
                 {   // y += (sw V_dn^T) (U2_d [+ U4_d]): z_d summed over the I / 128 groups written by the gate|up finishers
-                    const int prg = R.pick_rg[s];
-                    const _Float16* U2d = R.pick_lr[s] + (size_t)prg * (a.H + 2 * a.I) + (size_t)prd * a.I;
-                    const _Float16* U4d = R.pick_lr4[s] + (size_t)prg * 2 * a.I;
+                    const int prg = R.rg[s];
+                    const _Float16* U2d = R.lr[s] + (size_t)prg * (a.H + 2 * a.I) + (size_t)prd * a.I;
+                    const _Float16* U4d = R.lr4[s] + (size_t)prg * 2 * a.I;
 #pragma unroll
                     for (int r = 0; r < 4; ++r)
                         if (r < prd)
@@ -360,7 +441,7 @@ __device__ __forceinline__ void finish_dn(const MoeArgs& a, const RunInfo& R, in
                             for (int gq = 0; gq < a.I / 128; ++gq) zr += a.zd[((size_t)s * (a.I / 128) + gq) * 4 + r];
                             half2_t ud = *(const half2_t*)(U2d + (size_t)r * a.H + col);
                             v0 += zr * (float)ud.x; v1 += zr * (float)ud.y;
-                            if (R.pick_lv[s] == 4) { ud = *(const half2_t*)(U4d + (size_t)r * a.H + col); v0 += zr * (float)ud.x; v1 += zr * (float)ud.y; }
+                            if (R.lv[s] == 4) { ud = *(const half2_t*)(U4d + (size_t)r * a.H + col); v0 += zr * (float)ud.x; v1 += zr * (float)ud.y; }
                         }
                 }
                 o0 += w[q] * v0; o1 += w[q] * v1;
@@ -378,12 +459,6 @@ __device__ __forceinline__ void finish_dn(const MoeArgs& a, const RunInfo& R, in
     }
 }
 
-__device__ __forceinline__ uint64_t uni(uint64_t v)
-{
-    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
-    return (uint64_t)hi << 32 | lo;
-}
-
 // MODE 0: gate|up (N = 2I, K = H, input x rotated here). MODE 1: down (N = H, K = I, input h).
 // grid (N / 32 / SB, C / NC, S); block 64 * SB threads (SB = 1, 2 or 4: a block covers at most one 128-row group);
 // dynamic LDS = rows * (NC * 256 + 16) + 256 bytes (>= SB * 512 for the combine), one row per token of the call
@@ -397,19 +472,20 @@ template <int MODE, bool ANYROW>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) nq_gemv_k(MoeArgs a, int NC)
 {
     extern __shared__ __align__(16) char smem[];
-    __builtin_amdgcn_s_setprio(3);                               // routing and staging are chains of latencies (see progress_priority)
-    __shared__ RunInfo R;
+    __builtin_amdgcn_s_setprio(3);                               // the head is a chain of latencies (see progress_priority)
+    __shared__ float zl[MAXTOK][4];                              // gate|up finisher: x V_gu^T of the run's tokens (low-rank plane)
     __shared__ int last;
     const int lane = threadIdx.x & 63, warp = threadIdx.x >> 6, SB = blockDim.x >> 6;
-    if (warp == 0) route<MODE>(a, blockIdx.z, &R, lane);
-    if (MODE == 0 && a.hits && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x < a.B * a.topk)
+    // the run's header, written by nq_prep_k: block-uniform, read through the scalar cache (constant address space)
+    typedef const __attribute__((address_space(4))) RouteWs* cws_t;
+    const cws_t W = (cws_t)a.route;
+    struct RawHdr { uint32_t w[sizeof(RunHdr) / 4]; } raw;       // requested together with nruns: one round trip, not two
     {
-        const long long ee = sel_at(a, threadIdx.x);
-        if (rw_at(a, threadIdx.x) != 0.f && ee >= 0 && ee < a.E)
-            __hip_atomic_fetch_add(a.hits + ee, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        const __attribute__((address_space(4))) uint32_t* src = (const __attribute__((address_space(4))) uint32_t*)&a.route->run[MODE][blockIdx.z];
+#pragma unroll
+        for (int i = 0; i < (int)(sizeof(RunHdr) / 4); ++i) raw.w[i] = src[i];
     }
-    __syncthreads();
-    const int nruns = R.nruns;
+    const int nruns = W->nruns;
     const int N = MODE == 0 ? 2 * a.I : a.H, K = MODE == 0 ? a.H : a.I, C = K / 128, NY = C / NC;
     if (MODE == 1 && nruns == 0 && blockIdx.z == 0 && blockIdx.y == 0)
     {   // no active pick at all: nobody will arrive last, so the first plane of blocks writes the zero output
@@ -417,18 +493,16 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
             out2_store(a, (size_t)(i / (SB * 16)) * a.H + blockIdx.x * SB * 32 + 2 * (i % (SB * 16)), 0.f, 0.f);
     }
     if ((int)blockIdx.z >= nruns) return;                        // block-uniform
+    const RunHdr R = __builtin_bit_cast(RunHdr, raw);
     const int ntok = R.ntok, chunk0 = blockIdx.y * NC, k0 = chunk0 * 128;
     const int rowstride = NC * 256 + 16;                         // bytes per staged token (+16: spread tokens over banks)
     char* zero = smem + ntok * rowstride;                        // 256 zero bytes after the token rows
-    const _Float16* signs = (const _Float16*)uni((uint64_t)R.signs);
+    const _Float16* signs = R.signs;
 
     // ---- lane context; the first base record is requested now so that its latency overlaps the staging below
     const int t4 = lane >> 4, ss = (lane >> 3) & 1, g = lane & 7, n = lane & 15;
     const int strip = 2 * (blockIdx.x * SB + warp) + ss;
-    Planes P;                                                    // block-uniform: keep the plane addresses in scalar registers
-    P.base = (gp_u4)uni((uint64_t)R.P.base); P.res = (gp_u8)uni((uint64_t)R.P.res); P.dw = (gp_u32)uni((uint64_t)R.P.dw);
-    P.var = (gp_u8)uni((uint64_t)R.P.var); P.code = __builtin_amdgcn_readfirstlane(R.P.code); P.flags = (gp_u64)uni((uint64_t)R.P.flags);
-    P.bcode = __builtin_amdgcn_readfirstlane(R.P.bcode);
+    const Planes P = R.P;                                        // block-uniform: the plane addresses stay in scalar registers
     LaneCtx L;
     L.unit0 = (size_t)strip * C + chunk0; L.rec0 = L.unit0 * 32 + 4 * g + t4;
     L.nrec = (size_t)(N / 16) * C * 32;
@@ -458,7 +532,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
             {
                 const int task = t0 + u * SB < ntask ? t0 + u * SB : t0;
                 const int j = task / NC, c = task - j * NC, kk = k0 + c * 128 + 2 * lane;
-                const int tok = R.slot[j] / a.topk;
+                const int tok = R.slot_of(j) / a.topk;
                 xv[u] = x2_at(a, (size_t)tok * a.H + kk); sv[u] = *(const half2_t*)(su + kk);
                 dsto[u] = j * rowstride + c * 256;
             }
@@ -485,7 +559,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
         for (int task = warp; task < ntok * NC; task += SB)
         {
             const int j = task / NC, c = task - j * NC, col = k0 + c * 128 + 2 * lane;
-            const float* p = a.part_gu + (size_t)R.slot[j] * 2 * a.I + col;
+            const float* p = a.part_gu + (size_t)R.slot_of(j) * 2 * a.I + col;
             const float* const rows2[2] = {p, p + a.I};
             const half2_t svg = *(const half2_t*)(sv_g + col), svu = *(const half2_t*)(sv_u + col), sud = *(const half2_t*)(su_d + col);
             float2 pq[2];
@@ -502,7 +576,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
             if (blockIdx.x == 0)                                 // h stays inspectable, as the gate|up finisher leaves it
             {
                 half2_t hv; hv.x = (_Float16)v0; hv.y = (_Float16)v1;
-                *(half2_t*)(a.h + (size_t)R.slot[j] * a.I + col) = hv;
+                *(half2_t*)(a.h + (size_t)R.slot_of(j) * a.I + col) = hv;
             }
         }
     }
@@ -511,7 +585,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
         for (int i = threadIdx.x; i < ntok * NC * 64; i += blockDim.x)
         {
             const int j = i / (NC * 64), r = i % (NC * 64), c = r >> 6, p = r & 63;
-            const half2_t hv = *(const half2_t*)(a.h + (size_t)R.slot[j] * a.I + k0 + c * 128 + 2 * p);
+            const half2_t hv = *(const half2_t*)(a.h + (size_t)R.slot_of(j) * a.I + k0 + c * 128 + 2 * p);
             _Float16* dst = (_Float16*)(smem + j * rowstride + c * 256);
             dst[bop_index(2 * p)] = hv.x; dst[bop_index(2 * p + 1)] = hv.y;
         }
@@ -541,7 +615,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
     if (n < ntok)
     {
         const int S = a.B * a.topk;
-        float* part = (MODE == 0 ? a.part_gu : a.part_d) + ((size_t)blockIdx.y * S + R.slot[n]) * N;
+        float* part = (MODE == 0 ? a.part_gu : a.part_d) + ((size_t)blockIdx.y * S + R.slot_of(n)) * N;
         const int row = 16 * (2 * (blockIdx.x * SB + warp) + (t4 >> 1)) + 4 * (t4 & 1);
         st_dev4(part + row, acc[0]);
         st_dev4(part + row + 8, acc[1]);
@@ -561,8 +635,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
         last = __hip_atomic_fetch_add(cnt, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == expect - 1;
     __syncthreads();
     if (!last) return;                                           // block-uniform
-    if constexpr (MODE == 0) finish_gu(a, R, blockIdx.z, grp, NY, warp, SB, lane, last);
-    else finish_dn(a, R, grp, NY, warp, SB, lane, (float*)smem);
+    if constexpr (MODE == 0) finish_gu(a, R, zl, blockIdx.z, grp, NY, warp, SB, lane, last);
+    else finish_dn(a, a.route->picks, grp, NY, warp, SB, lane, (float*)smem);
     if (threadIdx.x == 0) __hip_atomic_store(cnt, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
@@ -584,6 +658,8 @@ __global__ void nq_mailbox_k(int64_t* table, const int64_t* stage, const int32_t
 int launch_moe(const MoeArgs& a, const int* cfg_gu, const int* cfg_dn, int which, hipStream_t st)
 {
     const int S = a.B * a.topk;
+    nq_prep_k<<<1, 320, 0, st>>>(a);
+    NQ_LAUNCH_CHECK("moe_forward (routing)");
     for (int mode = 0; mode < 2; ++mode)
     {
         if (!((which >> mode) & 1)) continue;
@@ -648,13 +724,14 @@ int launch_moe_static(MoeArgs a, const int* cfg_gu, const int* cfg_dn, int which
     auto take = [&](size_t bytes) { const size_t o = off; off += (bytes + 255) & ~(size_t)255; return o; };
     const size_t o_cnt = take((2 * S * G128 + (size_t)a.H / 128) * sizeof(int));       // cnt_gu | cnt_h | cnt_d: cleared below
     const size_t o_gu = take(ny_gu * S * 2 * a.I * sizeof(float)), o_d = take(ny_dn * S * a.H * sizeof(float));
-    const size_t o_h = take(S * a.I * sizeof(_Float16)), o_zd = take(S * G128 * 4 * sizeof(float));
+    const size_t o_h = take(S * a.I * sizeof(_Float16)), o_zd = take(S * G128 * 4 * sizeof(float)), o_route = take(sizeof(RouteWs));
     if (off > STATIC_SCRATCH_BYTES)
         return set_error("nq_moe_forward_static: this call needs %zu bytes of workspace (B=%d topk=%d H=%d I=%d, %zu and %zu k-slices), the built-in "
                          "scratch holds %zu: use coarser k-slices, or nq_moe_forward with workspaces of the caller's", off, a.B, a.topk, a.H, a.I, ny_gu, ny_dn,
                          STATIC_SCRATCH_BYTES);
     a.cnt_gu = (int*)(base + o_cnt); a.cnt_h = a.cnt_gu + S * G128; a.cnt_d = a.cnt_h + S * G128;
     a.part_gu = (float*)(base + o_gu); a.part_d = (float*)(base + o_d); a.h = (_Float16*)(base + o_h); a.zd = (float*)(base + o_zd);
+    a.route = (RouteWs*)(base + o_route);
     // the counters must be zero on entry; a fill kernel, not hipMemsetAsync, so that the call can be recorded into a graph
     const int ncnt = (int)(2 * S * G128 + (size_t)a.H / 128);
     nq_clear_k<<<(ncnt + 255) / 256, 256, 0, st>>>(a.cnt_gu, ncnt);

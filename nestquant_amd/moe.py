@@ -145,6 +145,7 @@ class MoELayer:
         s.wq = torch.zeros(4, dtype=i32, device=dev)
         s.zd = torch.zeros(S * (I // 128) * 4, dtype=f32, device=dev); s.cnt_h = torch.zeros(S * (I // 128), dtype=i32, device=dev)
         s.out = torch.zeros(Bmax, H, dtype=f32, device=dev)
+        s.route = torch.zeros(_lib.ROUTE_WS_BYTES, dtype=torch.uint8, device=dev)    # the routing launch's result for the projection launches
         s.hits_ptr = 0
         s.rare_rows = False                           # set once a row in mask mode or with a base window code other than 0 is
                                                       # installed (set / Mailbox.post): the decode call then runs the kernel that
@@ -200,12 +201,14 @@ class MoELayer:
         s.rare_rows |= bool(row[4] or row[8] or row[19])
         s.table[e].copy_(row.to(s.table.device), non_blocking=False)
 
-    def __call__(s, x, sel, rw, out=None, force_level=0, which=3, cfg_gu=None, cfg_dn=None, table=None, static_ws=False):
+    def __call__(s, x, sel, rw, out=None, force_level=0, which=3, cfg_gu=None, cfg_dn=None, table=None, static_ws=False, mailbox=None):
         """x [B, H], sel [B, topk], rw [B, topk] -> fp32 [B, H] (s.out[:B] unless `out` is given). As in the reference x
         and rw are fp16 and sel int64; the kernels also take x / rw in bf16 or fp32, sel in int32 and `out` in fp16 or
         bf16, with the roundings of x.half(), rw.half() and out.to(dtype) (the casts the reference's caller launches as
         separate kernels, sm120/serve/nq_vllm.py:522,560).
         table: optional [E, TBL_W] override. Everything is enqueued on torch's current stream; nothing syncs.
+        mailbox: a Mailbox of this layer to apply at the head of the call (same effect as mailbox.apply() right before it,
+        one launch less: the call's routing launch does it before it reads the table).
         static_ws: go through nq_moe_forward_static, which ignores this layer's workspaces and uses the library's built-in
         device scratch instead (for callers that must not allocate; calls on one GPU then share that scratch)."""
         assert x.dtype in _DT_IN and rw.dtype in _DT_IN and sel.dtype in _DT_SEL, (x.dtype, rw.dtype, sel.dtype)
@@ -230,6 +233,10 @@ class MoELayer:
         a.cnt_h, a.cnt_h_elems = s.cnt_h.data_ptr(), s.cnt_h.numel()
         a.zd, a.zd_elems = s.zd.data_ptr(), s.zd.numel()
         a.G = s.G
+        a.route_ws, a.route_ws_bytes = s.route.data_ptr(), s.route.numel()
+        if mailbox is not None:
+            a.mb_table, a.mb_stage, a.mb_seq = tb.data_ptr(), mailbox.stage.data_ptr(), mailbox.seq.data_ptr()
+            a.mb_applied, a.mb_applied_host = mailbox.applied.data_ptr(), mailbox.applied_host.data_ptr()
         a.common_rows = int(table is None and not s.rare_rows)     # a caller's own table: unknown
         a.x_dtype, a.sel_dtype, a.rw_dtype, a.out_dtype = _DT_IN[x.dtype], _DT_SEL[sel.dtype], _DT_IN[rw.dtype], _DT_OUT[out.dtype]
         _lib.check((s.M.nq_moe_forward_static if static_ws else s.M.nq_moe_forward)(C.byref(a), _lib.stream_ptr()))
@@ -410,13 +417,15 @@ def forward(layer, mailbox, x, topk_weights, topk_ids, pf_min=PF_MIN, sal=None):
     a step of up to 16 tokens; longer steps count as prefill and are left out)."""
     T = x.shape[0]
     x, w, ids = x.contiguous(), topk_weights.contiguous(), topk_ids.contiguous()
+    odt = x.dtype if x.dtype in _DT_OUT else torch.float32
+    if 0 < T <= layer.Bmax:
+        if sal is not None:
+            sal(x, w, ids)
+        return layer(x, ids, w, out=torch.empty(T, layer.H, dtype=odt, device=x.device), mailbox=mailbox)   # applied by the call's first launch
     if mailbox is not None:
         mailbox.apply()
-    odt = x.dtype if x.dtype in _DT_OUT else torch.float32
-    if T <= layer.Bmax:
-        if sal is not None and T:
-            sal(x, w, ids)
-        return layer(x, ids, w, out=torch.empty(T, layer.H, dtype=odt, device=x.device))
+    if T == 0:
+        return torch.empty(0, layer.H, dtype=odt, device=x.device)
     if T >= pf_min and not torch.cuda.is_current_stream_capturing():
         return layer.prefill(x.half(), ids.long(), w.half()).to(x.dtype)
     out = torch.empty(T, layer.H, dtype=odt, device=x.device)

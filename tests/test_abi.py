@@ -31,7 +31,7 @@ def test_every_declared_symbol_is_exported_and_bound():
         assert hasattr(L, n), n
         assert n in _lib.SIGNATURES, f"{n} has no ctypes signature"
     assert sorted(_lib.SIGNATURES) == names
-    assert L.nq_abi_version() == 1
+    assert L.nq_abi_version() == 2
 
 
 def _row(**kw):
@@ -83,7 +83,7 @@ def test_argument_checks_run_before_any_device_work():
     err = lambda: L.nq_last_error().decode()
     buf = (C.c_char * 4096)()
     base = C.addressof(buf)
-    base += (-base) % 16                                           # a 16-byte aligned address inside the buffer
+    base += (-base) % 64                                           # a 64-byte aligned address inside the buffer
     a = _lib.NqMoeArgs()
     for f in ("x", "sel", "rw", "table", "out", "acc_gu", "h", "acc_d", "cnt_gu", "cnt_d", "cnt_h", "zd"):
         setattr(a, f, base)
@@ -98,8 +98,14 @@ def test_argument_checks_run_before_any_device_work():
     a.B = 1; a.cfg_gu = (C.c_int32 * 4)(1, 3, 12, 0)
     assert L.nq_moe_forward(C.byref(a), None) != 0 and "bad cfg" in err()
     a.cfg_gu = (C.c_int32 * 4)(1, 4, 12, 0); a.G = 3
+    a.route_ws = base
     a.acc_gu_elems = a.acc_d_elems = a.h_elems = a.out_elems = a.cnt_gu_elems = a.cnt_d_elems = a.cnt_h_elems = a.zd_elems = 1 << 40
+    assert L.nq_moe_forward(C.byref(a), None) != 0 and "route_ws" in err()
+    a.route_ws_bytes = _lib.ROUTE_WS_BYTES
     assert L.nq_moe_forward(C.byref(a), None) != 0 and "G=3" in err()
+    a.G = 4; a.mb_table = base
+    assert L.nq_moe_forward(C.byref(a), None) != 0 and "mailbox needs" in err()
+    a.mb_table = None; a.G = 3
     a.G = 0; a.common_rows = 2
     assert L.nq_moe_forward(C.byref(a), None) != 0 and "common_rows" in err()
     assert L.nq_pf_plan(base, 256, 0, 1024, base, 256, None) != 0 and "cap" in err()

@@ -225,6 +225,40 @@ def test_mailbox_kernel_matches_state_machine():
     assert MB.applied_host.numpy()[[1, 4]].tolist() == [1, 5]
 
 
+def test_mailbox_applied_by_the_layer_call_equals_apply_then_call():
+    """L(..., mailbox=MB) = MB.apply() followed by L(...): same table, same applied / applied_host, same output bits; rows posted
+    between calls (level changes of routed experts, 260 experts so that one thread handles two rows) take effect in that call"""
+    H, I, NE = 256, 256, 260
+    ex = to_dev(experts_on_gpu(H, I, 6, 11, nested_ids=range(6)))
+    side = torch.cuda.Stream()
+    res = []
+    for fused in (False, True):
+        L = M.MoELayer(NE, H, I, Bmax=2, topk=4)
+        MB = M.Mailbox(L)
+        for e in range(NE):
+            L.set(e, ex[e % 6], 2)
+        g = torch.Generator().manual_seed(3)
+        x = (torch.randn(2, H, generator=g) * 0.05).half().to(DEV)
+        sel = torch.tensor([[0, 257, 2, 3], [3, 4, 259, 0]], device=DEV); rw = torch.full((2, 4), 0.25, device=DEV).half()
+        outs = []
+        for step, (e, lv) in enumerate([(257, 4), (3, 3), (259, 0), (0, 4), (257, 2)]):
+            MB.post(e, M.entry(ex[e % 6], lv), side)
+            side.synchronize()
+            if fused:
+                y = L(x, sel, rw, mailbox=MB)
+            else:
+                MB.apply(); y = L(x, sel, rw)
+            torch.cuda.synchronize()
+            assert MB.done(e), (fused, step)
+            outs.append(y.clone())
+        res.append((outs, L.table.clone(), MB.applied.clone(), MB.applied_host.clone()))
+        assert len({o.cpu().numpy().tobytes() for o in outs}) == 5          # every posted row changed the result
+    for a, b in zip(res[0][0], res[1][0]):
+        assert torch.equal(a, b)
+    assert torch.equal(res[0][2], res[1][2]) and torch.equal(res[0][3], res[1][3])
+    assert torch.equal(res[0][1][:, 0], res[1][1][:, 0])                     # levels (the other words are addresses of equal planes)
+
+
 def test_caller_dtypes_and_forward_dispatch():
     """bf16 / fp32 activations and weights, int32 ids, fp16 / bf16 results: bitwise what the reference's caller gets from
     x.half(), w.half(), ids.long() and out.to(dtype) around an fp16 call; forward() slices 9..383 tokens by Bmax"""
