@@ -83,6 +83,21 @@ def code_bytes(ex, levels, experts, which="all"):
     return tot
 
 
+def c_oracle_dense(ex, e, lv, proj):
+    """dense fp16 [N, K] of projection `proj` of (compacted, nested) expert e at level lv through the C oracle"""
+    from oracle import nq_oracle_c as OC
+    p = (ex[e].gu, ex[e].dn)[proj]
+    nrec = p.z["S"] * p.z["C"] * 32
+    base = (p.base.cpu().numpy().astype(np.int64) & 0xFFFFFFFF).astype(np.uint32).reshape(-1, 4)
+    code, res, dw = 0, None, None
+    if lv >= 3:
+        slot = p.slot.cpu().numpy()
+        code = 10 if lv == 3 else 11
+        res = OC.unpack(slot[: nrec * 2] if lv == 3 else slot, nrec, code, split=(lv == 4))
+        dw = ((p.d3 if lv == 3 else p.d4n).cpu().numpy().astype(np.int64) & 0xFFFFFFFF).astype(np.uint32)
+    return OC.decode_proj(base, p.N, p.K, lv, code, res, dw)
+
+
 def cpu_expert(ex, levels, e, xf):
     """C oracle on expert e (dense decode of both projections, OpenMP on the host cores) + the fp32 layer math:
     -> (y [H] fp32, seconds of decode, seconds of layer math)"""
@@ -113,11 +128,30 @@ def cpu_expert(ex, levels, e, xf):
     return y, t1 - t0, time.perf_counter() - t1
 
 
+def oracle_planes(ex, e):
+    """the planes of (compacted, nested) expert e as the oracle's host-side Plane objects: (gate|up, down, nested)"""
+    from oracle import nq_oracle as O
+    out = []
+    for p in (ex[e].gu, ex[e].dn):
+        nrec = p.z["S"] * p.z["C"] * 32
+        u32 = lambda t: (t.cpu().numpy().astype(np.int64) & 0xFFFFFFFF).astype(np.uint32)
+        slot = p.slot.cpu().numpy()
+        out.append(O.Plane(p.N, p.K, u32(p.base).reshape(-1, 4), p3=O.unpack_words(slot[: nrec * 2], nrec, 64), d3=u32(p.d3),
+                           p4n=O.unpack_words(slot[nrec * 2:], nrec, 64), d4n=u32(p.d4n)))
+    return out[0], out[1], True
+
+
 def cpu_baseline(ex, levels, routes, xs, budget_s=10.0):
-    """the same layer steps on the host through the C oracle: whole steps (every routed expert of the step, at its level, then
-    the top-k combine) until about `budget_s` seconds of CPU work are spent. Only the decode and the layer math are timed,
-    not the copies of the planes from the device. -> (record, y of step 0)"""
-    from oracle import nq_oracle_c as OC
+    """The same layer steps on the host cores, two ways, each on whole steps (every routed expert of the step, at its level, then
+    the top-k combine) until its budget of CPU seconds is spent; only the decode and the layer math are timed, not the copies
+    of the planes from the device:
+      value      the torch-CPU restatement of the reference's own CPU path (vectorised torch decode of each routed expert into
+                 a dense fp16 matrix + fp32 matmuls, reference sm120/moe.py:156-166,196-210,344-351) with
+                 torch.set_num_threads(all cores);
+      c_oracle   the C oracle (dense decode + fp32 matvecs, OpenMP on all cores).
+    -> (record, y of step 0 from the C oracle, y of step 0 from the torch path)"""
+    from oracle import nq_oracle_c as OC, nq_oracle_torch as OT
+    cores = int(os.environ["OMP_NUM_THREADS"]) if os.environ.get("OMP_NUM_THREADS") else os.cpu_count()
     OC.decode_proj(np.zeros((64, 4), np.uint32), 16, 256, 2)    # load the library, start its thread pool
     t_dec = t_math = 0.0
     nbytes = nsteps = 0
@@ -133,10 +167,34 @@ def cpu_baseline(ex, levels, routes, xs, budget_s=10.0):
         if nsteps == 0:
             y0 = y
         nsteps += 1
-    cores = int(os.environ["OMP_NUM_THREADS"]) if os.environ.get("OMP_NUM_THREADS") else os.cpu_count()
-    return dict(value=round(nbytes / (t_dec + t_math) / 1e9, 4), unit="GB/s", cores=cores, kind="port",
-                sample=f"the first {nsteps} of the timed layer steps (B=1, 8 routed experts each at its level, {nbytes / 1e6:.0f} MB of code): "
-                       f"dense decode {t_dec:.2f} s + fp32 layer math {t_math:.2f} s; {1e3 * (t_dec + t_math) / nsteps:.0f} ms per step"), y0
+    c_rec = dict(value=round(nbytes / (t_dec + t_math) / 1e9, 4), unit="GB/s", cores=cores, kind="port",
+                 sample=f"the first {nsteps} of the timed layer steps ({nbytes / 1e6:.0f} MB of code): dense decode {t_dec:.2f} s + "
+                        f"fp32 layer math {t_math:.2f} s; {1e3 * (t_dec + t_math) / nsteps:.0f} ms per step")
+    # torch path: planes converted beforehand (untimed), then moe_ref per step
+    prev = torch.get_num_threads()
+    torch.set_num_threads(cores)
+    tt = 0.0; tbytes = tsteps = 0; yt0 = None
+    try:
+        while tt < budget_s and tsteps < len(routes):
+            ids, w, _ = routes[tsteps]
+            planes = {e: oracle_planes(ex, e) for e in ids[0].tolist()}
+            signs = {e: ex[e].signs.cpu().numpy() for e in planes}
+            x = xs[tsteps].float().cpu().numpy(); sel = ids.cpu().numpy(); rwn = w.cpu().numpy()
+            t0 = time.perf_counter()
+            y = OT.moe_ref(lambda e: planes[e], levels, lambda e: signs[e], x, sel, rwn)
+            tt += time.perf_counter() - t0
+            tbytes += sum(ex[e].bytes(levels[e]) for e in planes)
+            if tsteps == 0:
+                yt0 = y.numpy()[0]
+            tsteps += 1
+    finally:
+        torch.set_num_threads(prev)
+    rec = dict(value=round(tbytes / tt / 1e9, 4), unit="GB/s", cores=cores, kind="port",
+               sample=f"torch-CPU restatement of the reference's CPU path (vectorised decode to dense fp16 + fp32 matmuls, torch.set_num_threads({cores})) "
+                      f"on the first {tsteps} of the timed layer steps (B=1, 8 routed experts each at its level, {tbytes / 1e6:.0f} MB of code): "
+                      f"{1e3 * tt / tsteps:.0f} ms per step",
+               ms_per_step=round(1e3 * tt / tsteps, 1), c_oracle=c_rec)
+    return rec, y0, yt0
 
 
 def zipf_routing(T, dev, seed=11, skew=1.1):
@@ -158,21 +216,73 @@ def prefill_leg(L, ex, dev, T=4096, reps=3):
     sel, rw = zipf_routing(T, dev)
     g = torch.Generator().manual_seed(12)
     x = (torch.randn(T, H, generator=g) * 0.05).half().to(dev)
-    L.prefill(x, sel, rw)
+    y = L.prefill(x, sel, rw)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(reps):
         L.prefill(x, sel, rw)
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / reps
+    # correctness of the full-size call: four tokens (first, last, two inside) against the float64 oracle layer math over the
+    # HIP-decoded dense weights of their routed experts (the decoder itself is proved bit-exact by the tests)
+    from oracle import nq_oracle as O
+    toks = [0, 1337, 2901, T - 1]
+    cache = {}
+
+    def dense(e):
+        if e not in cache:
+            cache[e] = (M.dense_W(ex[e], 0, 4).float().cpu().numpy(), M.dense_W(ex[e], 1, 4).float().cpu().numpy())
+        return cache[e]
+    signs = lambda e: ex[e].signs.cpu().numpy()
+    want = O.moe_forward(dense, [4] * E, signs, x[toks].cpu().numpy(), sel[toks].cpu().numpy(), rw[toks].cpu().numpy(), dtype=np.float64)
+    rel = float(np.linalg.norm(y[toks].cpu().numpy() - want) / np.linalg.norm(want))
+    assert rel < 1e-3, f"prefill output of tokens {toks} is {rel:.2e} from the oracle"
     L.table.copy_(saved)
     flops = T * TOPK * 6 * H * I
     cnt = torch.bincount(sel.flatten().cpu(), minlength=E)
     return dict(workload=f"prefill: T={T} tokens, top-8 over E=256 with Zipf(1.1) popularity, all experts at level 4, "
                          f"rows per expert max {int(cnt.max())} / median {int(cnt.median())}",
                 ms=round(dt * 1e3, 3), tflops=round(flops / dt / 1e12, 1), flop=flops, mfma_peak_tflops=MFMA_PEAK_TFLOPS,
-                mfma_frac=round(flops / dt / 1e12 / MFMA_PEAK_TFLOPS, 4),
+                mfma_frac=round(flops / dt / 1e12 / MFMA_PEAK_TFLOPS, 4), rel_err_vs_oracle=float(f"{rel:.2e}"), checked_tokens=toks,
                 note="whole prefill() call: sort, pre, 2 decode-fused grouped GEMMs, mid, post; bound by the VALU trellis decode")
+
+
+def batch_leg(L, MB, ex, levels, dev, R=32, blocks=8):
+    """config 3 at 1-4 tokens, as the reference tabulates its layer (threads/13-moe-layer-kernel/REPORT.md:62-65: all experts at
+    2 bit, all at 4 bit, mixed): median us per layer step (mailbox + layer call) over event-timed replays of a graph of R steps
+    with seeded routings that avoid the previous step's experts, and the GB/s of code bytes of the distinct routed experts"""
+    saved = L.table.clone()
+    s = torch.cuda.Stream()
+    out = {}
+    for name, lv_of in (("mixed", lambda e: levels[e]), ("all_2bit", lambda e: 2), ("all_4bit", lambda e: 4)):
+        lv = [lv_of(e) for e in range(E)]
+        for e in range(E):
+            L.set(e, ex[e], lv[e])
+        for B in (1, 2, 3, 4):
+            routes = make_routings(B, R, dev)
+            g = torch.Generator().manual_seed(100 + B)
+            xs = [(torch.randn(B, H, generator=g) * 0.05).half().to(dev) for _ in range(R)]
+            with torch.cuda.stream(s):
+                for i in range(R):
+                    L(xs[i], routes[i][0], routes[i][1], mailbox=MB)
+            torch.cuda.synchronize()
+            gr = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gr, stream=s):
+                for i in range(R):
+                    L(xs[i], routes[i][0], routes[i][1], mailbox=MB)
+            ev = []
+            with torch.cuda.stream(s):
+                gr.replay()
+                for _ in range(blocks):
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record(s); gr.replay(); e1.record(s); ev.append((e0, e1))
+            torch.cuda.synchronize()
+            us = sorted(a.elapsed_time(b) * 1e3 / R for a, b in ev)[blocks // 2]
+            nb = sum(code_bytes(ex, lv, r[2]) for r in routes) / R
+            out[f"{name}_B{B}"] = dict(us_per_layer=round(us, 2), GBps=round(nb / us / 1e3, 1), distinct_experts=round(sum(len(r[2]) for r in routes) / R, 1))
+    L.table.copy_(saved)
+    out["reference_A100_us"] = "B1-B4: 2 bit 132.7 / 192.6 / 249.5 / 313.7, 4 bit 220.5 / 320.7 / 412.7 / 516.7 (threads/13-moe-layer-kernel/REPORT.md:62-65)"
+    return out
 
 
 def caller_leg(L, MB, routes, xs, dev, reps=4):
@@ -272,24 +382,40 @@ def churn_leg(L, MB, ex, levels, routes, xs, dev, steps=64, ops_per_step=8, nati
                 e0.record(s); graphs[st % len(graphs)].replay(); e1.record(s)
             e1.synchronize()
             lat.append(e0.elapsed_time(e1) * 1e3)
-            for e in X.poll():
+            got = X.poll()
+            if got:
+                last_landed[:] = got
+            for e in got:
                 lags.append(st - issued.pop(e, st))
         if churn:
             settle()                                             # the H2D rate is over issue -> last copy landed and applied
         wall = time.perf_counter() - t0
         return sorted(lat)[len(lat) // 2], lags, wall
 
+    last_landed = []
     idle_us, _, _ = run(False)
     churn_us, lags, wall = run(True)
     torch.cuda.synchronize()
     settle()                                                     # drain outstanding ops, then check the books
     X.check_invariants()
+    # bit-exactness after the swaps: every expert whose op landed in the last step that landed any, dequantised by the HIP
+    # decoder from its live table row, against the C oracle's decode of its planes at the level the books say
+    nbad = 0
+    for e in last_landed:
+        for proj in (0, 1):
+            W = M.dequant(L.table[e].clone(), proj, H, I).cpu().numpy().view(np.uint16)
+            ref = c_oracle_dense(ex, e, X.level[e], proj).view(np.uint16)
+            nbad += int(((W != ref) & ~(((W | ref) & 0x7FFF) == 0)).sum())
+    assert nbad == 0, f"{nbad} weights of the experts swapped last differ from the oracle"
     res = dict(workload=f"plane churn: {steps} B=1 layer steps, {ops_per_step} promote(2->4)/demote(4->2) ops per step on a side "
                         f"stream, {X.lay.bytes} B per promotion from pinned host memory",
                step_us_idle=round(idle_us, 2), step_us_churn=round(churn_us, 2), ops=X.n_ops - len(lv4), refused=X.n_refused,
                h2d_GBps=round(X.bytes_copied / wall / 1e9, 2), h2d_MB=round(X.bytes_copied / 1e6, 1),
                lag_steps_median=(sorted(lags)[len(lags) // 2] if lags else None), lag_steps_max=(max(lags) if lags else None),
-               invariants="B,T,O,K hold after the run", issued_by="upgrade engine (upload)" if native else "torch copies")
+               invariants="B,T,O,K hold after the run",
+               dequant_after_last_swaps=f"bit-exact ({len(last_landed)} experts x 2 projections at their new levels vs the C oracle)",
+               note=("8 promotions per ~70 us step ask for ~1 TB/s of the ~50 GB/s host link: ops queue (lag) and experts with an op in "
+                     "flight refuse a second one (refused), as the one-op-per-expert rule demands"), issued_by="upgrade engine (upload)" if native else "torch copies")
     X.close()
     L.table.copy_(saved)
     MB.apply(); torch.cuda.synchronize()
@@ -418,6 +544,7 @@ def main():
     ap.add_argument("--no-config2", action="store_true", help="skip the single-projection leg (per-level GB/s at 1 / 4 / 8 tokens)")
     ap.add_argument("--no-stream", action="store_true", help="skip the record upgrade engine leg (file -> pinned -> slot)")
     ap.add_argument("--no-caller", action="store_true", help="skip the caller-dtype leg (bf16 / fp32 / int32 tensors)")
+    ap.add_argument("--no-batches", action="store_true", help="skip the 1-4 token table (mixed levels, all 2 bit, all 4 bit)")
     ap.add_argument("--calib", action="store_true", help="also run one 256 MiB device copy (reads 256 MiB, writes 256 MiB): "
                     "the known-size kernel that scales rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
     a = ap.parse_args()
@@ -505,16 +632,28 @@ def main():
     torch.cuda.synchronize()
     call_blocks = sorted(e0.elapsed_time(e1) * 1e3 / R for e0, e1 in call_blocks)
 
-    # dominant kernel alone: gate|up decode-GEMV (which = 1: the launch with its fused SwiGLU finisher); one graph of R launches, replayed between two events
-    # recorded on the launch stream (eager launches from Python would measure the host, not the kernel)
+    # dominant kernel alone: gate|up decode-GEMV (which = 1: the launch with its SwiGLU finisher); one graph of R launches, replayed
+    # between two events recorded on the launch stream (eager launches from Python would measure the host, not the kernel). Every
+    # routing gets route / xrot workspaces of its own, filled once by the call's first launch (which = 0), so that the timed
+    # launches are the projection kernel and nothing else (which = 1 | 4)
+    ws_main = (L.route, L.xrot)
+    ws = [(torch.zeros_like(L.route), torch.zeros_like(L.xrot)) for _ in range(R)]
+
+    def gu_only(i, which):
+        L.route, L.xrot = ws[i]
+        L(xs[i], routes[i][0], routes[i][1], which=which)
+
     with torch.cuda.stream(s):
         for i in range(R):
-            L(xs[i], routes[i][0], routes[i][1], which=1)
+            gu_only(i, 0)
+        for i in range(R):
+            gu_only(i, 5)
     torch.cuda.synchronize()
     gk = torch.cuda.CUDAGraph()
     with torch.cuda.graph(gk, stream=s):
         for i in range(R):
-            L(xs[i], routes[i][0], routes[i][1], which=1)
+            gu_only(i, 5)
+    L.route, L.xrot = ws_main
     nrep = max(1, (K + R - 1) // R)
     with torch.cuda.stream(s):
         gk.replay()
@@ -529,16 +668,22 @@ def main():
     achieved = kbytes / kdt / 1e9
     roofline = dict(bound="hbm", kernel="nq_gemv_k<0, false> (gate|up decode+GEMV)", achieved=round(achieved, 1), peak=HBM_PEAK_GBS, unit="GB/s",
                     frac=round(achieved / HBM_PEAK_GBS, 4), traffic=int(kbytes * TRAFFIC_RATIO), us_per_launch=round(kdt * 1e6, 2),
-                    algorithmic_bytes_per_launch=int(kbytes))
+                    algorithmic_bytes_per_launch=int(kbytes),
+                    traffic_source=f"algorithmic bytes x {TRAFFIC_RATIO}: rocprofv3 FETCH_SIZE + WRITE_SIZE of this kernel, scaled by a 256 MiB copy "
+                                   "(profiles/decode_gemv_hbm_traffic_pmc.txt), not a counter read in this run",
+                    timed="the gate|up projection launch alone (which = 1 | 4: with its SwiGLU finisher, routing and rotated activations "
+                          "prepared beforehand), 64 routings in one graph, HIP events on the launch stream")
     cpu = None
     if not a.no_cpu:
-        cpu, y0 = cpu_baseline(ex, levels, routes, xs)
-        err = float(np.linalg.norm(eager[0, 0].cpu().numpy() - y0) / np.linalg.norm(y0))
-        assert err < 1e-3, f"GPU layer output of step 0 is {err:.2e} from the CPU oracle's"
-        cpu["gpu_vs_cpu_rel_err_step0"] = float(f"{err:.2e}")
+        cpu, y0, yt0 = cpu_baseline(ex, levels, routes, xs)
+        for name, yy in (("gpu_vs_cpu_rel_err_step0", yt0), ("gpu_vs_c_oracle_rel_err_step0", y0)):
+            err = float(np.linalg.norm(eager[0, 0].cpu().numpy() - yy) / np.linalg.norm(yy))
+            assert err < 1e-3, f"GPU layer output of step 0 is {err:.2e} from the CPU path's ({name})"
+            cpu[name] = float(f"{err:.2e}")
     lv_counts = {lv: levels.count(lv) for lv in (2, 3, 4)}
     prefill = None if a.no_prefill else prefill_leg(L, ex, dev)
     caller = None if a.no_caller else caller_leg(L, MB, routes, xs, dev)
+    batches = None if a.no_batches else batch_leg(L, MB, ex, levels, dev)
     churn = None
     if not a.no_churn:
         churn = churn_leg(L, MB, ex, levels, routes[:16], xs, dev, native=True)
@@ -556,7 +701,7 @@ def main():
         "config": {"workload": f"decode MoE layer: E=256 top-8 B={B}, H=6144 I=2048, levels 2/3/4 = "
                                f"{lv_counts[2]}/{lv_counts[3]}/{lv_counts[4]} experts, seeded softmax routing avoiding the previous step",
                    "code_MB_per_step": round(nbytes / K / 1e6, 2), "hbm_frac_layer": round(gbs / HBM_PEAK_GBS, 4)},
-        "roofline": roofline, "cpu_baseline": cpu, "prefill": prefill, "caller_dtypes": caller, "churn": churn, "stream": stream, "config2": config2}))
+        "roofline": roofline, "cpu_baseline": cpu, "prefill": prefill, "batches": batches, "caller_dtypes": caller, "churn": churn, "stream": stream, "config2": config2}))
 
 
 if __name__ == "__main__":

@@ -60,7 +60,9 @@ int nq_pf_decode(const int64_t* table, const int32_t* experts, int G, void* Wgu_
  * acc_gu >= (H/128/(cpw*nst)) * B*topk * 2I floats, acc_d >= (I/128/(cpw*nst)) * B*topk * H floats, h >= B*topk * I
  * halfs; cnt_gu >= B*topk * I/128 and cnt_d >= H/128 int32 arrival counters, zero on entry and zero again on exit (the
  * reference's workspace contract, sm120/nqmoe.cu:855-857). Picks with rw == 0, level <= 0 or an expert id outside
- * [0, E) contribute nothing. which: bit 0 = gate|up launch, bit 1 = down launch. hits: optional int32[E] pick counters
+ * [0, E) contribute nothing. which: bit 0 = gate|up launch, bit 1 = down launch; bit 2 = skip the call's first launch (routing
+ * and rotation of the activations) because route_ws and xrot still hold what an earlier call with the same x, sel, rw and table
+ * rows left there (what a benchmark of one projection launch alone uses). hits: optional int32[E] pick counters
  * (device or host-mapped memory), incremented once per pick with rw != 0 (reference :784-787). */
 /* Element types of the caller's tensors. The casts the reference's caller launches around the call (x.half(), ids.long(),
  * w.half(), out.to(x.dtype): sm120/serve/nq_vllm.py:522,560,573; fusing them is the open item of
@@ -112,10 +114,15 @@ typedef struct NqMoeArgs
                                  rows (reference route(), sm120/nqmoe.cu:379-449, which every block of the reference repeats) -- and
                                  leaves it here for the two projection launches */
     int64_t route_ws_bytes;
-    int64_t* mb_table;        /* optional mailbox, applied by the call's first launch before it reads the table: exactly
-                                 nq_mailbox(mb_table, mb_stage, mb_seq, mb_applied, mb_applied_host, E) followed by the layer call, in
-                                 one launch less (the reference's caller applies the mailbox at the top of every layer step,
-                                 sm120/serve/nq_vllm.py:546). NULL = no mailbox in this call; otherwise normally == table */
+    void* xrot;               /* fp16 [B*topk][2][H], 16-byte aligned, contents irrelevant on entry: the first launch also rotates the
+                                 activations of every active pick, once (x * su_g and x * su_u -> Hadamard-128 -> fp16; reference
+                                 sm120/nqmoe.cu:506-519, which every block repeats for its k-slice), for the gate|up launch */
+    int64_t xrot_elems;
+    int64_t* mb_table;        /* optional mailbox: the effect of nq_mailbox(mb_table, mb_stage, mb_seq, mb_applied, mb_applied_host, E)
+                                 followed by the layer call, without a launch of its own (the reference's caller applies the mailbox
+                                 at the top of every layer step, sm120/serve/nq_vllm.py:546): the routing launch takes the staged row
+                                 of every picked expert whose update is pending, and one extra workgroup of the first projection
+                                 launch writes the table and publishes applied. NULL = no mailbox in this call; otherwise == table */
     const int64_t* mb_stage;
     const int32_t* mb_seq;
     int32_t* mb_applied;
@@ -127,11 +134,11 @@ int nq_moe_forward(const NqMoeArgs* args, void* stream);
 /* nq_moe_forward for callers that cannot allocate device memory or keep workspaces of their own (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc). It has no counterpart in the reference, whose MoELayer
  * always owns its workspaces (sm120/moe.py:231-241). Same arguments, kernels and results as nq_moe_forward, except that the
- * workspace fields of *args (acc_gu, h, acc_d, cnt_gu, cnt_d, cnt_h, zd, route_ws and their capacities) are not looked at:
+ * workspace fields of *args (acc_gu, h, acc_d, cnt_gu, cnt_d, cnt_h, zd, route_ws, xrot and their capacities) are not looked at:
  * partial sums, h, z_d, the routing result and the arrival counters live in one array of NQ_STATIC_SCRATCH_BYTES that is part of the library's device
  * image (every GPU the library runs on holds its own copy until the process ends). The call allocates and frees nothing; it
  * clears the counters with a small kernel, then makes the two launches. A call whose shape and k-slices need more than the
- * array holds is refused with an error (full shape H=6144, I=2048, B*topk=64 picks with the default k-slices: about 7.3 MiB).
+ * array holds is refused with an error (full shape H=6144, I=2048, B*topk=64 picks with the default k-slices: about 8.9 MiB).
  * All calls on one GPU share the array: calls that overlap on one GPU (different streams) race; order them on one stream.
  * The first call on a device looks up the array's address (hipGetSymbolAddress) and so must not be made under stream
  * capture; later calls may be. */
@@ -177,7 +184,8 @@ int nq_pf_pre_rows(const void* x_f16, const int32_t* pt, const int32_t* pe, int 
  * mode 0: gate|up, K = H, N = 2I, A0 = xg feeds weight rows [0, I), A1 = xu feeds rows [I, 2I), C = [np][2I];
  * mode 1: down, K = I, N = H, A0 = h, A1 ignored, C = [np][H]. mode | 2: the variant for experts in mask mode (flags word of
  * the table row set): it handles only their tiles, the plain variant only the others, so a layer with such experts makes
- * both calls. Replaces pf_decode + the Triton grouped GEMM / aten.mm
+ * both calls; mode | 4: this is the only call for these tiles (the host knows every row to be of one kind), so a tile of the
+ * other kind, which nothing would compute, gets NaN results instead of stale scratch. Replaces pf_decode + the Triton grouped GEMM / aten.mm
  * (reference sm120/pf_gemm.py:7-34, sm120/moe.py:303-324); decoded weights never touch HBM. */
 int nq_pf_gemm(const int64_t* table, const int32_t* tiles, int ntiles, int bm, int mode, const void* A0_f16,
                const void* A1_f16, float* C, int E, int H, int I, void* stream);

@@ -23,7 +23,7 @@ class NqMoeArgs(C.Structure):
                 ("x_dtype", C.c_int32), ("sel_dtype", C.c_int32), ("rw_dtype", C.c_int32), ("out_dtype", C.c_int32),
                 ("cnt_h", C.c_void_p), ("cnt_h_elems", C.c_int64), ("zd", C.c_void_p), ("zd_elems", C.c_int64),
                 ("common_rows", C.c_int32), ("G", C.c_int32),
-                ("route_ws", C.c_void_p), ("route_ws_bytes", C.c_int64),
+                ("route_ws", C.c_void_p), ("route_ws_bytes", C.c_int64), ("xrot", C.c_void_p), ("xrot_elems", C.c_int64),
                 ("mb_table", C.c_void_p), ("mb_stage", C.c_void_p), ("mb_seq", C.c_void_p), ("mb_applied", C.c_void_p),
                 ("mb_applied_host", C.c_void_p)]
 

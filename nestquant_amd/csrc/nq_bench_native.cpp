@@ -129,6 +129,7 @@ int main(int argc, char** argv)
     HIPCHK(hipMalloc(&cnt_h, (size_t)S * (I / 128) * 4)); HIPCHK(hipMemset(cnt_h, 0, (size_t)S * (I / 128) * 4));
     HIPCHK(hipMalloc(&zd, (size_t)S * (I / 128) * 4 * sizeof(float)));
     void* route_ws; HIPCHK(hipMalloc(&route_ws, NQ_ROUTE_WS_BYTES));
+    void* xrot; HIPCHK(hipMalloc(&xrot, (size_t)S * 2 * H * 2));
     HIPCHK(hipMemset(cnt_gu, 0, (size_t)S * (I / 128) * 4)); HIPCHK(hipMemset(cnt_d, 0, (size_t)(H / 128) * 4));
     std::vector<int64_t> hsel((size_t)steps * S);
     for (int st = 0; st < steps; ++st)                                        // distinct picks; a step never reuses the previous step's experts
@@ -148,7 +149,7 @@ int main(int argc, char** argv)
     NqMoeArgs a; memset(&a, 0, sizeof a);
     a.x = x; a.rw = rw; a.table = d_table; a.out = out; a.acc_gu = acc_gu; a.h = h; a.acc_d = acc_d; a.cnt_gu = cnt_gu; a.cnt_d = cnt_d;
     a.acc_gu_elems = (int64_t)ny_gu * S * 2 * I; a.acc_d_elems = (int64_t)ny_dn * S * H; a.h_elems = (int64_t)S * I; a.out_elems = (int64_t)B * H;
-    a.cnt_gu_elems = (int64_t)S * (I / 128); a.cnt_d_elems = H / 128; a.cnt_h = cnt_h; a.cnt_h_elems = (int64_t)S * (I / 128); a.zd = zd; a.zd_elems = (int64_t)S * (I / 128) * 4; a.route_ws = route_ws; a.route_ws_bytes = NQ_ROUTE_WS_BYTES; a.common_rows = 1;   /* every row here has the K=2 base and a dense residual plane */
+    a.cnt_gu_elems = (int64_t)S * (I / 128); a.cnt_d_elems = H / 128; a.cnt_h = cnt_h; a.cnt_h_elems = (int64_t)S * (I / 128); a.zd = zd; a.zd_elems = (int64_t)S * (I / 128) * 4; a.route_ws = route_ws; a.route_ws_bytes = NQ_ROUTE_WS_BYTES; a.xrot = xrot; a.xrot_elems = (int64_t)S * 2 * H; a.common_rows = 1;   /* every row here has the K=2 base and a dense residual plane */
     a.B = B; a.topk = topk; a.E = E; a.H = H; a.I = I; a.which = 3;
     memcpy(a.cfg_gu, cfg_gu, sizeof cfg_gu); memcpy(a.cfg_dn, cfg_dn, sizeof cfg_dn);
     hipEvent_t e0, e1; HIPCHK(hipEventCreate(&e0)); HIPCHK(hipEventCreate(&e1));

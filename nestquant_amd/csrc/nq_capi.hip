@@ -105,7 +105,8 @@ static int moe_args(const char* who, const NqMoeArgs* p, bool own_ws, MoeArgs& a
     NQ_REQUIRE(p->B >= 1 && p->B <= 8 && p->topk >= 1 && p->B * p->topk <= 64, "%s: B=%d topk=%d (B <= 8, B*topk <= 64)", who, p->B, p->topk);
     NQ_REQUIRE(p->E >= 1, "%s: E=%d", who, p->E);
     NQ_REQUIRE(shape_ok(p->H, p->I), "%s: H=%d I=%d must be positive multiples of 128", who, p->H, p->I);
-    NQ_REQUIRE((p->which & ~3) == 0, "%s: which=%d", who, p->which);
+    NQ_REQUIRE((p->which & ~7) == 0, "%s: which=%d", who, p->which);
+    NQ_REQUIRE(!(p->which & 4) || (own_ws && !p->mb_table), "%s: which bit 2 (routing of an earlier call) needs the caller's route_ws / xrot and no mailbox", who);
     NQ_REQUIRE(p->force_level == 0 || p->force_level == 2 || p->force_level == 3 || p->force_level == 4, "%s: force_level=%d", who, p->force_level);
     NQ_REQUIRE(p->x_dtype >= 0 && p->x_dtype <= 2 && p->rw_dtype >= 0 && p->rw_dtype <= 2 && p->sel_dtype >= 0 && p->sel_dtype <= 1 && p->out_dtype >= 0 && p->out_dtype <= 2,
                "%s: dtype codes x=%d sel=%d rw=%d out=%d", who, p->x_dtype, p->sel_dtype, p->rw_dtype, p->out_dtype);
@@ -140,10 +141,13 @@ static int moe_args(const char* who, const NqMoeArgs* p, bool own_ws, MoeArgs& a
         NQ_REQUIRE(p->route_ws && p->route_ws_bytes >= NQ_ROUTE_WS_BYTES && ((uintptr_t)p->route_ws & 63) == 0,
                    "workspace too small: route_ws needs %d bytes, 64-byte aligned", NQ_ROUTE_WS_BYTES);
         a.route = (RouteWs*)p->route_ws;
+        NQ_REQUIRE(p->xrot && p->xrot_elems >= S * 2 * p->H && aligned16(p->xrot), "workspace too small: xrot needs B*topk * 2 * H halfs, 16-byte aligned");
+        a.xrot = (_Float16*)p->xrot;
     }
     if (p->mb_table)
     {
         NQ_REQUIRE(p->mb_stage && p->mb_seq && p->mb_applied, "%s: mailbox needs stage, seq and applied", who);
+        NQ_REQUIRE((const int64_t*)p->mb_table == p->table, "%s: the mailbox must be the one of the table the call reads", who);
         a.mb_table = p->mb_table; a.mb_stage = p->mb_stage; a.mb_seq = p->mb_seq; a.mb_applied = p->mb_applied; a.mb_applied_host = p->mb_applied_host;
     }
     NQ_REQUIRE(p->common_rows == 0 || p->common_rows == 1, "%s: common_rows=%d (0 or 1)", who, p->common_rows);
@@ -203,7 +207,7 @@ extern "C" int nq_pf_gemm(const int64_t* table, const int32_t* tiles, int ntiles
     NQ_REQUIRE(ntiles >= 0, "nq_pf_gemm: ntiles=%d", ntiles);
     if (ntiles == 0) return 0;
     NQ_REQUIRE(table && tiles && A0 && C, "nq_pf_gemm: null pointer");
-    NQ_REQUIRE(mode >= 0 && mode <= 3, "nq_pf_gemm: mode %d not in 0..3", mode);
+    NQ_REQUIRE(mode >= 0 && mode <= 7, "nq_pf_gemm: mode %d not in 0..7", mode);
     NQ_REQUIRE((mode & 1) == 1 || A1, "nq_pf_gemm: gate|up needs both activation buffers");
     NQ_REQUIRE(ntiles <= 65535, "nq_pf_gemm: %d tiles exceed one launch (65535)", ntiles);
     NQ_REQUIRE(E >= 1 && shape_ok(H, I), "nq_pf_gemm: E=%d H=%d I=%d (H, I positive multiples of 128)", E, H, I);

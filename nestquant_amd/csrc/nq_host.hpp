@@ -38,8 +38,10 @@ struct MoeArgs
                                       // 512-wide rotation the down launch's staging does the gate|up finisher (set by launch_moe)
     int ny_gu;                        // k-slices of the gate|up launch (the down launch's fused staging sums that many partials)
     RouteWs* route;                   // NQ_ROUTE_WS_BYTES of device memory: what the routing launch hands to the projection launches
+    _Float16* xrot;                   // [B * topk][2][H] fp16: rotated activations of every active pick (gate, up), B-operand order
+    int mb_apply;                     // this projection launch carries the block that applies the mailbox (set by launch_moe)
     int64_t* mb_table; const int64_t* mb_stage; const int32_t* mb_seq; int32_t* mb_applied; int32_t* mb_applied_host;
-                                      // mailbox applied by the routing launch before it reads the table (mb_table == nullptr: none)
+                                      // mailbox of the call (mb_table == nullptr: none): pending rows are honoured by the routing launch, written by the first projection launch
 };
 
 // kernel launchers defined next to their kernels

@@ -123,6 +123,7 @@ struct alignas(64) RunHdr
     int level, ntok;
     int had;                      // width of the Hadamard on the down projection's input: 128 or 512
     int rg, rd;
+    int q0;                       // rotated activations of the run's token j: row q0 + j of MoeArgs::xrot
     unsigned char slot[MAXTOK];   // pick index (token * topk + k) of the run's tokens
     __device__ __forceinline__ int slot_of(int j) const       // by shifts: a run-time index into slot[] would put the header into scratch memory
     {
@@ -158,7 +159,8 @@ __device__ __forceinline__ void ld_sys_row(const int64_t* p, int64_t* f)
 // in the call the lane also reads the expert's seq / applied pair: when they differ, its row is the staged one (read after
 // seq, as the mailbox does), which is what the table holds once the mailbox part of this kernel has written it; nothing
 // writes the table before every routing read is done (see nq_prep_k), so the plain loads of the row cannot be torn.
-__device__ __forceinline__ void route(const MoeArgs& a, RouteWs* W, int lane)
+struct PrepRows { int nq; unsigned char tok[64]; const _Float16* signs[64]; };    // LDS: the rows of xrot, one per active pick
+__device__ __forceinline__ void route(const MoeArgs& a, RouteWs* W, int lane, bool writer, PrepRows* Q)
 {
     const int S = a.B * a.topk;
     int e = -1, lv = 0; bool ok = false, inrange = false;
@@ -184,7 +186,7 @@ __device__ __forceinline__ void route(const MoeArgs& a, RouteWs* W, int lane)
             ok = rw_at(a, lane) != 0.f && lv > 0;
         }
     }
-    if (a.hits && inrange && rw_at(a, lane) != 0.f)
+    if (writer && a.hits && inrange && rw_at(a, lane) != 0.f)
         __hip_atomic_fetch_add(a.hits + e, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     const int level = a.force_level ? a.force_level : lv;
     // Runs of refined experts (level 3, 4: twice the decode work per chunk) are numbered before the level-2 ones, each group
@@ -195,7 +197,7 @@ __device__ __forceinline__ void route(const MoeArgs& a, RouteWs* W, int lane)
     const unsigned long long below = (1ull << lane) - 1ull;
     const int tok = lane / a.topk, sh = tok * a.topk;
     const unsigned long long mytok = sh < 64 ? (a.topk >= 64 ? ~0ull : ((1ull << a.topk) - 1ull)) << sh : 0ull;
-    int r = 0;
+    int r = 0, cum = 0;
     for (int pass = 0; pass < 2; ++pass)
     {
         unsigned long long rem = pass == 0 ? heavy : okm & ~heavy;
@@ -206,6 +208,11 @@ __device__ __forceinline__ void route(const MoeArgs& a, RouteWs* W, int lane)
             const unsigned long long same = __ballot(((rem >> lane) & 1ull) && e == ev);
             const unsigned long long m = __ballot(((same >> lane) & 1ull) && (same & mytok & below) == 0ull);   // first pick per token
             if ((m >> lane) & 1ull)
+            {
+                const int pos = __popcll(m & below);
+                Q->tok[cum + pos] = (unsigned char)tok; Q->signs[cum + pos] = (const _Float16*)f[9];
+            }
+            if (writer && ((m >> lane) & 1ull))
             {
                 const int pos = __popcll(m & below);
                 W->run[0][r].slot[pos] = (unsigned char)lane; W->run[1][r].slot[pos] = (unsigned char)lane;
@@ -222,13 +229,15 @@ __device__ __forceinline__ void route(const MoeArgs& a, RouteWs* W, int lane)
                         R.level = level;
                         R.had = f[18] == 512 ? 512 : 128;
                         R.lr = (const _Float16*)f[14]; R.lr4 = (const _Float16*)f[15]; R.rg = (int)f[16]; R.rd = (int)f[17];
-                        R.ntok = __popcll(m);
+                        R.ntok = __popcll(m); R.q0 = cum;
                     }
                 }
             }
-            rem &= ~m; ++r;
+            rem &= ~m; ++r; cum += __popcll(m);
         }
     }
+    if (lane == 0) Q->nq = cum;
+    if (!writer) return;
     PickInfo& K = W->picks;
     K.w[lane] = ok ? rw_at(a, lane) : 0.f; K.signs[lane] = (const _Float16*)f[9];
     K.lr[lane] = (const _Float16*)f[14]; K.lr4[lane] = (const _Float16*)f[15];
@@ -236,42 +245,49 @@ __device__ __forceinline__ void route(const MoeArgs& a, RouteWs* W, int lane)
     if (lane == 0) W->nruns = r;
 }
 
-// First launch of every layer call, one workgroup of five wavefronts: wavefront 0 does the routing, once for both projection
-// launches (which then read one RunHdr each instead of repeating the dependent loads sel -> table row in every one of their
-// ~1800 workgroups) and the hits export; wavefronts 1..4 are the mailbox, when the caller hands its buffers over with the call
-// (table[e] <- stage[e] where seq[e] != applied[e], then applied[e] <- seq[e], as nq_mailbox_k). Both read at the same time,
-// so the call's chain of memory round trips is sel -> row (+ the staged row of an expert whose update is pending); the
-// mailbox writes the table only after the barrier that the routing wavefront reaches when all its reads are done.
-__global__ void __launch_bounds__(320) nq_prep_k(MoeArgs a)
+// The mailbox's write half: table[e] <- stage[e] where seq[e] != applied[e], then applied[e] <- seq[e] (device copy and the
+// optional host-mapped mirror), by the threads of one workgroup.
+__device__ __forceinline__ void mailbox_apply(int64_t* table, const int64_t* stage, const int32_t* seq, int32_t* applied, int32_t* applied_host, int E)
 {
-    const int t = (int)threadIdx.x - 64;
-    int64_t row[TBL_W];
-    int32_t sq = 0; bool pend = false;
-    if (t < 0) route(a, a.route, threadIdx.x);
-    else if (a.mb_table && t < a.E)
+    for (int e = threadIdx.x; e < E; e += blockDim.x)
     {
-        const int32_t ap = a.mb_applied[t];
-        sq = __hip_atomic_load(a.mb_seq + t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-        pend = sq != ap;
-        if (pend) ld_sys_row(a.mb_stage + (size_t)t * TBL_W, row);
-    }
-    if (!a.mb_table) return;                                     // block-uniform
-    __syncthreads();
-    if (t < 0) return;
-    for (int e = t; e < a.E; e += 256)
-    {
-        if (e != t)
-        {
-            sq = __hip_atomic_load(a.mb_seq + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-            pend = sq != a.mb_applied[e];
-            if (pend) ld_sys_row(a.mb_stage + (size_t)e * TBL_W, row);
-        }
-        if (!pend) continue;
+        const int32_t ap = applied[e];
+        const int32_t sq = __hip_atomic_load(seq + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        if (sq == ap) continue;
+        int64_t row[TBL_W];
+        ld_sys_row(stage + (size_t)e * TBL_W, row);
 #pragma unroll
-        for (int i = 0; i < TBL_W; ++i) a.mb_table[(size_t)e * TBL_W + i] = row[i];
+        for (int i = 0; i < TBL_W; ++i) table[(size_t)e * TBL_W + i] = row[i];
         __threadfence();
-        a.mb_applied[e] = sq;
-        if (a.mb_applied_host) __hip_atomic_store(a.mb_applied_host + e, sq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        applied[e] = sq;
+        if (applied_host) __hip_atomic_store(applied_host + e, sq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+}
+
+// First launch of every layer call. Every workgroup repeats the routing (its first wavefront; workgroup 0 writes the result:
+// run headers for both projection launches, which then read one header each instead of repeating the dependent loads
+// sel -> table row in every one of their ~1800 workgroups, the per-pick data of the combine, the hits export); then the
+// wavefronts of the grid share the rotation of the activations: one task per (active pick q, gate or up, 128-column chunk):
+// xrot[q][gate|up][chunk] = fp16(Hadamard-128(x[token] * su)) in the MFMA B-operand column order, which the gate|up launch
+// copies into LDS (before, each of the 32 row blocks of a run repeated these rotations: 9 % of the launch's vector
+// instructions). With a mailbox in the call nothing here writes the table: a pick whose expert has an update pending takes
+// the staged row, and the first projection launch carries the workgroup that applies the mailbox (mailbox_apply).
+__global__ void __launch_bounds__(256) nq_prep_k(MoeArgs a)
+{
+    __shared__ PrepRows Q;
+    const int lane = threadIdx.x & 63;
+    if (threadIdx.x < 64) route(a, a.route, lane, blockIdx.x == 0, &Q);
+    __syncthreads();
+    const int C = a.H / 128, ntask = Q.nq * 2 * C;
+    for (int t = blockIdx.x * 4 + (threadIdx.x >> 6); t < ntask; t += gridDim.x * 4)
+    {
+        const int q = t / (2 * C), r = t - q * 2 * C, up = r / C, c = r - up * C, kk = c * 128 + 2 * lane;
+        const _Float16* su = Q.signs[q] + (up ? 2 * a.H + 3 * a.I : 0);
+        const half2_t xv = x2_at(a, (size_t)Q.tok[q] * a.H + kk), sv = *(const half2_t*)(su + kk);
+        float v0 = (float)xv.x * (float)sv.x, v1 = (float)xv.y * (float)sv.y;
+        wht128(v0, v1, lane);
+        _Float16* dst = a.xrot + ((size_t)q * 2 + up) * a.H + c * 128;
+        dst[bop_index(2 * lane)] = (_Float16)v0; dst[bop_index(2 * lane + 1)] = (_Float16)v1;
     }
 }
 
@@ -416,6 +432,7 @@ __device__ __forceinline__ void finish_dn(const MoeArgs& a, const PickInfo& R, i
                 const int kq = k + q * SB, s = b * a.topk + kq;
                 if (kq >= a.topk || R.w[s] == 0.f) continue;     // what route() saw: no second look at the table
                 w[q] = R.w[s]; rows2[q] = a.part_d + (size_t)s * a.H + col;
+
                 sv[q] = *(const half2_t*)(R.signs[s] + a.H + 3 * a.I + col);
             }
             if (w[0] == 0.f && w[1] == 0.f) continue;
@@ -476,6 +493,12 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
     __shared__ float zl[MAXTOK][4];                              // gate|up finisher: x V_gu^T of the run's tokens (low-rank plane)
     __shared__ int last;
     const int lane = threadIdx.x & 63, warp = threadIdx.x >> 6, SB = blockDim.x >> 6;
+    if (a.mb_apply && blockIdx.z == gridDim.z - 1)
+    {   // the extra plane of blocks of a call with a mailbox: one of them applies it (the routing launch has already taken the
+        // staged rows of pending experts, and neither projection launch reads the table)
+        if (blockIdx.x == 0 && blockIdx.y == 0) mailbox_apply(a.mb_table, a.mb_stage, a.mb_seq, a.mb_applied, a.mb_applied_host, a.E);
+        return;
+    }
     // the run's header, written by nq_prep_k: block-uniform, read through the scalar cache (constant address space)
     typedef const __attribute__((address_space(4))) RouteWs* cws_t;
     const cws_t W = (cws_t)a.route;
@@ -486,7 +509,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
         for (int i = 0; i < (int)(sizeof(RunHdr) / 4); ++i) raw.w[i] = src[i];
     }
     const int nruns = W->nruns;
-    const int N = MODE == 0 ? 2 * a.I : a.H, K = MODE == 0 ? a.H : a.I, C = K / 128, NY = C / NC;
+    const int N = MODE == 0 ? 2 * a.I : a.H, K = MODE == 0 ? a.H : a.I, C = K / 128;
     if (MODE == 1 && nruns == 0 && blockIdx.z == 0 && blockIdx.y == 0)
     {   // no active pick at all: nobody will arrive last, so the first plane of blocks writes the zero output
         for (int i = threadIdx.x; i < a.B * SB * 16; i += blockDim.x)
@@ -494,6 +517,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
     }
     if ((int)blockIdx.z >= nruns) return;                        // block-uniform
     const RunHdr R = __builtin_bit_cast(RunHdr, raw);
+    const int NY = C / NC;
     const int ntok = R.ntok, chunk0 = blockIdx.y * NC, k0 = chunk0 * 128;
     const int rowstride = NC * 256 + 16;                         // bytes per staged token (+16: spread tokens over banks)
     char* zero = smem + ntok * rowstride;                        // 256 zero bytes after the token rows
@@ -518,33 +542,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
     // ---- stage the run's tokens for this k-slice in B-operand order
     if constexpr (MODE == 0)
     {
-        const bool up = (int)(blockIdx.x * SB * 32) >= a.I;      // gate rows use su_g, up rows su_u
-        const _Float16* su = up ? signs + 2 * a.H + 3 * a.I : signs;
-        // task = (token j, chunk c); a wavefront takes tasks warp, warp + SB, .. four at a time so that their activation and
-        // scale reads are in flight together
-        const int ntask = ntok * NC;
-        for (int t0 = warp; t0 < ntask; t0 += 4 * SB)
+        // rotated by nq_prep_k, already in B-operand order: 16 bytes per thread and step
+        const bool up = (int)(blockIdx.x * SB * 32) >= a.I;      // gate rows were rotated with su_g, up rows with su_u
+        const _Float16* xr = a.xrot + ((size_t)R.q0 * 2 + (up ? 1 : 0)) * a.H + k0;
+        for (int i = threadIdx.x; i < ntok * NC * 16; i += blockDim.x)
         {
-            half2_t xv[4], sv[4];
-            int dsto[4];
-#pragma unroll
-            for (int u = 0; u < 4; ++u)
-            {
-                const int task = t0 + u * SB < ntask ? t0 + u * SB : t0;
-                const int j = task / NC, c = task - j * NC, kk = k0 + c * 128 + 2 * lane;
-                const int tok = R.slot_of(j) / a.topk;
-                xv[u] = x2_at(a, (size_t)tok * a.H + kk); sv[u] = *(const half2_t*)(su + kk);
-                dsto[u] = j * rowstride + c * 256;
-            }
-#pragma unroll
-            for (int u = 0; u < 4; ++u)
-            {
-                if (t0 + u * SB >= ntask) break;
-                float v0 = (float)xv[u].x * (float)sv[u].x, v1 = (float)xv[u].y * (float)sv[u].y;
-                wht128(v0, v1, lane);
-                _Float16* dst = (_Float16*)(smem + dsto[u]);
-                dst[bop_index(2 * lane)] = (_Float16)v0; dst[bop_index(2 * lane + 1)] = (_Float16)v1;
-            }
+            const int j = i / (NC * 16), r = i - j * NC * 16;
+            *(u32x4*)(smem + j * rowstride + r * 16) = *(const u32x4*)(xr + (size_t)j * 2 * a.H + r * 8);
         }
     }
     else if (a.fuse && R.had != 512 && R.lr == nullptr)
@@ -658,8 +662,16 @@ __global__ void nq_mailbox_k(int64_t* table, const int64_t* stage, const int32_t
 int launch_moe(const MoeArgs& a, const int* cfg_gu, const int* cfg_dn, int which, hipStream_t st)
 {
     const int S = a.B * a.topk;
-    nq_prep_k<<<1, 320, 0, st>>>(a);
-    NQ_LAUNCH_CHECK("moe_forward (routing)");
+    const bool reuse = (which & 4) != 0;                          // the routing launch of an earlier call left route_ws / xrot as this call needs them
+    which &= 3;
+    if (!reuse)
+    {
+        const int ntask = S * 2 * (a.H / 128);                   // upper bound: every pick active
+        nq_prep_k<<<std::min((ntask + 3) / 4, 1024), 256, 0, st>>>(a);
+        NQ_LAUNCH_CHECK("moe_forward (routing)");
+    }
+    if (a.mb_table && which == 0) return launch_mailbox(a.mb_table, a.mb_stage, a.mb_seq, a.mb_applied, a.mb_applied_host, a.E, st);
+    bool mb_todo = a.mb_table != nullptr;
     for (int mode = 0; mode < 2; ++mode)
     {
         if (!((which >> mode) & 1)) continue;
@@ -672,13 +684,14 @@ int launch_moe(const MoeArgs& a, const int* cfg_gu, const int* cfg_dn, int which
         MoeArgs b = a;
         b.fuse = which == 3;                                      // both launches belong to this call
         b.ny_gu = (a.H / 128) / (cfg_gu[0] * cfg_gu[2]);
+        b.mb_apply = mb_todo; mb_todo = false;                    // the call's first projection launch carries the mailbox block
         auto kern = mode == 0 ? (any ? nq_gemv_k<0, true> : nq_gemv_k<0, false>) : (any ? nq_gemv_k<1, true> : nq_gemv_k<1, false>);
         if (shm > 48 * 1024)
         {
             hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, shm);
             if (e != hipSuccess) return set_error("moe_forward: LDS %d bytes: %s", shm, hipGetErrorString(e));
         }
-        kern<<<dim3(NX, NY, S), 64 * SB, shm, st>>>(b, NC);
+        kern<<<dim3(NX, NY, S + (b.mb_apply ? 1 : 0)), 64 * SB, shm, st>>>(b, NC);
         NQ_LAUNCH_CHECK("moe_forward");
     }
     return 0;
@@ -724,14 +737,14 @@ int launch_moe_static(MoeArgs a, const int* cfg_gu, const int* cfg_dn, int which
     auto take = [&](size_t bytes) { const size_t o = off; off += (bytes + 255) & ~(size_t)255; return o; };
     const size_t o_cnt = take((2 * S * G128 + (size_t)a.H / 128) * sizeof(int));       // cnt_gu | cnt_h | cnt_d: cleared below
     const size_t o_gu = take(ny_gu * S * 2 * a.I * sizeof(float)), o_d = take(ny_dn * S * a.H * sizeof(float));
-    const size_t o_h = take(S * a.I * sizeof(_Float16)), o_zd = take(S * G128 * 4 * sizeof(float)), o_route = take(sizeof(RouteWs));
+    const size_t o_h = take(S * a.I * sizeof(_Float16)), o_zd = take(S * G128 * 4 * sizeof(float)), o_route = take(sizeof(RouteWs)), o_xrot = take(S * 2 * a.H * sizeof(_Float16));
     if (off > STATIC_SCRATCH_BYTES)
         return set_error("nq_moe_forward_static: this call needs %zu bytes of workspace (B=%d topk=%d H=%d I=%d, %zu and %zu k-slices), the built-in "
                          "scratch holds %zu: use coarser k-slices, or nq_moe_forward with workspaces of the caller's", off, a.B, a.topk, a.H, a.I, ny_gu, ny_dn,
                          STATIC_SCRATCH_BYTES);
     a.cnt_gu = (int*)(base + o_cnt); a.cnt_h = a.cnt_gu + S * G128; a.cnt_d = a.cnt_h + S * G128;
     a.part_gu = (float*)(base + o_gu); a.part_d = (float*)(base + o_d); a.h = (_Float16*)(base + o_h); a.zd = (float*)(base + o_zd);
-    a.route = (RouteWs*)(base + o_route);
+    a.route = (RouteWs*)(base + o_route); a.xrot = (_Float16*)(base + o_xrot);
     // the counters must be zero on entry; a fill kernel, not hipMemsetAsync, so that the call can be recorded into a graph
     const int ncnt = (int)(2 * S * G128 + (size_t)a.H / 128);
     nq_clear_k<<<(ncnt + 255) / 256, 256, 0, st>>>(a.cnt_gu, ncnt);

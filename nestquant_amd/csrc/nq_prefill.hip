@@ -392,6 +392,7 @@ struct PfGemm
     const int64_t* table; const int32_t* tiles;   // tiles [ntiles][4]: expert, first row, rows (<= 16 TG), unused
     const _Float16* A0; const _Float16* A1;         // activations in B-operand order: A0 for weight rows < I (or all rows of down), A1 above
     float* C; int mode, E, H, I;
+    int solo;                                       // the other kernel variant will not be launched on these tiles: a tile that is its kind comes out NaN
 };
 
 // body for one (RES, CODE): all K / 128 chunks of this wave's two strips against the tile's tokens
@@ -555,7 +556,16 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) n
     const _Float16* A = (a.mode == 0 && (int)(blockIdx.x * 128) >= a.I) ? a.A1 : a.A0;
     const int t4 = lane >> 4, ss = (lane >> 3) & 1, g = lane & 7, n = lane & 15;
     const Planes P = planes_of(ent, a.mode);
-    if (((P.flags != nullptr && lv == 4) || P.bcode != 0) != MASKED) return;       // block-uniform
+    if (((P.flags != nullptr && lv == 4) || P.bcode != 0) != MASKED)              // block-uniform: the other variant's tile
+    {
+        if (a.solo)
+        {   // nobody will compute it (the host vouched for rows of one kind only): NaN, not whatever the scratch held
+            const float nan = __builtin_nanf("");
+            for (int i = threadIdx.x; i < nrows * 32; i += blockDim.x)
+                *(float4_t*)(a.C + (size_t)(row0 + i / 32) * N + blockIdx.x * 128 + 4 * (i % 32)) = float4_t{nan, nan, nan, nan};
+        }
+        return;
+    }
     LaneCtx L;
     L.unit0 = (size_t)(2 * sp + ss) * C; L.rec0 = L.unit0 * 32 + 4 * g + t4;
     L.nrec = (size_t)(N / 16) * C * 32;
@@ -639,7 +649,7 @@ int launch_pf_gemm(const int64_t* table, const int32_t* tiles, int ntiles, int b
                    int E, int H, int I, hipStream_t st)
 {
     if (!ntiles) return 0;
-    PfGemm a{table, tiles, (const _Float16*)A0, (const _Float16*)A1, C, mode & 1, E, H, I};
+    PfGemm a{table, tiles, (const _Float16*)A0, (const _Float16*)A1, C, mode & 1, E, H, I, (mode & 4) != 0};
     const int N = (mode & 1) == 0 ? 2 * I : H;
     const bool masked = (mode & 2) != 0;
     switch (bm)

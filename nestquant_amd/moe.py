@@ -146,6 +146,7 @@ class MoELayer:
         s.zd = torch.zeros(S * (I // 128) * 4, dtype=f32, device=dev); s.cnt_h = torch.zeros(S * (I // 128), dtype=i32, device=dev)
         s.out = torch.zeros(Bmax, H, dtype=f32, device=dev)
         s.route = torch.zeros(_lib.ROUTE_WS_BYTES, dtype=torch.uint8, device=dev)    # the routing launch's result for the projection launches
+        s.xrot = torch.zeros(S, 2, H, dtype=torch.float16, device=dev)               # and the rotated activations of every pick
         s.hits_ptr = 0
         s.rare_rows = False                           # set once a row in mask mode or with a base window code other than 0 is
                                                       # installed (set / Mailbox.post): the decode call then runs the kernel that
@@ -157,7 +158,7 @@ class MoELayer:
     # k-slice lengths (chunks) per token count 1..8 at the full shape H = 6144, I = 2048, top-8 over 256 experts, measured on
     # an MI355X with the routing of the layer benchmark; the reference keeps such tables for its GPUs
     # (sm120/serve/nq_vllm.py:32-33). Index = tokens of the call; other shapes use default_cfg for every count.
-    TUNED_NST = {(6144, 2048): ([12, 12, 24, 12, 24, 24, 24, 24, 24], [8, 8, 16, 16, 16, 16, 16, 16, 16])}
+    TUNED_NST = {(6144, 2048): ([12, 12, 24, 12, 24, 24, 24, 24, 24], [4, 4, 16, 16, 16, 16, 16, 16, 16])}
 
     def cfg_for(s, T):
         """(cfg_gu, cfg_dn) for a decode call of T tokens: the layer's defaults, with the tuned k-slice length for T where this
@@ -180,15 +181,29 @@ class MoELayer:
         return C // (cfg[0] * cfg[2])
 
     def _alloc_partials(s, cfg_gu=None, cfg_dn=None):
+        """Partial-sum workspaces for the given (default: the layer's) tilings. At construction they are sized for the finest
+        k-split among the layer's default and its tuned tilings, so the calls a serving loop makes never re-size them. A call
+        that brings a finer split of its own replaces them -- graphs captured before hold the old addresses and must be
+        captured again -- and that is refused while the stream is capturing (an allocation cannot be captured)."""
         S, dev = s.Bmax * s.topk, s.table.device
         ny_gu, ny_dn = s._ny(cfg_gu or s.cfg_gu, s.H // 128), s._ny(cfg_dn or s.cfg_dn, s.I // 128)
-        if getattr(s, "acc_gu", None) is None or s.acc_gu.shape[0] < ny_gu:
+        first = getattr(s, "acc_gu", None) is None
+        if first:
+            t = s.TUNED_NST.get((s.H, s.I))
+            if t is not None:
+                ny_gu = max([ny_gu] + [(s.H // 128) // (s.cfg_gu[0] * n) for n in t[0]])
+                ny_dn = max([ny_dn] + [(s.I // 128) // (s.cfg_dn[0] * n) for n in t[1]])
+        grow_gu, grow_dn = first or s.acc_gu.shape[0] < ny_gu, first or s.acc_d.shape[0] < ny_dn
+        if (grow_gu or grow_dn) and not first and torch.cuda.is_current_stream_capturing():
+            raise RuntimeError("this call's k-split needs larger partial-sum workspaces than the layer holds; make one call with "
+                               "these tilings (or set_cfg) before capturing")
+        if grow_gu:
             s.acc_gu = torch.zeros(ny_gu, S, 2 * s.I, dtype=torch.float32, device=dev)
-        if getattr(s, "acc_d", None) is None or s.acc_d.shape[0] < ny_dn:
+        if grow_dn:
             s.acc_d = torch.zeros(ny_dn, S, s.H, dtype=torch.float32, device=dev)
 
     def set_cfg(s, cfg_gu=None, cfg_dn=None):
-        """change the default tilings (re-sizes the partial-sum workspaces; not graph-safe)"""
+        """change the default tilings (may replace the partial-sum workspaces: graphs captured before must be captured again)"""
         s.cfg_gu, s.cfg_dn = list(cfg_gu or s.cfg_gu), list(cfg_dn or s.cfg_dn)
         s._tuned = False
         s._alloc_partials()
@@ -234,6 +249,7 @@ class MoELayer:
         a.zd, a.zd_elems = s.zd.data_ptr(), s.zd.numel()
         a.G = s.G
         a.route_ws, a.route_ws_bytes = s.route.data_ptr(), s.route.numel()
+        a.xrot, a.xrot_elems = s.xrot.data_ptr(), s.xrot.numel()
         if mailbox is not None:
             a.mb_table, a.mb_stage, a.mb_seq = tb.data_ptr(), mailbox.stage.data_ptr(), mailbox.seq.data_ptr()
             a.mb_applied, a.mb_applied_host = mailbox.applied.data_ptr(), mailbox.applied_host.data_ptr()
@@ -351,7 +367,9 @@ def prefill(s, x, sel, rw, out=None, R=None, G=None, table=None):
     R = min(P, R or int(__import__("os").environ.get("NQ_PF_ROWS", "32768")))
     S = pf_scratch(dev, H, I, R)
     cap = E + R // 256 + 1
-    variants = (0, 2) if s.rare_rows else (0,)                    # mask mode / other base codes run in their own kernel variant
+    # mask mode / other base codes run in their own kernel variant; a caller's own table may hold such rows, so it gets both,
+    # and a lone variant is told so (| 4): should it meet a row of the other kind after all, the result is NaN, not stale scratch
+    variants = (0, 2) if (s.rare_rows or table is not None) else (4,)
     for c in range(0, P, R):
         d = min(P, c + R); n = d - c
         # tile lists of the chunk, built on the device from the expert counts: list i = tiles of height 16 << i, entries

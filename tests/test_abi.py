@@ -102,6 +102,8 @@ def test_argument_checks_run_before_any_device_work():
     a.acc_gu_elems = a.acc_d_elems = a.h_elems = a.out_elems = a.cnt_gu_elems = a.cnt_d_elems = a.cnt_h_elems = a.zd_elems = 1 << 40
     assert L.nq_moe_forward(C.byref(a), None) != 0 and "route_ws" in err()
     a.route_ws_bytes = _lib.ROUTE_WS_BYTES
+    assert L.nq_moe_forward(C.byref(a), None) != 0 and "xrot" in err()
+    a.xrot, a.xrot_elems = base, 1 << 40
     assert L.nq_moe_forward(C.byref(a), None) != 0 and "G=3" in err()
     a.G = 4; a.mb_table = base
     assert L.nq_moe_forward(C.byref(a), None) != 0 and "mailbox needs" in err()

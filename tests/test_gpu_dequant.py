@@ -249,3 +249,22 @@ def test_base_code_1_layer_decode_and_prefill():
     assert not L.cnt_gu.any() and not L.cnt_d.any()                  # the workspace contract holds on that path too
     L.rare_rows = True
     assert torch.equal(L(x, sel, rw), ref)
+    # the same in prefill: a table handed over with the call is of unknown kind, so both kernel variants run and the result is
+    # right whatever the layer object believes; a wrong "all rows common" makes the lone variant write NaN for the tiles it has
+    # no loop for (never the stale contents of the shared scratch) and leaves the tokens of common rows alone
+    T = 24
+    selp = torch.stack([torch.randperm(NE, generator=g)[:3] for _ in range(T)]).to(DEV)
+    selp[:4] = 1                                                     # four tokens that pick only the common expert 1
+    rwp = (torch.rand(T, 3, generator=g) + 0.1).half().to(DEV)
+    xp = (torch.randn(T, H, generator=g) * 0.05).half().to(DEV)
+    want = L.prefill(xp, selp, rwp).clone()
+    assert rel_err(want.cpu().numpy(), oracle_layer(planes, levels, signs, xp, selp, rwp)) < 5e-5
+    L.rare_rows = False
+    assert torch.equal(L.prefill(xp, selp, rwp, table=L.table.clone()), want)
+    yp = L.prefill(xp, selp, rwp).clone()
+    torch.cuda.synchronize()
+    assert torch.equal(yp[:4], want[:4])
+    rare = torch.tensor([bool(L.table[e, 19]) or bool(L.table[e, 4]) for e in range(NE)], device=DEV)
+    hit = rare[selp].any(1)
+    assert bool(hit.any()) and bool(torch.isnan(yp[hit]).any(1).all()) and torch.equal(yp[~hit], want[~hit])
+    L.rare_rows = True

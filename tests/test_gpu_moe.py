@@ -143,9 +143,9 @@ def test_full_shape_layer_like_reference_check():
                 worst = max(worst, err)
                 assert err < 5e-5, (B, mode, cg, cd, err)
                 assert rel_err(y.cpu().numpy(), pure) < 1e-3, (B, mode, cg, cd)
-            # no tiling given: the k-slice lengths tuned for this shape and token count (the default ones at B = 1 and 3)
+            # no tiling given: the k-slice lengths tuned for this shape and token count (gate|up: the default one at B = 1 and 3)
             tg, td = L.cfg_for(B)
-            assert (tg[2], td[2]) == {1: (12, 8), 2: (24, 16), 3: (12, 16), 4: (24, 16)}[B] and tg[:2] == L.cfg_gu[:2]
+            assert (tg[2], td[2]) == {1: (12, 4), 2: (24, 16), 3: (12, 16), 4: (24, 16)}[B] and tg[:2] == L.cfg_gu[:2]
             y = L(x, sel, rw)
             torch.cuda.synchronize()
             assert rel_err(y.cpu().numpy(), want) < 5e-5 and torch.equal(y, L(x, sel, rw, cfg_gu=tg, cfg_dn=td))
@@ -163,7 +163,9 @@ def test_force_level_which_hits_and_out_of_range_ids():
     for e in range(NE):
         L.set(e, ex[e], 4)
     sel = torch.tensor([[0, 1, 2, 3], [3, 4, 5, 0]], device=DEV); rw = torch.full((2, 4), 0.25, device=DEV).half()
-    x = (torch.randn(2, H, device=DEV) * 0.05).half()
+    # seeded on the host: drawn from the device's default generator, x depended on every test that ran before this one, and at this
+    # small shape an unlucky draw puts the fp32 sums themselves (numpy's as much as the kernels') 6e-5 from the float64 arbiter
+    x = (torch.randn(2, H, generator=torch.Generator().manual_seed(3)) * 0.05).half().to(DEV)
     signs = [e.signs.cpu().numpy() for e in ex]
     for lv in (2, 4):                                            # rows are level 4; force_level = 2 must read the base only
         dense = _dense_from_gpu(ex, [lv] * NE)
