@@ -153,9 +153,11 @@ int nq_mailbox(int64_t* table, const int64_t* stage, const int32_t* seq, int32_t
 /* Decode salience export: acc[e] += sum over the picks (t, k) with ids[t][k] == e of (rsf * w[t][k])^2 * sum_i x[t][i]^2, for
  * T <= 8 tokens of K <= 8 picks; acc fp64 [E] on the device, every touched entry also stored to host [host-mapped fp64 [E]].
  * x [T][H] with row stride x_row_stride elements, NQ_DT_F16 / NQ_DT_BF16 (or NQ_DT_F32, rounded through fp16); w [T][K]
- * likewise (rounded through fp16); ids NQ_DT_I64 / NQ_DT_I32. Picks with w == 0 or an id outside [0, E) are skipped. fp32
- * sums in the reference kernel's order, so the exported values are the same bits. Calls on one layer must be stream-ordered
- * (acc is updated without atomics). Replaces sal (reference sm120/nqsal.cu:19-78, called at sm120/serve/nq_vllm.py:558,572). */
+ * likewise (rounded through fp16); ids NQ_DT_I64 / NQ_DT_I32. Picks with w == 0 or an id outside [0, E) are skipped. The
+ * squared norm is an fp32 sum in this kernel's own order (one wavefront per token), the per-pick terms and the running sums
+ * are fp64: values agree with the reference's to fp32 rounding of the norm, not bit for bit. Calls on one layer must be
+ * stream-ordered (acc is updated without atomics). Replaces sal (reference sm120/nqsal.cu:19-78, called at
+ * sm120/serve/nq_vllm.py:558,572). */
 int nq_sal(const void* x, int x_dtype, int64_t x_row_stride, const void* w, int w_dtype, const void* ids, int ids_dtype, int T,
            int H, int K, int E, double rsf, double* acc, double* host, void* stream);
 

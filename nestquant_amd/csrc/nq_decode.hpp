@@ -17,6 +17,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <utility>
 
 namespace nq {
 
@@ -42,6 +43,8 @@ typedef const NQ_GLOBAL uint8_t* gp_u8;
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
+
+template <int C> struct CodeTag { static constexpr int value = C; };        // a compile-time integer passed to generic lambdas
 
 // ---- window patterns (reference sm120/moe.py:10-12, sm120/nqmoe.cu:128-138) ----------------------------------------
 template <int CODE> struct Pat;
@@ -80,59 +83,80 @@ __host__ inline int rec_bits(int code)
 }
 
 // ---- record loads ---------------------------------------------------------------------------------------------------
-// Residual plane = sub-arrays uint4 x n4 | uint2 | uint | ushort, each contiguous over all nrec records, then a tail of
-// BITS % 16 bits per record bit-packed over records (reference sm120/moe.py:36-49, sm120/nqmoe.cu:17-20).
-// Code 11 stores its 128-bit record as uint2 (plane P3) | uint2 (plane P4).
+// A residual plane stores the BITS bits of a record as a series of sub-arrays, each contiguous over all nrec records so that
+// the loads of a wavefront stay coalesced whatever BITS is: as many 128-bit elements as fit, then at most one 64-bit, one
+// 32-bit and one 16-bit element, then a tail of BITS % 16 bits per record, bit-packed over the records and followed by a
+// 4-byte pad (reference sm120/moe.py:36-49, sm120/nqmoe.cu:17-20). SubArrays is that layout as a compile-time table: for
+// every piece its width, the bit position it fills inside the record, and the bytes per record that all earlier sub-arrays
+// take (so piece i of record r starts at byte nrec * before[i] + r * width[i] / 8 of the plane).
+struct SubArrays { int n; int width[8]; int pos[8]; int before[8]; int tail, tail_pos, tail_before; };
+constexpr SubArrays sub_arrays(int bits)
+{
+    SubArrays L{};
+    int pos = 0;
+    for (int w = 128; w >= 16; w >>= 1)
+        while (bits - pos >= w)                                  // several 128-bit elements, at most one of each smaller width
+        {
+            L.width[L.n] = w; L.pos[L.n] = pos; L.before[L.n] = pos / 8; ++L.n;
+            pos += w;
+        }
+    L.tail = bits - pos; L.tail_pos = pos; L.tail_before = pos / 8;
+    return L;
+}
+
+template <int... Is, class F> __device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, Is...>) { (f(CodeTag<Is>{}), ...); }
+template <int N, class F> __device__ __forceinline__ void static_for(F&& f) { static_for_impl(f, std::make_integer_sequence<int, N>{}); }
+
+// the record `rec` of a plane at p, as 32-bit words w[0 .. NW). Code 11 stores its 128-bit record as the 64-bit records of
+// plane P3 followed by those of plane P4.
 template <int CODE>
 __device__ __forceinline__ void load_record(uint32_t* w, gp_u8 p, size_t rec, size_t nrec)
 {
-    constexpr int BITS = Rec<CODE>::BITS;
     if constexpr (Pat<CODE>::SPLIT)
     {
-        const u32x2 a = ((gp_u2)p)[rec], b = ((gp_u2)(p + nrec * 8))[rec];
-        w[0] = a.x; w[1] = a.y; w[2] = b.x; w[3] = b.y;
+        const u32x2 lo = ((gp_u2)p)[rec], hi = ((gp_u2)(p + nrec * 8))[rec];
+        w[0] = lo.x; w[1] = lo.y; w[2] = hi.x; w[3] = hi.y;
     }
     else
     {
-        constexpr int n4 = BITS / 128, r1 = BITS % 128, n2 = r1 / 64, r2 = r1 % 64, n1 = r2 / 32, nh = (r2 % 32) / 16;
-        constexpr int T = BITS % 16;
-        int k = 0;
-#pragma unroll
-        for (int i = 0; i < n4; ++i)
+        static constexpr SubArrays L = sub_arrays(Rec<CODE>::BITS);
+        static_for<L.n>([&](auto tag) {
+            constexpr int i = decltype(tag)::value, W = L.width[i], at = L.pos[i] >> 5;
+            const gp_u8 q = p + nrec * (size_t)L.before[i] + rec * (size_t)(W / 8);
+            if constexpr (W == 128) { const u32x4 v = *(gp_u4)q; w[at] = v.x; w[at + 1] = v.y; w[at + 2] = v.z; w[at + 3] = v.w; }
+            else if constexpr (W == 64) { const u32x2 v = *(gp_u2)q; w[at] = v.x; w[at + 1] = v.y; }
+            else if constexpr (W == 32) w[at] = *(gp_u32)q;
+            else w[at] = *(gp_u16)q;                              // a 16-bit piece always starts a word
+        });
+        if constexpr (L.tail != 0)
         {
-            const u32x4 v = ((gp_u4)p)[rec * n4 + i];
-            w[k++] = v.x; w[k++] = v.y; w[k++] = v.z; w[k++] = v.w;
-        }
-        p += nrec * 16 * n4;
-        if constexpr (n2) { const u32x2 v = ((gp_u2)p)[rec]; w[k++] = v.x; w[k++] = v.y; p += nrec * 8; }
-        if constexpr (n1) { w[k++] = ((gp_u32)p)[rec]; p += nrec * 4; }
-        if constexpr (nh) { w[k++] = ((gp_u16)p)[rec]; p += nrec * 2; }
-        if constexpr (T)
-        {
-            const size_t b = rec * T;
-            gp_u32 q = (gp_u32)p + (b >> 5);
-            const int sh = (int)(b & 31);
-            uint32_t v;
-            if constexpr (32 % T) v = __builtin_amdgcn_alignbit(q[1], q[0], sh);   // q[1] lies inside the 4-byte pad
-            else v = q[0] >> sh;
-            v &= (1u << T) - 1u;
-            if constexpr (((BITS - T) & 31) == 16) w[k - 1] |= v << 16; else w[k++] = v;
+            // bits [rec * tail, + tail) of the bit-packed tail array; a field that can straddle two words (tail does not divide
+            // 32) takes the second word too, which for the last record is the pad
+            const size_t bit = rec * (size_t)L.tail;
+            const gp_u32 q = (gp_u32)(p + nrec * (size_t)L.tail_before) + (bit >> 5);
+            const int sh = (int)(bit & 31);
+            uint32_t v = (32 % L.tail) ? __builtin_amdgcn_alignbit(q[1], q[0], sh) : q[0] >> sh;
+            v &= (1u << L.tail) - 1u;
+            if constexpr ((L.tail_pos & 31) == 0) w[L.tail_pos >> 5] = v;       // the tail opens a word of its own,
+            else w[L.tail_pos >> 5] |= v << (L.tail_pos & 31);                 // or sits above the 16-bit piece
         }
     }
 }
 
-// stream bits [BITS, BITS + 32) of a lane = first word of the next lane of its ring (tail-biting)
+// A lane's stream continues, after the BITS bits of its own record, with the record of the next lane of its ring (the rings
+// are tail-biting): the windows of the last steps reach at most 32 bits into it, so its first word nb is spliced in at bit
+// BITS and the word after that cleared. w holds NW + 2 words.
 template <int BITS, int NW>
 __device__ __forceinline__ void ext_words(uint32_t* w, uint32_t nb)
 {
-    constexpr int T = BITS % 32;
-    if constexpr (T == 0) { w[NW] = nb; w[NW + 1] = 0; }
+    constexpr int at = BITS >> 5, s = BITS & 31;
+    if constexpr (s == 0) w[at] = nb;
     else
     {
-        w[NW - 1] = (w[NW - 1] & ((1u << T) - 1u)) | (nb << T);
-        w[NW] = nb >> (32 - T);
-        w[NW + 1] = 0;
+        w[at] = (w[at] & ((1u << s) - 1u)) | (nb << s);
+        w[at + 1] = nb >> (32 - s);
     }
+    w[NW + 1] = 0;
 }
 
 // ---- hash -----------------------------------------------------------------------------------------------------------
@@ -228,7 +252,6 @@ __device__ __forceinline__ uint32_t weight_pair(const uint32_t* wb, const uint32
 //   [0] level 0/2/3/4  [1..4] gate|up base, residual plane, block words, flags (mask mode, 0 = dense)  [5..8] down  [9] sign/scale vector
 //   [10],[11] residual window code of gate|up, down  [12],[13] sign-variant planes  [14..17] low-rank plane (buffers, ranks)
 //   [18] in_had_down (0 / 128 / 512)  [19] base window codes, gate|up | down << 8 (0 or 1)
-template <int C> struct CodeTag { static constexpr int value = C; };
 typedef const NQ_GLOBAL uint64_t* gp_u64;
 struct Planes { gp_u4 base; gp_u8 res; gp_u32 dw; gp_u8 var; gp_u64 flags; int code; int bcode; };
 

@@ -1,12 +1,14 @@
 // Decode salience export: sal[e] += sum over the picks (t, k) of expert e of (rsf * w[t][k])^2 * |x[t]|^2, a running fp64 sum per
 // expert on the device, every touched entry mirrored to host-mapped memory (what the level scheduler's predictor reads next to
-// the routing hit counters). One workgroup per call, at most 8 tokens x 8 picks, no host synchronisation, static pointers.
+// the routing hit counters; reference sm120/nqsal.cu:19-78, called at sm120/serve/nq_vllm.py:558,572). At most 8 tokens of 8
+// picks per call, no host synchronisation, static pointers, so the call can sit in a captured decode step.
 //
-// The fp32 arithmetic follows the reference kernel's order (sm120/nqsal.cu:20-60) so that the exported numbers are the same
-// bits: 256 threads, thread tid takes elements 8 i .. 8 i + 7 for i = tid, tid + 256, ... (or single elements i = tid, tid + 256,
-// ... when H is not a multiple of 8 or the row is not 16-byte aligned), fused multiply-adds in that order, a butterfly over
-// groups of 32 threads (offsets 16, 8, 4, 2, 1), then the eight group sums added in order. A wavefront holds two such groups;
-// the butterfly offsets stay below 32, so each half reduces on its own.
+// Built for 64-wide wavefronts: one workgroup of eight wavefronts, wavefront t owns token t. Its lanes walk the row in 16-byte
+// steps (eight fp16 / bf16 values, or four fp32 values rounded through fp16) with two independent fp32 accumulators, the 64
+// lane sums meet in a butterfly of lane exchanges, and nothing but the eight norms crosses wavefronts (through LDS). The picks
+// are then the lanes of wavefront 0: a ballot loop groups the picks of one expert, their fp64 terms are added in pick order
+// and the group's first lane updates the accumulator once (calls on one layer are stream-ordered, so no atomics). The squared
+// norm is an fp32 sum (about 1e-6 relative at H = 6144); weights pass through fp16 as the caller's cast would leave them.
 #include "nq_host.hpp"
 
 namespace nq {
@@ -18,75 +20,87 @@ struct SalArgs
     float rsf; double* acc; double* host;
 };
 
-__device__ __forceinline__ float bf16_bits_to_f(uint16_t b) { return __builtin_bit_cast(float, (uint32_t)b << 16); }
-__device__ __forceinline__ float elem_f(const void* p, int64_t i, int dt)
+__device__ __forceinline__ float sal_bf16(uint32_t b) { return __builtin_bit_cast(float, b << 16); }
+__device__ __forceinline__ float sal_elem(const void* p, int64_t i, int dt)
 {
     if (dt == 0) return (float)((const _Float16*)p)[i];
-    if (dt == 1) return bf16_bits_to_f(((const uint16_t*)p)[i]);
+    if (dt == 1) return sal_bf16(((const uint16_t*)p)[i]);
     return (float)(_Float16)((const float*)p)[i];
 }
-
-__global__ void __launch_bounds__(256) nq_sal_k(SalArgs a)
+// squares of the two 16-bit values of a word, added to s
+__device__ __forceinline__ float sal_sq2(uint32_t u, int dt, float s)
 {
-    __shared__ float red[8][8];                  // [token][group of 32 threads]
-    __shared__ float xn[8];
-    __shared__ int se[64];
-    __shared__ double sv[64];
-    const int tid = threadIdx.x, sub = tid & 31, grp = tid >> 5;
-    const int esz = a.x_dtype == 2 ? 4 : 2;
-    for (int t = 0; t < a.T; ++t)
+    const float lo = dt == 0 ? (float)__builtin_bit_cast(_Float16, (uint16_t)u) : sal_bf16(u & 0xFFFFu);
+    const float hi = dt == 0 ? (float)__builtin_bit_cast(_Float16, (uint16_t)(u >> 16)) : sal_bf16(u >> 16);
+    return __builtin_fmaf(hi, hi, __builtin_fmaf(lo, lo, s));
+}
+
+__global__ void __launch_bounds__(512) nq_sal_k(SalArgs a)
+{
+    __shared__ float norm2[8];
+    const int lane = threadIdx.x & 63, t = threadIdx.x >> 6;
+    if (t < a.T)
     {
+        const int esz = a.x_dtype == 2 ? 4 : 2;
         const char* row = (const char*)a.x + (int64_t)t * a.sx * esz;
-        float s = 0.f;
-        // an fp32 row stands for the contiguous fp16 copy a caller would make of it, which is always aligned
-        const bool by8 = (a.H & 7) == 0 && (a.x_dtype == 2 || ((uintptr_t)row & 15) == 0);
-        if (by8 && a.x_dtype != 2)
+        const int per = 16 / esz;                                  // values per 16-byte step
+        float s0 = 0.f, s1 = 0.f;
+        int done = 0;
+        if (((uintptr_t)row & 15) == 0)
         {
-            for (int i = tid; i < a.H / 8; i += 256)
+            const int nv = a.H / per;
+            for (int i = lane; i < nv; i += 128)
             {
                 const uint4 u = ((const uint4*)row)[i];
-                const uint32_t q[4] = {u.x, u.y, u.z, u.w};
-#pragma unroll
-                for (int j = 0; j < 8; ++j)
+                const bool two = i + 64 < nv;
+                const uint4 v = two ? ((const uint4*)row)[i + 64] : uint4{0u, 0u, 0u, 0u};       // zero bits are 0.0 in all three types
+                if (a.x_dtype == 2)
                 {
-                    const uint16_t b = (uint16_t)(q[j >> 1] >> (16 * (j & 1)));
-                    const float f = a.x_dtype == 0 ? (float)__builtin_bit_cast(_Float16, b) : bf16_bits_to_f(b);
-                    s = __builtin_fmaf(f, f, s);
+                    const float f[8] = {__builtin_bit_cast(float, u.x), __builtin_bit_cast(float, u.y), __builtin_bit_cast(float, u.z), __builtin_bit_cast(float, u.w),
+                                        __builtin_bit_cast(float, v.x), __builtin_bit_cast(float, v.y), __builtin_bit_cast(float, v.z), __builtin_bit_cast(float, v.w)};
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                    {
+                        const float p = (float)(_Float16)f[j], q = (float)(_Float16)f[4 + j];
+                        s0 = __builtin_fmaf(p, p, s0); s1 = __builtin_fmaf(q, q, s1);
+                    }
+                }
+                else
+                {
+                    s0 = sal_sq2(u.x, a.x_dtype, s0); s0 = sal_sq2(u.y, a.x_dtype, s0); s0 = sal_sq2(u.z, a.x_dtype, s0); s0 = sal_sq2(u.w, a.x_dtype, s0);
+                    s1 = sal_sq2(v.x, a.x_dtype, s1); s1 = sal_sq2(v.y, a.x_dtype, s1); s1 = sal_sq2(v.z, a.x_dtype, s1); s1 = sal_sq2(v.w, a.x_dtype, s1);
                 }
             }
+            done = nv * per;
         }
-        else if (by8)
-        {
-            for (int i = tid; i < a.H / 8; i += 256)
+        for (int i = done + lane; i < a.H; i += 64) { const float f = sal_elem(row, i, a.x_dtype); s0 = __builtin_fmaf(f, f, s0); }   // rest, or a row off 16-byte alignment
+        float s = s0 + s1;
 #pragma unroll
-                for (int j = 0; j < 8; ++j) { const float f = elem_f(row, (int64_t)i * 8 + j, 2); s = __builtin_fmaf(f, f, s); }
-        }
-        else
-            for (int i = tid; i < a.H; i += 256) { const float f = elem_f(row, i, a.x_dtype); s = __builtin_fmaf(f, f, s); }
-#pragma unroll
-        for (int o = 16; o; o >>= 1) s += __shfl_xor(s, o);
-        if (sub == 0) red[t][grp] = s;
+        for (int m = 32; m; m >>= 1) s += __shfl_xor(s, m);
+        if (lane == 0) norm2[t] = s;
     }
     __syncthreads();
-    if (tid < a.T) { float s = 0.f; for (int j = 0; j < 8; ++j) s += red[tid][j]; xn[tid] = s; }
-    __syncthreads();
-    const int n = a.T * a.K;
-    if (tid < n)
+    if (t != 0) return;
+    const int n = a.T * a.K;                                        // <= 64: one pick per lane
+    long long e = -1; double term = 0.0;
+    if (lane < n)
     {
-        float ww = (float)(_Float16)elem_f(a.w, tid, a.w_dtype);
-        const int64_t e = a.ids_dtype == 0 ? ((const int64_t*)a.ids)[tid] : (int64_t)((const int32_t*)a.ids)[tid];
-        se[tid] = (ww != 0.f && e >= 0 && e < a.E) ? (int)e : -1;        // weight 0 or an id outside the table: skipped, as the hit counters do
-        ww *= a.rsf;
-        sv[tid] = (double)(ww * ww * xn[tid / a.K]);
+        const float wf = (float)(_Float16)sal_elem(a.w, lane, a.w_dtype);
+        e = a.ids_dtype == 0 ? (long long)((const int64_t*)a.ids)[lane] : (long long)((const int32_t*)a.ids)[lane];
+        if (wf == 0.f || e < 0 || e >= a.E) e = -1;                 // weight 0 or an id outside the table: skipped, as the hit counters do
+        const double ww = (double)(wf * a.rsf);
+        term = ww * ww * (double)norm2[lane / a.K];
     }
-    __syncthreads();
-    if (tid < n && se[tid] >= 0)
+    unsigned long long rem = __ballot(e >= 0);
+    while (rem)
     {
-        // the first pick of an expert adds all of that expert's picks, in pick order, and writes once
-        const int e = se[tid]; double tot = 0.0; bool first = true;
-        for (int j = 0; j < n; ++j)
-            if (se[j] == e) { if (j < tid) { first = false; break; } tot += sv[j]; }
-        if (first) { const double v = a.acc[e] + tot; a.acc[e] = v; a.host[e] = v; }
+        const int first = __ffsll((long long)rem) - 1;
+        const long long ev = __shfl(e, first);
+        const unsigned long long same = __ballot(e == ev);
+        double tot = 0.0;
+        for (unsigned long long m = same; m; m &= m - 1) tot += __shfl(term, __ffsll((long long)m) - 1);     // in pick order
+        if (lane == first) { const double v = a.acc[ev] + tot; a.acc[ev] = v; a.host[ev] = v; }
+        rem &= ~same;
     }
 }
 
@@ -94,7 +108,7 @@ int launch_sal(const void* x, int x_dtype, int64_t sx, const void* w, int w_dtyp
                int E, float rsf, double* acc, double* host, hipStream_t st)
 {
     SalArgs a{x, sx, w, ids, T, H, K, E, x_dtype, w_dtype, ids_dtype, rsf, acc, host};
-    nq_sal_k<<<1, 256, 0, st>>>(a);
+    nq_sal_k<<<1, 512, 0, st>>>(a);
     NQ_LAUNCH_CHECK("nq_sal");
     return 0;
 }

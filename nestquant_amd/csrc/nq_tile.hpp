@@ -65,9 +65,6 @@ __device__ __forceinline__ int bop_index(int c)
     return (mm * 4 + kg) * 8 + 2 * i + hi;
 }
 
-template <int... Is, class F> __device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, Is...>) { (f(CodeTag<Is>{}), ...); }
-template <int N, class F> __device__ __forceinline__ void static_for(F&& f) { static_for_impl(f, std::make_integer_sequence<int, N>{}); }
-
 // A operand of MFMA (MM, RHO): rows g + 8 RHO, columns of t = 2 MM and 2 MM + 1
 template <bool RES, int CODE, int MM, int RHO, int BK = 0>
 __device__ __forceinline__ half8_t a_operand(const uint32_t* wb, const uint32_t* wr, const FoldK& k)

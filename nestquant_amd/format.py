@@ -24,21 +24,41 @@ def popc(m):
     return bin(m).count("1")
 
 
+def _step_bits(KA, MASK):
+    """bits carried by each of the 16 steps of a pattern period"""
+    return [KA + (MASK >> r & 1) for r in range(16)]
+
+
 def rbits(rk):
-    ka, mask = RKP[rk]
-    return 4 * (16 * ka + popc(mask))
+    """bits of one lane record: 64 steps = four periods of the code's window pattern"""
+    return 4 * sum(_step_bits(*RKP[rk]))
 
 
 def step_off(p, KA, MASK):
-    per = [sum(KA + ((MASK >> i) & 1) for i in range(r)) for r in range(16)]
+    """bit offset of step p in a stream with window pattern (KA, MASK): whole periods before it plus the steps of its own"""
     p = torch.as_tensor(p)
-    return (p >> 4) * (16 * KA + popc(MASK)) + torch.tensor(per, device=p.device)[p & 15]
+    bits = torch.tensor([0] + _step_bits(KA, MASK), device=p.device).cumsum(0)
+    return (p >> 4) * bits[16] + bits[p & 15]
+
+
+def sub_arrays(bits):
+    """The sub-array layout of a plane whose records hold `bits` bits (reference sm120/moe.py:36-49, sm120/nqmoe.cu:17-20):
+    [(width, pos)] for the whole elements, in storage order -- as many 128-bit ones as fit, then at most one of 64, 32 and 16
+    bits, each sub-array contiguous over all records -- and the tail (bits % 16 bits per record, bit-packed over the records
+    and followed by 4 bytes of padding) as (tail width, its position in the record). pos = first bit of the record the piece
+    holds. The kernels walk the same table (SubArrays in csrc/nq_decode.hpp)."""
+    pieces, pos = [], 0
+    for width in (128, 64, 32, 16):
+        while bits - pos >= width:
+            pieces.append((width, pos)); pos += width
+    return pieces, (bits - pos, pos)
 
 
 def split_bits(bits):
     """(#uint4, uint2?, uint?, ushort?, tail bits) of a record of `bits` bits"""
-    rem = bits % 128
-    return bits // 128, rem // 64, (rem % 64) // 32, (rem % 32) // 16, bits % 16
+    pieces, (tail, _) = sub_arrays(bits)
+    count = lambda w: sum(1 for width, _ in pieces if width == w)
+    return count(128), count(64), count(32), count(16), tail
 
 
 def proj_sizes(N, K, nm=None, rk=0, bk=0):
@@ -53,72 +73,53 @@ def proj_sizes(N, K, nm=None, rk=0, bk=0):
 
 
 def make_flags(S, C, nm, gen, grp=8):
-    """nm flagged chunks per strip, identical across each group of `grp` strips (reference sm120/moe.py:28-34):
-    (int64 [S], bit c = chunk c is refined; bool [S, C])"""
+    """nm flagged chunks per strip, identical across each group of `grp` strips (reference sm120/moe.py:28-34; the draw is the
+    reference's, one uniform per (group, chunk), so equal seeds flag equal chunks): the nm chunks of a group whose draws rank
+    lowest. -> (int64 [S], bit c = chunk c is refined; bool [S, C])"""
     dev = gen.device
-    ng = (S + grp - 1) // grp
-    idx = torch.rand(ng, C, generator=gen, device=dev).argsort(1)[:, :nm]
-    fl = torch.zeros(ng, C, dtype=torch.bool, device=dev); fl.scatter_(1, idx, True)
-    fl = fl.repeat_interleave(grp, 0)[:S]
+    draws = torch.rand((S + grp - 1) // grp, C, generator=gen, device=dev)
+    rank = draws.argsort(1).argsort(1)                            # rank of every chunk's draw within its group
+    fl = (rank < nm)[torch.arange(S, device=dev) // grp]
     return (fl.long() << torch.arange(C, device=dev)).sum(1), fl
 
 
-def _bytes_le(t, nb):
-    return torch.stack([(t >> (8 * i)) & 255 for i in range(nb)], -1).to(torch.uint8).reshape(-1)
+def _record_bits(w, bits):
+    """w [nrec, NW] (uint32 values) -> uint8 [nrec, bits], bit i of a record = bit i % 32 of its word i // 32"""
+    sh = torch.arange(32, device=w.device)
+    return ((w[:, :, None] >> sh) & 1).to(torch.uint8).reshape(w.shape[0], -1)[:, :bits]
 
 
 def pack_words(w, bits):
-    """w [nrec, NW] int64 (uint32 values) -> int32 tensor in the sub-array layout uint4 x n4 | uint2 | uint | ushort |
-    tail (bits % 16 bits per record, bit-packed over records, + 4 bytes of padding)"""
-    n4, n2, n1, nh, T = split_bits(bits)
-    parts, k = [], 0
-    if n4:
-        parts.append(_bytes_le(w[:, :4 * n4], 4)); k = 4 * n4
-    if n2:
-        parts.append(_bytes_le(w[:, k:k + 2], 4)); k += 2
-    if n1:
-        parts.append(_bytes_le(w[:, k], 4)); k += 1
-    if nh:
-        parts.append(_bytes_le(w[:, k] & 0xFFFF, 2))
-    if T:
-        a = bits - T
-        t = (w[:, a // 32] >> (a % 32)) & ((1 << T) - 1)
-        b = ((t[:, None] >> torch.arange(T, device=w.device)) & 1).reshape(-1)
-        b = torch.cat([b, torch.zeros(32, dtype=b.dtype, device=w.device)])
-        b = b[: b.numel() // 8 * 8].view(-1, 8)
-        parts.append((b << torch.arange(8, device=w.device)).sum(1).to(torch.uint8))
-    return torch.cat(parts).view(torch.int32)
+    """w [nrec, NW] int64 (uint32 values) -> int32 tensor in the sub-array layout of sub_arrays(bits). The plane is one long
+    bit string: for every piece of the layout the matching columns of the record-by-bit matrix, record after record, then the
+    tail columns, then zero bits up to a whole 32-bit word (a whole extra word after a tail)."""
+    nrec = w.shape[0]
+    B = _record_bits(w, bits)
+    pieces, (tail, tpos) = sub_arrays(bits)
+    runs = [B[:, pos:pos + width].reshape(-1) for width, pos in pieces]
+    if tail:
+        runs.append(B[:, tpos:].reshape(-1))
+        fill = (-nrec * tail) % 8 + 32                            # to the byte boundary, then the 4-byte pad
+        runs.append(torch.zeros(fill, dtype=torch.uint8, device=w.device))
+    flat = torch.cat(runs).view(-1, 8)
+    by = (flat << torch.arange(8, dtype=torch.uint8, device=w.device)).sum(1, dtype=torch.uint8)
+    return by.view(torch.int32)
 
 
 def unpack_words(t, nrec, bits):
-    """inverse of pack_words -> [nrec, NW] int64 (uint32 values)"""
-    n4, n2, n1, nh, T = split_bits(bits)
+    """inverse of pack_words -> [nrec, NW] int64 (uint32 values): the plane's bit string cut back into the columns of the
+    record-by-bit matrix, piece by piece"""
     dev = t.device
-    b = t.contiguous().view(torch.uint8).long()
-    w = torch.zeros(nrec, (bits + 31) // 32, dtype=torch.int64, device=dev)
-    pos = 0
-
-    def take(nwords, nb):
-        nonlocal pos
-        x = b[pos:pos + nrec * nwords * nb].view(nrec, nwords, nb)
-        pos += nrec * nwords * nb
-        return (x << (8 * torch.arange(nb, device=dev))).sum(-1)
-
-    k = 0
-    if n4:
-        w[:, :4 * n4] = take(4 * n4, 4); k = 4 * n4
-    if n2:
-        w[:, k:k + 2] = take(2, 4); k += 2
-    if n1:
-        w[:, k] = take(1, 4)[:, 0]; k += 1
-    if nh:
-        w[:, k] = take(1, 2)[:, 0]
-    if T:
-        a = bits - T
-        bb = b[pos:pos + (nrec * T + 7) // 8]
-        bit = ((bb[:, None] >> torch.arange(8, device=dev)) & 1).reshape(-1)[: nrec * T].view(nrec, T)
-        w[:, a // 32] |= (bit << torch.arange(T, device=dev)).sum(-1) << (a % 32)
-    return w
+    by = t.contiguous().view(torch.uint8)
+    flat = ((by[:, None] >> torch.arange(8, dtype=torch.uint8, device=dev)) & 1).reshape(-1)
+    nw = (bits + 31) // 32
+    B = torch.zeros(nrec, nw * 32, dtype=torch.uint8, device=dev)
+    pieces, (tail, tpos) = sub_arrays(bits)
+    at = 0
+    for width, pos in pieces + ([(tail, tpos)] if tail else []):
+        B[:, pos:pos + width] = flat[at:at + nrec * width].view(nrec, width)
+        at += nrec * width
+    return (B.view(nrec, nw, 32).long() << torch.arange(32, device=dev)).sum(-1)
 
 
 def lane_words_from_rings(raw, bits, G=4):

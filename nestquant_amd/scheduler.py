@@ -1,22 +1,73 @@
 """Level policy: which experts are served at level 4. Fixed experts always are; a floating set follows decayed routing counts.
 
-Host-side mirror of the reference's streaming/scheduler.py with its 'ema' rule (:62-118,160-189): the same constructor
-arguments, `step(counts, ntok) -> (ups, downs)`, the executor's callbacks `landed / released / failed`, `kv_pressure(n)`
-and `level()`, and the same decisions on the same counts (pinned by a trace of the reference's class,
-tests/golden/sched_trace.json). Pure policy on the CPU: it sees the per-step routing counts (the kernels' `hits` export)
-and returns level ops for executor.RankExecutor.apply. The learned predictors of the reference (its default,
-gbdt_predictor*.py over LightGBM models) and its C++ host loop are not part of this build: any predictor other than
-'ema' is refused.
+Takes the place of the reference's streaming/scheduler.py with its 'ema' rule (:62-118,160-189): the same constructor
+arguments, `step(counts, ntok) -> (ups, downs)`, the executor's callbacks `landed / released / failed / cancelled`,
+`kv_pressure(n)` and `level()`, the arrays its callers read (`want`, `state`, `score`, `hold`, `fixed`, `pin`, `budget`,
+`tok`, `stats`, `li`), and the same decisions on the same counts: tests/golden/sched_trace.json holds every step's ops, the
+number of level-4 experts and the byte budget that the reference's class produced on seeded counts with executor feedback.
+Pure policy on the CPU: it sees the per-step routing counts (the kernels' `hits` export) and returns level ops for
+executor.RankExecutor.apply. The learned predictors of the reference (its default, gbdt_predictor*.py over LightGBM models)
+and its C++ host loop are not part of this build: any predictor other than 'ema' is refused.
 
-Rule: score = counts decayed with a half-life of `half_life` tokens; every `refresh` tokens the floating target of a layer
-that has seen counts becomes its `n_float` best non-fixed experts (a layer without counts keeps `floating_default`);
-level-4 experts outside the target are downgraded at once; wanted level-2 experts are upgraded best score first while the
-byte budget (cap_GBps at tok_per_s, at most burst_tokens of credit) and the slot pool allow, the rest wait; a step that
-routes to more than big_frac of a layer's experts starts no upgrade; a failed read is not retried before retry_tokens.
+The rule, and the piece of this module that holds each part of it:
+  DecayedCounts   score = routing counts decayed with a half-life of `half_life` tokens;
+  FloatingSet     every `refresh` tokens the floating target of a layer that has seen counts becomes its `n_float` best
+                  non-fixed experts (a layer without counts keeps `floating_default`);
+  ByteBudget      upgrades cost one record each out of a budget that fills with cap_GBps at tok_per_s, holding at most
+                  burst_tokens of credit;
+  Scheduler.step  level-4 experts outside the target are downgraded at once; wanted level-2 experts are upgraded best score
+                  first while the budget and the slot pool allow, the rest wait; a step that routes to more than big_frac of
+                  a layer's experts starts no upgrade; a failed read is not retried before retry_tokens.
 """
 import numpy as np
 
 IDLE, RISING, UP, FALLING = 0, 1, 2, 3        # floating expert: level 2 / upgrade in flight / level 4 / downgrade in flight
+# what an executor callback does to an expert's state: callback -> (state it applies to, state it leaves)
+ON_FEEDBACK = {"landed": (RISING, UP), "released": (FALLING, IDLE), "failed": (RISING, IDLE)}
+
+
+class ByteBudget:
+    """bytes of upgrades that may start: fills per token, is capped at a burst, is spent per record"""
+
+    def __init__(s, per_token, burst_tokens):
+        s.per_token, s.cap, s.level = per_token, per_token * burst_tokens, 0.0
+
+    def refill(s, ntok):
+        s.level = min(s.cap, s.level + s.per_token * ntok)
+
+    def records(s, rec_bytes):
+        return int(s.level // rec_bytes)
+
+    def spend(s, nbytes):
+        s.level -= nbytes
+
+
+class DecayedCounts:
+    """exponentially decayed routing counts, one per (layer, expert)"""
+
+    def __init__(s, shape, half_life):
+        s.keep = 0.5 ** (1 / half_life)
+        s.value = np.zeros(shape)
+
+    def add(s, counts, ntok):
+        s.value = s.value * s.keep ** ntok + counts
+
+
+class FloatingSet:
+    """the floating experts a layer wants at level 4: the default until the layer has counts, then its best n by score"""
+
+    def __init__(s, fixed, default_of, n):
+        s.n = n
+        s.mask = np.zeros_like(fixed)
+        for i, default in enumerate(default_of):
+            s.mask[i, [e for e in default if not fixed[i, e]][:n]] = True
+
+    def refresh(s, score, fixed):
+        ranked = np.where(fixed, -np.inf, score)
+        # position of every expert in its layer's order by falling score, equal scores by rising index
+        place = np.argsort(np.argsort(-ranked, 1, kind="stable"), 1, kind="stable")
+        seen = score.sum(1) > 0
+        s.mask[seen] = (place < s.n)[seen]
 
 
 class Scheduler:
@@ -25,102 +76,102 @@ class Scheduler:
         if predictor not in (None, "ema"):
             raise ValueError(f"predictor {predictor!r}: only the 'ema' rule is built")
         s.layers = list(layers)
-        s.li = {L: i for i, L in enumerate(s.layers)}
-        nl = len(s.layers)
-        s.NE, s.nf, s.R, s.rb, s.big, s.slots = NE, n_float, refresh, rec_bytes, big_frac, slots
-        s.a = 0.5 ** (1 / half_life)
-        s.fixed = np.zeros((nl, NE), bool)
-        s.want = np.zeros((nl, NE), bool)
-        for L in s.layers:
-            i = s.li[L]
-            s.fixed[i, list(fixed[L])] = True
-            s.want[i, [e for e in floating_default[L] if not s.fixed[i, e]][:n_float]] = True
-        s.score = np.zeros((nl, NE))
-        s.state = np.zeros((nl, NE), np.int8)
-        s.hold = np.zeros((nl, NE))                     # token count before which a failed read is not retried
-        s.per_tok = cap_GBps * 1e9 / tok_per_s
-        s.cap = s.per_tok * burst_tokens
-        s.budget = 0.0
+        s.li = dict(zip(s.layers, range(len(s.layers))))          # layer id -> row of the arrays below
+        shape = (len(s.layers), NE)
+        s.NE, s.rec_bytes, s.big_frac, s.slots, s.refresh_every = NE, rec_bytes, big_frac, slots, refresh
+        s.fixed = np.zeros(shape, bool)
+        for row, L in enumerate(s.layers):
+            s.fixed[row, sorted(fixed[L])] = True
+        s.counts = DecayedCounts(shape, half_life)
+        s.floating = FloatingSet(s.fixed, [floating_default[L] for L in s.layers], n_float)
+        s.bytes = ByteBudget(cap_GBps * 1e9 / tok_per_s, burst_tokens)
+        s.state = np.zeros(shape, np.int8)
+        s.hold = np.zeros(shape)                        # token count before which a failed read is not retried
         s.retry = refresh if retry_tokens is None else retry_tokens
         s.tok, s.next_refresh = 0, refresh
         s.pin = None                                    # optional bool [layers, NE]: floating experts kept wanted while set
         s.predictor_name = "ema"
         s.stats = dict(ups=0, downs=0, deferred_steps=0, big_steps=0, bytes=0)
 
-    def _refresh(s):
-        seen = s.score.sum(1) > 0
-        ranked = np.argsort(-np.where(s.fixed, -np.inf, s.score), 1, kind="stable")[:, :s.nf]
-        target = np.zeros_like(s.want)
-        np.put_along_axis(target, ranked, True, 1)
-        s.want[seen] = target[seen]
+    # arrays and figures callers read under the reference's names
+    want = property(lambda s: s.floating.mask, lambda s, v: setattr(s.floating, "mask", v))
+    score = property(lambda s: s.counts.value, lambda s, v: setattr(s.counts, "value", v))
+    budget = property(lambda s: s.bytes.level, lambda s, v: setattr(s.bytes, "level", v))
+
+    def _keys(s, flat):
+        """flat indices into [layers, NE] -> [(L, E)]"""
+        li, e = np.unravel_index(flat, s.state.shape)
+        return [(s.layers[i], int(x)) for i, x in zip(li, e)]
+
+    def _to_falling(s, flat):
+        s.state.flat[flat] = FALLING
+        s.stats["downs"] += len(flat)
+        return s._keys(flat)
+
+    def _start_upgrades(s, hits):
+        """wanted level-2 experts, best score first, as far as budget and slots reach"""
+        ready = np.flatnonzero((s.state == IDLE) & s.floating.mask & (s.hold <= s.tok))
+        if ((hits > 0).sum(1) > s.big_frac * s.NE).any():
+            s.stats["big_steps"] += 1                   # a step that touches most of a layer (a prefill) says nothing about locality
+            return []
+        if not len(ready):
+            return []
+        room = s.bytes.records(s.rec_bytes)
+        if s.slots is not None:                         # slots are held by experts in flight, landed and draining
+            in_use = int(np.count_nonzero(s.state != IDLE))
+            room = min(room, max(s.slots - in_use, 0))
+        if len(ready) > room:
+            s.stats["deferred_steps"] += 1
+        go = ready[np.argsort(-s.counts.value.flat[ready], kind="stable")[:room]]
+        s.state.flat[go] = RISING
+        s.bytes.spend(len(go) * s.rec_bytes)
+        s.stats["bytes"] += len(go) * s.rec_bytes
+        s.stats["ups"] += len(go)
+        return s._keys(go)
 
     def step(s, counts, ntok=1, token_ids=None, new_request=False, sal=None):
         """counts [len(layers), NE]: routing hits of this model step (ntok tokens) -> (ups, downs) as lists of (L, E).
         token_ids, new_request and sal are accepted for the reference's call sites; the 'ema' rule does not use them."""
-        c = np.asarray(counts, np.float64)
-        s.score = s.score * s.a ** ntok + c
+        hits = np.asarray(counts, np.float64)
+        s.counts.add(hits, ntok)
         s.tok += ntok
-        s.budget = min(s.cap, s.budget + s.per_tok * ntok)
+        s.bytes.refill(ntok)
         if s.tok >= s.next_refresh:
-            s.next_refresh += s.R
-            s._refresh()
+            s.next_refresh += s.refresh_every
+            s.floating.refresh(s.counts.value, s.fixed)
         if s.pin is not None:
-            s.want |= s.pin & ~s.fixed
-        downs = [(s.layers[i], int(e)) for i, e in zip(*np.nonzero((s.state == UP) & ~s.want))]
-        for L, e in downs:
-            s.state[s.li[L], e] = FALLING
-        ups = []
-        ready = (s.state == IDLE) & s.want & (s.hold <= s.tok)
-        if ((c > 0).sum(1) > s.big * s.NE).any():
-            s.stats["big_steps"] += 1
-        elif ready.any():
-            i, e = np.nonzero(ready)
-            order = np.argsort(-s.score[i, e], kind="stable")
-            n = int(s.budget // s.rb)
-            if s.slots is not None:                     # slots are held by experts in flight, landed and draining
-                n = max(0, min(n, s.slots - int((s.state > IDLE).sum())))
-            if len(order) > n:
-                s.stats["deferred_steps"] += 1
-            for k in order[:n]:
-                ups.append((s.layers[i[k]], int(e[k])))
-                s.state[i[k], e[k]] = RISING
-            s.budget -= len(ups) * s.rb
-            s.stats["bytes"] += len(ups) * s.rb
-        s.stats["ups"] += len(ups)
-        s.stats["downs"] += len(downs)
-        return ups, downs
+            s.floating.mask |= s.pin & ~s.fixed
+        downs = s._to_falling(np.flatnonzero((s.state == UP) & ~s.floating.mask))
+        return s._start_upgrades(hits), downs
 
     # executor feedback
+    def _feedback(s, what, L, e):
+        i = s.li[L]
+        before, after = ON_FEEDBACK[what]
+        if s.state[i, e] != before:
+            return False
+        s.state[i, e] = after
+        return True
+
     def landed(s, L, e):
-        if s.state[s.li[L], e] == RISING:
-            s.state[s.li[L], e] = UP
+        s._feedback("landed", L, e)
 
     def released(s, L, e):
-        if s.state[s.li[L], e] == FALLING:
-            s.state[s.li[L], e] = IDLE
+        s._feedback("released", L, e)
 
     def failed(s, L, e, read_error=False):
-        i = s.li[L]
-        if s.state[i, e] == RISING:
-            s.state[i, e] = IDLE
-            if read_error:
-                s.hold[i, e] = s.tok + s.retry
-                s.stats["read_errors"] = s.stats.get("read_errors", 0) + 1
+        if s._feedback("failed", L, e) and read_error:
+            s.hold[s.li[L], e] = s.tok + s.retry
+            s.stats["read_errors"] = s.stats.get("read_errors", 0) + 1
 
     cancelled = failed
 
     def kv_pressure(s, n):
         """downgrade the n lowest-score level-4 floating experts now; they stay unwanted until a refresh selects them again"""
-        i, e = np.nonzero(s.state == UP)
-        if not len(i):
-            return []
-        low = np.argsort(s.score[i, e], kind="stable")[:n]
-        downs = [(s.layers[i[k]], int(e[k])) for k in low]
-        for L, x in downs:
-            s.state[s.li[L], x] = FALLING
-            s.want[s.li[L], x] = False
-        s.stats["downs"] += len(downs)
-        return downs
+        up = np.flatnonzero(s.state == UP)
+        low = up[np.argsort(s.counts.value.flat[up], kind="stable")[:n]]
+        s.floating.mask.flat[low] = False
+        return s._to_falling(low)
 
     def level(s):
         """[len(layers), NE]: the level each expert is served at, as far as the scheduler knows"""

@@ -13,7 +13,7 @@ cpu_baseline leg may. It restates, in plain numpy, the algorithm of the referenc
   Hadamard-128, expert and layer math reference sm120/moe.py:168-172,196-210,344-351
   routing dedup into runs             reference sm120/nqmoe.cu:375-449
   mailbox state machine               reference sm120/nqmoe.cu:908-923, tests/test_prefill_borrow_cpu.py:36-42
-  decode salience export              reference sm120/nqsal.cu:20-60 (fp32 summation order included)
+  decode salience export              reference sm120/nqsal.cu:20-60 (the value, in float64)
 
 Two independent decoders live here on purpose: `lane_sums` (lane-local view: a lane's own record plus the first word
 of its ring neighbour) and `ring_states` (ring bit-stream view). Tests require them to agree; either alone could hide
@@ -424,57 +424,29 @@ def mailbox_apply(table, stage, seq, applied):
     return int(m.sum())
 
 
-def salience(x, w, ids, rsf, acc, E=None, by8=None):
-    """acc[e] += sum over picks (t, k) of expert e of (rsf * w[t, k])^2 * |x[t]|^2 (reference sm120/nqsal.cu:20-60), in place
-    on the float64 array `acc`; returns the indices written. x [T, H] float16 (or float32 holding bf16 / fp16 values), w
-    [T, K] float16, ids [T, K] integers. The fp32 arithmetic follows the reference kernel's order: thread tid of 256 takes the
-    elements 8 i .. 8 i + 7 for i = tid, tid + 256, ... when H is a multiple of 8 (a 16-byte aligned row is assumed), else
-    single elements i = tid, tid + 256, ...; x * x is exact in fp32 for 11-bit and 8-bit significands, so the fused
-    multiply-add equals a rounded add; then a butterfly over groups of 32 threads and the 8 group sums added in order.
-    by8=False forces the single-element order (what the kernel does for a row that is not 16-byte aligned).
-    Pinned by exact known answers and the float64 closed form; the summation ORDER is restated from the reference's text
-    and no stored output of the reference's kernel exists to pin it: the last-bit agreement with that kernel is unpinned."""
+def salience(x, w, ids, rsf, acc, E=None):
+    """acc[e] += sum over picks (t, k) of expert e of (rsf * w[t, k])^2 * |x[t]|^2 (reference sm120/nqsal.cu:20-60), in place on
+    the float64 array `acc`; returns the indices written, in first-pick order. x [T, H] float16 (or float32 holding bf16 /
+    fp16 values), w [T, K] float16, ids [T, K] integers; picks with w == 0 or an id outside [0, E) are skipped.
+    This is the value the export stands for, in float64 throughout except that rsf * w is formed in fp32 as the kernels form
+    it; a kernel's fp32 norm agrees with it to fp32 rounding (tests allow 1e-5 relative) and exactly where every partial sum
+    is exact (rows of small powers of two). Pinned by exact known answers; the reference holds no stored output of its kernel."""
     x = np.asarray(x); w = np.asarray(w, np.float16); ids = np.asarray(ids)
     T, H = x.shape
     K = ids.shape[1]
     E = len(acc) if E is None else E
     assert T <= 8 and K <= 8
-    f = x.astype(np.float32)
-    xn = np.zeros(T, np.float32)
-    for t in range(T):
-        s = np.zeros(256, np.float32)
-        if H % 8 == 0 and by8 is not False:
-            nv = H // 8
-            rounds = -(-nv // 256)
-            v = np.zeros((rounds * 256, 8), np.float32); v[:nv] = f[t].reshape(nv, 8)
-            v = v.reshape(rounds, 256, 8)
-            for m in range(rounds):
-                for j in range(8):
-                    s = (s + v[m, :, j] * v[m, :, j]).astype(np.float32)
-        else:
-            rounds = -(-H // 256)
-            v = np.zeros(rounds * 256, np.float32); v[:H] = f[t]
-            v = v.reshape(rounds, 256)
-            for m in range(rounds):
-                s = (s + v[m] * v[m]).astype(np.float32)
-        lane = np.arange(256)
-        for o in (16, 8, 4, 2, 1):
-            s = (s + s[lane ^ o]).astype(np.float32)
-        tot = np.float32(0)
-        for g in range(8):
-            tot = np.float32(tot + s[32 * g])
-        xn[t] = tot
+    xn = (x.astype(np.float64) ** 2).sum(1)
     wf = w.astype(np.float32).reshape(-1)
     idf = ids.reshape(-1).astype(np.int64)
-    ww = (wf * np.float32(rsf)).astype(np.float32)
-    sv = ((ww * ww).astype(np.float32) * np.repeat(xn, K)).astype(np.float32).astype(np.float64)
+    ww = (wf * np.float32(rsf)).astype(np.float32).astype(np.float64)
+    term = ww * ww * np.repeat(xn, K)
     live = (wf != 0) & (idf >= 0) & (idf < E)
     touched = []
     for e in dict.fromkeys(idf[live].tolist()):                  # first-pick order; each expert's picks added in pick order
         tot = 0.0
         for j in np.nonzero(live & (idf == e))[0]:
-            tot += sv[j]
+            tot += term[j]
         acc[e] = acc[e] + tot
         touched.append(e)
     return touched
-

@@ -125,6 +125,33 @@ def test_refused_failed_and_cancelled_upgrades_return_their_slot():
     assert not ex.free and ex.slot_of == {(L, 5): 0}
 
 
+def test_a_failed_downgrade_keeps_its_slot_and_is_posted_again():
+    """the engine reports an op whose copies failed with t_read < 0 whatever its kind; for a downgrade the level-4 row is
+    still live and points into the slot, so the slot stays owned, the scheduler hears nothing, and the row is posted again"""
+    import pytest
+    ex, eng, mb, exs, lay = make(nslot=1)
+    log = Log()
+    ex.apply([(L, 1)], [], log)
+    eng.finish(1); ex.poll(log); mb.applied_host[1] = 1; ex.poll(log)
+    assert log.ev == [("landed", 1)] and ex.slot_of == {(L, 1): 0}
+    ex.apply([], [(L, 1)], log)
+    eng.finish(2, trd=-5.0)                                              # the row copy failed
+    ex.poll(log)
+    assert log.ev == [("landed", 1)] and ex.slot_of == {(L, 1): 0} and not ex.free and ex.n_failed == 0
+    assert list(eng.q) == [3] and eng.q[3]["kind"] == 2 and eng.q[3]["seq"] == 2 and ex.count["reposted"] == 1
+    eng.finish(3, trd=0.0); ex.poll(log); mb.applied_host[1] = 2; ex.poll(log)
+    assert log.ev[-1] == ("released", 1) and ex.free == [0] and not ex.busy()
+    # an engine that keeps failing surfaces as an error, not as a silent loop
+    ex.apply([(L, 1)], [], log)
+    eng.finish(4); ex.poll(log); mb.applied_host[1] = 3; ex.poll(log)
+    ex.apply([], [(L, 1)], log)
+    with pytest.raises(RuntimeError, match="failed to post"):
+        for tag in range(5, 12):
+            eng.finish(tag, trd=-5.0)
+            ex.poll(log)
+    assert ex.slot_of == {(L, 1): 0}
+
+
 def test_shadow_posts_level_2_rows_and_io_stats_reports_intervals():
     ex, eng, mb, exs, lay = make(shadow=True)
     ex.apply([(L, 1)], [])

@@ -1,5 +1,6 @@
-"""Decode salience export (sal[e] += (rsf w)^2 |x|^2 per pick): the oracle against exact known answers and the float64 closed
-form on the CPU; the HIP kernel against the oracle, bit for bit, on the GPU."""
+"""Decode salience export (sal[e] += (rsf w)^2 |x|^2 per pick): the oracle against exact known answers and an independent
+float64 closed form on the CPU; the HIP kernel against the oracle on the GPU -- exactly where every partial sum is exact (rows
+of small powers of two), to fp32 rounding of the squared norm (1e-5 relative) otherwise."""
 import numpy as np
 import pytest
 import torch
@@ -35,44 +36,56 @@ def test_oracle_known_answers():
     assert acc[3] == want[3] + (0.25 + 1.0) * 6144 and acc[5] == want[5] + 0.0625 * 6144
 
 
-@pytest.mark.parametrize("H,by8", [(6144, None), (6144, False), (100, None), (8, None), (2056, None)])
-def test_oracle_matches_float64_closed_form(H, by8):
+@pytest.mark.parametrize("H", [6144, 100, 8, 2056])
+def test_oracle_matches_float64_closed_form(H):
     rng = np.random.default_rng(H)
     E, T, K = 32, 5, 8
     x = (rng.standard_normal((T, H)) * 0.7).astype(np.float16)
     w = rng.random((T, K)).astype(np.float16); w[2, 3] = 0
     ids = rng.integers(0, E, (T, K))
     acc = np.zeros(E)
-    O.salience(x, w, ids, 2.5, acc, by8=by8)
-    want = closed_form(x, w, ids, np.float32(2.5), E)
-    assert np.allclose(acc, want, rtol=3e-6, atol=0)
-    # the two element orders give sums that differ in the last bits only
-    acc2 = np.zeros(E)
-    O.salience(x, w, ids, 2.5, acc2, by8=False)
-    assert np.allclose(acc, acc2, rtol=1e-6)
+    O.salience(x, w, ids, 2.5, acc)
+    assert np.allclose(acc, closed_form(x, w, ids, 2.5, E), rtol=3e-7, atol=0)        # rsf * w is an fp32 product in the oracle, as in the kernels
 
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
-def test_hip_salience_bit_exact(dtype):
+def test_hip_salience(dtype):
     from nestquant_amd import salience as SA
     g = torch.Generator().manual_seed(11)
     E, K = 256, 8
-    S = SA.Salience(E, rsf=2.5)
+    # exact cases: rows of +-1 and +-2 (every partial sum is a small integer), weights that are powers of two
+    S = SA.Salience(E, rsf=2.0)
     want = np.zeros(E)
-    for T, H, cut in ((1, 6144, 0), (8, 6144, 0), (3, 100, 0), (4, 2048, 1), (5, 4096, 8)):
-        big = (torch.randn(T, H + 16, generator=g) * 0.7).to(dtype)
-        x = big[:, cut:cut + H]                                       # cut = 1: rows off 16-byte alignment -> element order
-        w = torch.rand(T, K, generator=g).half(); w[0, 1] = 0
+    for T, H, cut in ((2, 6144, 0), (8, 6144, 0), (3, 100, 0), (4, 2048, 1), (1, 8, 0)):
+        sign = torch.randint(0, 2, (T, H + 16), generator=g) * 2 - 1
+        big = (sign * (1 + torch.arange(T)[:, None] % 2)).to(dtype)
+        x = big[:, cut:cut + H]                                       # cut = 1: rows off 16-byte alignment
+        w = (0.5 ** torch.randint(0, 4, (T, K), generator=g)).half(); w[0, 1] = 0
         ids = torch.randint(0, E, (T, K), generator=g); ids[-1, 0] = E + 3; ids[0, 2] = ids[0, 5]
-        xo = x.float().half().numpy() if dtype != torch.bfloat16 else x.float().numpy()
-        aligned = dtype == torch.float32 or (cut * x.element_size()) % 16 == 0 and (big.stride(0) * x.element_size()) % 16 == 0
-        touched = O.salience(xo, w.numpy(), ids.numpy(), 2.5, want, by8=None if aligned else False)
-        S(x.cuda(), w.cuda(), ids.cuda()) if cut == 0 else SA.sal(big.cuda()[:, cut:cut + H], w.cuda(), ids.cuda(), 2.5, S.acc, S.host)
+        touched = O.salience(x.float().numpy(), w.numpy(), ids.numpy(), 2.0, want)
+        S(x.cuda(), w.cuda(), ids.cuda()) if cut == 0 else SA.sal(big.cuda()[:, cut:cut + H], w.cuda(), ids.cuda(), 2.0, S.acc, S.host)
         torch.cuda.synchronize()
         got = S.acc.cpu().numpy()
         assert np.array_equal(got, want), (T, H, cut, np.abs(got - want).max())
         assert np.array_equal(S.host.numpy()[touched], want[touched])
+    # general values: fp32 rounding of the squared norm
+    S = SA.Salience(E, rsf=2.5)
+    want = np.zeros(E)
+    for T, H, cut in ((1, 6144, 0), (8, 6144, 0), (3, 100, 0), (4, 2048, 1), (5, 4096, 8), (7, 2056, 0)):
+        big = (torch.randn(T, H + 16, generator=g) * 0.7).to(dtype)
+        x = big[:, cut:cut + H]
+        w = torch.rand(T, K, generator=g).half(); w[0, 1] = 0
+        ids = torch.randint(0, E, (T, K), generator=g); ids[-1, 0] = E + 3; ids[0, 2] = ids[0, 5]
+        xo = x.float().half().float().numpy() if dtype != torch.bfloat16 else x.float().numpy()
+        touched = O.salience(xo, w.numpy(), ids.numpy(), 2.5, want)
+        S(x.cuda(), w.cuda(), ids.cuda()) if cut == 0 else SA.sal(big.cuda()[:, cut:cut + H], w.cuda(), ids.cuda(), 2.5, S.acc, S.host)
+        torch.cuda.synchronize()
+        got = S.acc.cpu().numpy()
+        assert np.allclose(got, want, rtol=1e-5, atol=0), (T, H, cut, np.abs(got / np.maximum(want, 1e-30) - 1).max())
+        assert np.array_equal(S.host.numpy()[touched], got[touched])
+        assert np.array_equal(got == 0, want == 0)                     # skipped picks touch nothing
+        want = got.copy()                                              # the running sums continue from the device's values
     # int32 ids and bf16 / fp32 weights read as the casts would leave them
     x = (torch.randn(2, 512, generator=g)).to(dtype).cuda()
     w32 = torch.rand(2, K, generator=g); ids = torch.randint(0, E, (2, K), generator=g)
@@ -113,4 +126,4 @@ def test_salience_errors_and_forward_hook():
             for i in range(0, T, 4):
                 O.salience(xt[i:i + 4].float().cpu().numpy(), wt[i:i + 4].half().cpu().numpy(), it[i:i + 4].cpu().numpy(), 1.5, want)
     torch.cuda.synchronize()
-    assert np.array_equal(S.acc.cpu().numpy(), want) and np.array_equal(S.host.numpy(), want)
+    assert np.allclose(S.acc.cpu().numpy(), want, rtol=1e-5, atol=0) and np.array_equal(S.host.numpy(), S.acc.cpu().numpy())
