@@ -190,7 +190,17 @@ int nq_pf_pre_rows(const void* x_f16, const int32_t* pt, const int32_t* pe, int 
  * other kind, which nothing would compute, gets NaN results instead of stale scratch. Replaces pf_decode + the Triton grouped GEMM / aten.mm
  * (reference sm120/pf_gemm.py:7-34, sm120/moe.py:303-324); decoded weights never touch HBM. */
 int nq_pf_gemm(const int64_t* table, const int32_t* tiles, int ntiles, int bm, int mode, const void* A0_f16,
-               const void* A1_f16, float* C, int E, int H, int I, void* stream);
+               const void* A1_f16, float* C, int E, int H, int I, const void* Wop, void* stream);
+
+/* Decode the experts that nq_pf_plan marked hot (hot[e] = their slot, -1 = none; device int32 [E]) once per call: projection
+ * `mode` (0 gate|up, 1 down) of each into slot hot[e] of the scratch Wop (slots x 3 * H * I fp16, 16-byte aligned), in the
+ * order in which nq_pf_gemm holds weights in registers, so that every tile of such an expert (fourth word of the tile = slot + 1)
+ * loads its operands instead of decoding the expert again. Experts at level <= 0, in mask mode or with a base code other than 0
+ * are left out (their tiles decode in the GEMM as before). Pass the same Wop to nq_pf_gemm; NULL there = every tile decodes.
+ * The reference decodes every expert of a group once too, but into dense [2I][H] / [H][I] matrices for a library GEMM
+ * (pf_decode, sm120/nqmoe.cu:1013-1080,1247-1257; sm120/moe.py:303-324). */
+int nq_pf_wdecode(const int64_t* table, const int32_t* hot, int E, int mode, void* Wop, int64_t wop_bytes, int slots, int H, int I,
+                  void* stream);
 
 /* h = fp16(Hadamard(silu(g) * u * su_d)), g = Hadamard(acc_gu[:, :I]) * sv_g, u = Hadamard(acc_gu[:, I:]) * sv_u; the last
  * Hadamard is 128 or 512 wide (table word 18). Low-rank plane: g / u += zg (U2 [+ U4 at level 4]) and zd[p] = (silu(g) * u)
@@ -216,9 +226,13 @@ int nq_pf_post(const float* y, const int32_t* pos, const int64_t* sel, const voi
  * sorted by expert); the chunk holds the pair rows [row_lo, row_lo + nrows). tiles: int32 [5][cap][4], list k for tile height
  * 16 << k, cap >= E + nrows / 256 + 1. An expert's rows inside the chunk are cut into 256-row tiles (indices E.. of list 4);
  * the remainder goes to index e of the list of the smallest height that holds it; every other entry gets expert -1, which
- * nq_pf_gemm skips. Launch nq_pf_gemm on list k with ntiles = E (k < 4) or cap (k = 4). Replaces the host loop over the
+ * nq_pf_gemm skips. Launch nq_pf_gemm on list k with ntiles = E (k < 4) or cap (k = 4). hot (device int32 [E], may be NULL):
+ * experts with at least hot_min rows in the chunk get a slot 0 .. hot_cap - 1 of the decoded-weight scratch, in expert order as
+ * far as the slots reach: hot[e] = slot or -1, and the fourth word of each of their tiles = slot + 1 (0 otherwise); see
+ * nq_pf_wdecode. Replaces the host loop over the
  * expert counts of the reference's prefill (sm120/moe.py:296-302) and the host synchronisation that feeds it. */
-int nq_pf_plan(const int32_t* counts, int E, int row_lo, int nrows, int32_t* tiles, int cap, void* stream);
+int nq_pf_plan(const int32_t* counts, int E, int row_lo, int nrows, int32_t* tiles, int cap, int32_t* hot, int hot_min, int hot_cap,
+               void* stream);
 
 /* hits[e] += counts[e] (hits may be host-mapped). Replaces pf_hits (reference sm120/nqmoe.cu:1241-1245,1288-1293). */
 int nq_pf_hits(const int32_t* counts, int32_t* hits, int E, void* stream);

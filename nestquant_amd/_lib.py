@@ -46,11 +46,12 @@ SIGNATURES = {
     "nq_mailbox": (C.c_int, [_i64p, _i64p, _i32p, _i32p, _i32p, _i, _vp]),
     "nq_pf_pre": (C.c_int, [_vp, _i32p, _i32p, _i, _i64p, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "nq_pf_pre_rows": (C.c_int, [_vp, _i32p, _i32p, _i, _i64p, _vp, _vp, _vp, _i, _i, _i, _i32p, _i, _i, _vp]),
-    "nq_pf_gemm": (C.c_int, [_i64p, _i32p, _i, _i, _i, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "nq_pf_gemm": (C.c_int, [_i64p, _i32p, _i, _i, _i, _vp, _vp, _vp, _i, _i, _i, _vp, _vp]),
+    "nq_pf_wdecode": (C.c_int, [_i64p, _i32p, _i, _i, _vp, C.c_int64, _i, _i, _i, _vp]),
     "nq_pf_mid": (C.c_int, [_vp, _i32p, _i, _i64p, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "nq_pf_mid_rows": (C.c_int, [_vp, _i32p, _i, _i64p, _vp, _vp, _vp, _i, _i, _i, _i32p, _i, _i, _vp]),
     "nq_pf_post": (C.c_int, [_vp, _i32p, _i64p, _vp, _i, _i, _i, _i, _i64p, _vp, _vp, _i, _i, _i, _vp]),
-    "nq_pf_plan": (C.c_int, [_i32p, _i, _i, _i, _i32p, _i, _vp]),
+    "nq_pf_plan": (C.c_int, [_i32p, _i, _i, _i, _i32p, _i, _i32p, _i, _i, _vp]),
     "nq_pf_hits": (C.c_int, [_i32p, _i32p, _i, _vp]),
     # record upgrade engine (host threads; structures mirrored in stream_engine.py)
     "nq_stream_open": (C.c_void_p, [C.c_char_p, C.c_char_p, C.c_int64, _i, _i, _i, _i]),

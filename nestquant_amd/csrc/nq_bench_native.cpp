@@ -101,13 +101,13 @@ int main(int argc, char** argv)
         for (int e = 0; e < E; ++e) { ht[4 * e] = e; ht[4 * e + 1] = e * pf_rows; ht[4 * e + 2] = pf_rows; ht[4 * e + 3] = 0; }
         HIPCHK(hipMalloc(&tiles, ht.size() * 4)); HIPCHK(hipMemcpy(tiles, ht.data(), ht.size() * 4, hipMemcpyHostToDevice));
         hipEvent_t e0, e1; HIPCHK(hipEventCreate(&e0)); HIPCHK(hipEventCreate(&e1));
-        NQCHK(nq_pf_gemm(d_table, tiles, E, bm, 0, xg, xu, cgu, E, H, I, nullptr)); NQCHK(nq_pf_gemm(d_table, tiles, E, bm, 1, hh, nullptr, cdn, E, H, I, nullptr));
+        NQCHK(nq_pf_gemm(d_table, tiles, E, bm, 0, xg, xu, cgu, E, H, I, nullptr, nullptr)); NQCHK(nq_pf_gemm(d_table, tiles, E, bm, 1, hh, nullptr, cdn, E, H, I, nullptr, nullptr));
         HIPCHK(hipDeviceSynchronize());
         HIPCHK(hipEventRecord(e0, nullptr));
         for (int st = 0; st < steps; ++st)
         {
-            NQCHK(nq_pf_gemm(d_table, tiles, E, bm, 0, xg, xu, cgu, E, H, I, nullptr));
-            NQCHK(nq_pf_gemm(d_table, tiles, E, bm, 1, hh, nullptr, cdn, E, H, I, nullptr));
+            NQCHK(nq_pf_gemm(d_table, tiles, E, bm, 0, xg, xu, cgu, E, H, I, nullptr, nullptr));
+            NQCHK(nq_pf_gemm(d_table, tiles, E, bm, 1, hh, nullptr, cdn, E, H, I, nullptr, nullptr));
         }
         HIPCHK(hipEventRecord(e1, nullptr)); HIPCHK(hipEventSynchronize(e1));
         float ms; HIPCHK(hipEventElapsedTime(&ms, e0, e1));

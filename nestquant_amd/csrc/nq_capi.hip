@@ -202,7 +202,7 @@ extern "C" int nq_pf_pre_rows(const void* x, const int32_t* pt, const int32_t* p
 }
 
 extern "C" int nq_pf_gemm(const int64_t* table, const int32_t* tiles, int ntiles, int bm, int mode, const void* A0, const void* A1,
-                          float* C, int E, int H, int I, void* stream)
+                          float* C, int E, int H, int I, const void* Wop, void* stream)
 {
     NQ_REQUIRE(ntiles >= 0, "nq_pf_gemm: ntiles=%d", ntiles);
     if (ntiles == 0) return 0;
@@ -212,7 +212,8 @@ extern "C" int nq_pf_gemm(const int64_t* table, const int32_t* tiles, int ntiles
     NQ_REQUIRE(ntiles <= 65535, "nq_pf_gemm: %d tiles exceed one launch (65535)", ntiles);
     NQ_REQUIRE(E >= 1 && shape_ok(H, I), "nq_pf_gemm: E=%d H=%d I=%d (H, I positive multiples of 128)", E, H, I);
     NQ_REQUIRE(aligned16(A0) && aligned16(A1) && aligned16(C) && aligned16(tiles), "nq_pf_gemm: tiles, activations and C must be 16-byte aligned");
-    return launch_pf_gemm(table, tiles, ntiles, bm, mode, A0, A1, C, E, H, I, (hipStream_t)stream);
+    NQ_REQUIRE(aligned16(Wop), "nq_pf_gemm: the decoded-weight scratch must be 16-byte aligned");
+    return launch_pf_gemm(table, tiles, ntiles, bm, mode, A0, A1, C, E, H, I, Wop, (hipStream_t)stream);
 }
 
 extern "C" int nq_pf_mid(const float* acc_gu, const int32_t* pe, int np, const int64_t* table, void* h, const float* zg, float* zd,
@@ -249,13 +250,23 @@ extern "C" int nq_pf_post(const float* y, const int32_t* pos, const int64_t* sel
     return launch_pf_post(y, pos, sel, rw, T, topk, row_lo, nrows, table, out, zd, E, H, I, (hipStream_t)stream);
 }
 
-extern "C" int nq_pf_plan(const int32_t* counts, int E, int row_lo, int nrows, int32_t* tiles, int cap, void* stream)
+extern "C" int nq_pf_wdecode(const int64_t* table, const int32_t* hot, int E, int mode, void* Wop, int64_t wop_bytes, int slots, int H, int I, void* stream)
+{
+    NQ_REQUIRE(table && hot && Wop, "nq_pf_wdecode: null pointer");
+    NQ_REQUIRE(E >= 1 && E <= 65535 && (mode == 0 || mode == 1) && slots >= 1, "nq_pf_wdecode: E=%d (1..65535) mode=%d slots=%d", E, mode, slots);
+    NQ_REQUIRE(shape_ok(H, I), "nq_pf_wdecode: H=%d I=%d (positive multiples of 128)", H, I);
+    NQ_REQUIRE(aligned16(Wop) && wop_bytes >= (int64_t)slots * 3 * H * I * 2, "nq_pf_wdecode: the scratch needs %d slots of 3 * H * I halfs, 16-byte aligned", slots);
+    return launch_pf_wdecode(table, hot, E, mode, Wop, H, I, (hipStream_t)stream);
+}
+
+extern "C" int nq_pf_plan(const int32_t* counts, int E, int row_lo, int nrows, int32_t* tiles, int cap, int32_t* hot, int hot_min, int hot_cap, void* stream)
 {
     NQ_REQUIRE(counts && tiles, "nq_pf_plan: null pointer");
     NQ_REQUIRE(E >= 1 && E <= 4096 && row_lo >= 0 && nrows >= 0, "nq_pf_plan: E=%d (1..4096) row_lo=%d nrows=%d", E, row_lo, nrows);
     NQ_REQUIRE(aligned16(tiles), "nq_pf_plan: tiles must be 16-byte aligned");
     NQ_REQUIRE(cap >= E + nrows / 256 + 1, "nq_pf_plan: cap=%d, need at least E + nrows / 256 + 1 = %d", cap, E + nrows / 256 + 1);
-    return launch_pf_plan(counts, E, row_lo, nrows, tiles, cap, (hipStream_t)stream);
+    NQ_REQUIRE(!hot || (hot_min >= 1 && hot_cap >= 1), "nq_pf_plan: hot_min=%d hot_cap=%d (both at least 1 with a hot list)", hot_min, hot_cap);
+    return launch_pf_plan(counts, E, row_lo, nrows, tiles, cap, hot, hot_min, hot_cap, (hipStream_t)stream);
 }
 
 extern "C" int nq_pf_hits(const int32_t* counts, int32_t* hits, int E, void* stream)

@@ -59,9 +59,10 @@ int launch_pf_post(const float* y, const int32_t* pos, const int64_t* sel, const
                    const int64_t* table, float* out, const float* zd, int E, int H, int I, hipStream_t st);
 int launch_sal(const void* x, int x_dtype, int64_t sx, const void* w, int w_dtype, const void* ids, int ids_dtype, int T, int H, int K,
                int E, float rsf, double* acc, double* host, hipStream_t st);
-int launch_pf_plan(const int32_t* counts, int E, int row_lo, int nrows, int32_t* tiles, int cap, hipStream_t st);
+int launch_pf_plan(const int32_t* counts, int E, int row_lo, int nrows, int32_t* tiles, int cap, int32_t* hot, int hot_min, int hot_cap, hipStream_t st);
+int launch_pf_wdecode(const int64_t* table, const int32_t* hot, int E, int mode, void* Wop, int H, int I, hipStream_t st);
 int launch_pf_hits(const int32_t* counts, int32_t* hits, int E, hipStream_t st);
 int launch_pf_gemm(const int64_t* table, const int32_t* tiles, int ntiles, int bm, int mode, const void* A0, const void* A1, float* C,
-                   int E, int H, int I, hipStream_t st);
+                   int E, int H, int I, const void* Wop, hipStream_t st);
 
 }  // namespace nq

@@ -344,10 +344,13 @@ __device__ __forceinline__ void block_scan(int* a, int* b, int E)
     }
 }
 
-__global__ void __launch_bounds__(256) nq_pf_plan_k(const int32_t* __restrict__ counts, int E, int row_lo, int nrows, int32_t* tiles, int cap)
+// hot (may be null): experts with at least hot_min rows in the chunk get a slot 0 .. hot_cap - 1 of the decoded-weight scratch (in
+// expert order, as far as the slots reach), written to hot[e] (-1: none) and, plus one, into the fourth word of their tiles.
+__global__ void __launch_bounds__(256) nq_pf_plan_k(const int32_t* __restrict__ counts, int E, int row_lo, int nrows, int32_t* tiles, int cap,
+                                                    int32_t* hot, int hot_min, int hot_cap)
 {
     extern __shared__ int plan_sh[];
-    int *incl = plan_sh, *tmp = plan_sh + E, *full = plan_sh + 2 * E;
+    int *incl = plan_sh, *tmp = plan_sh + E, *full = plan_sh + 2 * E, *hrank = plan_sh + 3 * E;
     for (int e = threadIdx.x; e < E; e += blockDim.x) incl[e] = counts[e] > 0 ? counts[e] : 0;
     __syncthreads();
     block_scan(incl, tmp, E);
@@ -358,8 +361,10 @@ __global__ void __launch_bounds__(256) nq_pf_plan_k(const int32_t* __restrict__ 
         const int u = start > row_lo ? start : row_lo, v = start + c < row_hi ? start + c : row_hi;
         const int n = v > u ? v - u : 0;
         full[e] = n / 256;
+        hrank[e] = hot != nullptr && n >= hot_min ? 1 : 0;
     }
     __syncthreads();
+    block_scan(hrank, tmp, E);                                   // inclusive: hot experts up to and including e
     int* fincl = tmp;                                            // inclusive scan of the full-tile counts
     for (int e = threadIdx.x; e < E; e += blockDim.x) fincl[e] = full[e];
     __syncthreads();
@@ -371,18 +376,21 @@ __global__ void __launch_bounds__(256) nq_pf_plan_k(const int32_t* __restrict__ 
         const int u = start > row_lo ? start : row_lo, v = start + c < row_hi ? start + c : row_hi;
         const int n = v > u ? v - u : 0, r0 = u - row_lo, nf = n / 256, rem = n % 256;
         const int k = rem == 0 ? -1 : rem <= 16 ? 0 : rem <= 32 ? 1 : rem <= 64 ? 2 : rem <= 128 ? 3 : 4;
+        const bool is_hot = hot != nullptr && n >= hot_min && hrank[e] <= hot_cap;
+        const int slot1 = is_hot ? hrank[e] : 0;                 // scratch slot + 1
+        if (hot != nullptr) hot[e] = slot1 - 1;
 #pragma unroll
-        for (int q = 0; q < 5; ++q) T4[(size_t)q * cap + e] = q == k ? make_int4(e, r0 + 256 * nf, rem, 0) : make_int4(-1, 0, 0, 0);
+        for (int q = 0; q < 5; ++q) T4[(size_t)q * cap + e] = q == k ? make_int4(e, r0 + 256 * nf, rem, slot1) : make_int4(-1, 0, 0, 0);
         const int base = E + fincl[e] - nf;
-        for (int j = 0; j < nf; ++j) T4[(size_t)4 * cap + base + j] = make_int4(e, r0 + 256 * j, 256, 0);
+        for (int j = 0; j < nf; ++j) T4[(size_t)4 * cap + base + j] = make_int4(e, r0 + 256 * j, 256, slot1);
     }
     const int total = E + fincl[E - 1];
     for (int i = total + threadIdx.x; i < cap; i += blockDim.x) T4[(size_t)4 * cap + i] = make_int4(-1, 0, 0, 0);
 }
 
-int launch_pf_plan(const int32_t* counts, int E, int row_lo, int nrows, int32_t* tiles, int cap, hipStream_t st)
+int launch_pf_plan(const int32_t* counts, int E, int row_lo, int nrows, int32_t* tiles, int cap, int32_t* hot, int hot_min, int hot_cap, hipStream_t st)
 {
-    nq_pf_plan_k<<<1, 256, 3 * E * sizeof(int), st>>>(counts, E, row_lo, nrows, tiles, cap);
+    nq_pf_plan_k<<<1, 256, 4 * E * sizeof(int), st>>>(counts, E, row_lo, nrows, tiles, cap, hot, hot_min, hot_cap);
     NQ_LAUNCH_CHECK("nq_pf_plan");
     return 0;
 }
@@ -393,7 +401,173 @@ struct PfGemm
     const _Float16* A0; const _Float16* A1;         // activations in B-operand order: A0 for weight rows < I (or all rows of down), A1 above
     float* C; int mode, E, H, I;
     int solo;                                       // the other kernel variant will not be launched on these tiles: a tile that is its kind comes out NaN
+    const u32x4* Wop;                               // decoded weights of hot experts in A-operand order (nq_pf_wdecode_k), or null
+    int skip_hot;                                   // leave the 256-row tiles of hot experts to nq_pf_dense_k
 };
+
+// ---- decoded-weight scratch of hot experts --------------------------------------------------------------------------------
+// An expert with many pair rows is cut into several 256-row tiles, and every tile's workgroups would decode the expert again.
+// Such experts are decoded once per call instead, into fp16 scratch laid out exactly as the grouped GEMM holds weights in
+// registers: for strip pair sp (32 weight rows), chunk c, MFMA (mm, rho) one 1 KB block of 64 lanes x 16 bytes, the A operand of
+// that MFMA. A tile of a hot expert then loads its operands (coalesced, 16 bytes per lane) where the others decode.
+// Slot k of the scratch holds gate|up ([2I / 32][H / 128][8] blocks) followed by down ([H / 32][I / 128][8] blocks).
+__device__ __forceinline__ size_t wop_base(int slot, int mode, int H, int I)
+{   // in 16-byte units
+    const size_t gu = (size_t)(2 * I / 32) * (H / 128) * 8 * 64, dn = (size_t)(H / 32) * (I / 128) * 8 * 64;
+    return (size_t)slot * (gu + dn) + (mode ? gu : 0);
+}
+
+template <bool RES, int CODE>
+__device__ __forceinline__ void wdecode_chunks(const Planes& P, const LaneCtx& L, int C, u32x4* dst, int lane)
+{
+    constexpr int NW = RES ? Rec<CODE>::NW : 1;
+    u32x4 nb = P.base[L.rec0];
+    uint32_t nr[NW + 2] = {0}, ndw = 0, nvar = 0;
+    if constexpr (RES) { load_record<CODE>(nr, P.res, L.rec0, L.nrec); ndw = P.dw[L.unit0]; }
+    if (P.var) nvar = P.var[L.unit0];
+    for (int c = 0; c < C; ++c)
+    {
+        uint32_t wb[6], wr[NW + 2];
+        wb[0] = nb.x; wb[1] = nb.y; wb[2] = nb.z; wb[3] = nb.w;
+#pragma unroll
+        for (int i = 0; i < NW; ++i) wr[i] = nr[i];
+        const uint32_t dw = ndw, var = nvar;
+        if (c + 1 < C)
+        {
+            nb = P.base[L.rec0 + (size_t)(c + 1) * 32];
+            if constexpr (RES) { load_record<CODE>(nr, P.res, L.rec0 + (size_t)(c + 1) * 32, L.nrec); ndw = P.dw[L.unit0 + c + 1]; }
+            if (P.var) nvar = P.var[L.unit0 + c + 1];
+        }
+        ext_base<0>(wb, __shfl(wb[0], L.src));
+        const uint32_t sgm = ((var >> L.g) & 1u) * 0x80008000u;
+        FoldK k;
+        if constexpr (RES) { ext_words<Rec<CODE>::BITS, Rec<CODE>::NW>(wr, __shfl(wr[0], L.src)); k = consts_fold(dw, sgm); }
+        else k = consts_l2(sgm);
+        u32x4* d = dst + (size_t)c * 8 * 64 + lane;
+        static_for<4>([&](auto mm) {
+            constexpr int MM = decltype(mm)::value;
+            d[(MM * 2 + 0) * 64] = __builtin_bit_cast(u32x4, a_operand<RES, CODE, MM, 0>(wb, wr, k));
+            d[(MM * 2 + 1) * 64] = __builtin_bit_cast(u32x4, a_operand<RES, CODE, MM, 1>(wb, wr, k));
+        });
+    }
+}
+
+// grid (N / 128, E), block 256: block (x, e) decodes 128 weight rows of expert e if it has a scratch slot (hot[e] >= 0) and its
+// row is of the common kind (K = 2 base plane, no mask-mode flags; others keep decoding inside the GEMM, whatever hot[] says)
+__global__ void __launch_bounds__(256) nq_pf_wdecode_k(const int64_t* table, const int32_t* hot, int mode, u32x4* Wop, int H, int I)
+{
+    const int e = blockIdx.y, slot = hot[e];
+    if (slot < 0) return;
+    const int64_t* ent = table + (size_t)e * TBL_W;
+    const int lv = (int)ent[0];
+    if (lv <= 0) return;
+    const Planes P = planes_of(ent, mode);
+    if (P.bcode != 0 || P.flags != nullptr) return;
+    const int lane = threadIdx.x & 63, warp = threadIdx.x >> 6;
+    const int N = mode == 0 ? 2 * I : H, K = mode == 0 ? H : I, C = K / 128;
+    const int sp = blockIdx.x * 4 + warp, t4 = lane >> 4, ss = (lane >> 3) & 1, g = lane & 7;
+    LaneCtx L;
+    L.unit0 = (size_t)(2 * sp + ss) * C; L.rec0 = L.unit0 * 32 + 4 * g + t4;
+    L.nrec = (size_t)(N / 16) * C * 32;
+    L.src = (lane + 16) & 63; L.g = g; L.xs = nullptr; L.xstep = 0;
+    L.strip = (size_t)(2 * sp + ss); L.nstrips = (size_t)(N / 16); L.chunk0 = 0;
+    u32x4* dst = Wop + wop_base(slot, mode, H, I) + (size_t)sp * C * 8 * 64;
+    if (lv == 2) wdecode_chunks<false, 0>(P, L, C, dst, lane);
+    else dispatch_code(P.code, [&](auto tag) { wdecode_chunks<true, decltype(tag)::value>(P, L, C, dst, lane); });
+}
+
+int launch_pf_wdecode(const int64_t* table, const int32_t* hot, int E, int mode, void* Wop, int H, int I, hipStream_t st)
+{
+    const int N = mode == 0 ? 2 * I : H;
+    nq_pf_wdecode_k<<<dim3(N / 128, E), 256, 0, st>>>(table, hot, mode, (u32x4*)Wop, H, I);
+    NQ_LAUNCH_CHECK("nq_pf_wdecode");
+    return 0;
+}
+
+
+// The MFMA phase of one chunk: TG x 8 MFMAs, tokens 16 tg + n as the N dimension (row groups beyond the tile multiply stale
+// LDS rows whose results are never stored). Two row groups are interleaved so that four different accumulators separate an
+// MFMA from the next one that depends on it, and the operand reads run one group (one mm of two row groups) ahead of the
+// MFMAs that use them.
+template <int TG>
+__device__ __forceinline__ void pf_mfmas(const half8_t (*aop)[2], const char* smem, const uint32_t* boff, float4_t (*acc)[2])
+{
+    constexpr int TS = TG >= 2 ? 2 : 1, NGRP = TG / TS * 4;
+    half8_t bq[2][TS];
+    auto bread = [&](int grp, half8_t* dst) {
+        const int tg = grp / 4 * TS, mm = grp % 4;
+#pragma unroll
+        for (int u = 0; u < TS; ++u) dst[u] = *(const half8_t*)(smem + boff[mm] + (tg + u) * 16 * PF_ROW);
+    };
+    bread(0, bq[0]);
+#pragma unroll
+    for (int gq = 0; gq < NGRP; ++gq)
+    {
+        if (gq + 1 < NGRP) bread(gq + 1, bq[(gq + 1) % 2]);
+        __builtin_amdgcn_sched_barrier(0);
+        const int tg = gq / 4 * TS, mm = gq % 4;
+#pragma unroll
+        for (int u = 0; u < TS; ++u)
+        {
+            const half8_t b = bq[gq % 2][u];
+            acc[tg + u][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aop[mm][0], b, acc[tg + u][0], 0, 0, 0);
+            acc[tg + u][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aop[mm][1], b, acc[tg + u][1], 0, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+
+// Token staging shared by the GEMM bodies: wavefront w copies rows 16 u + 4 w + (lane >> 4), u = 0 .. TG - 1, of the tile, one
+// 1 KB global -> LDS load per u (64 lanes x 16 bytes land in LDS in lane order, so a load fills 4 rows x 256 bytes). The lane
+// picks which 16-byte column of its row it fetches: column (lane & 15) ^ (row & 15) goes to slot lane & 15, and the MFMA reads
+// undo the XOR, which spreads the 16 tokens of an operand read over all banks without padding. Rows beyond the tile re-read
+// its last row: their products are never stored.
+template <int TG>
+__device__ __forceinline__ void pf_stage_tokens(const _Float16* A, int K, int row0, int nrows, int c, char* smem, int warp, int srow, uint32_t scol)
+{
+    typedef const __attribute__((address_space(1))) void* gvp;
+    typedef __attribute__((address_space(3))) void* lvp;
+#pragma unroll
+    for (int u = 0; u < TG; ++u)
+    {
+        if (16 * u >= nrows) break;                              // block-uniform
+        const int row = 16 * u + srow, grow = row < nrows ? row : nrows - 1;
+        const char* src = (const char*)A + ((size_t)(row0 + grow) * K + c * 128) * 2 + scol;
+        __builtin_amdgcn_global_load_lds((gvp)src, (lvp)(smem + (16 * u + 4 * warp) * PF_ROW), 16, 0, 0);
+    }
+}
+
+// body for a tile of a hot expert: the A operands of this wavefront's two strips come from the decoded-weight scratch
+// (w: this strip pair's blocks, [C][8][64] x 16 bytes), one chunk ahead of the MFMAs that use them
+template <int TG>
+__device__ __forceinline__ void pf_chunks_pre(const u32x4* w, int C, const _Float16* A, int K, int row0, int nrows, char* smem, float4_t (*acc)[2])
+{
+    const int lane = threadIdx.x & 63, warp = threadIdx.x >> 6, t4 = lane >> 4, n = lane & 15;
+    const int srow = 4 * warp + t4;
+    const uint32_t scol = (uint32_t)((n ^ srow) * 16);
+    uint32_t boff[4];
+#pragma unroll
+    for (int mm = 0; mm < 4; ++mm) boff[mm] = (uint32_t)(n * PF_ROW + (((4 * mm + t4) ^ n) << 4));
+    u32x4 nx[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) nx[i] = w[(size_t)i * 64 + lane];
+    for (int c = 0; c < C; ++c)
+    {
+        pf_stage_tokens<TG>(A, K, row0, nrows, c, smem, warp, srow, scol);
+        half8_t aop[4][2];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) aop[i >> 1][i & 1] = __builtin_bit_cast(half8_t, nx[i]);
+        if (c + 1 < C)
+        {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) nx[i] = w[((size_t)(c + 1) * 8 + i) * 64 + lane];
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");         // the tokens have landed (and the next chunk's operands, requested with them)
+        __syncthreads();
+        pf_mfmas<TG>(aop, smem, boff, acc);
+        __syncthreads();
+    }
+}
 
 // body for one (RES, CODE): all K / 128 chunks of this wave's two strips against the tile's tokens
 template <int TG, bool RES, int CODE, bool MASKED, int BK = 0>
@@ -425,14 +599,7 @@ __device__ __forceinline__ void pf_chunks(const Planes& P, const LaneCtx& L, int
     for (int c = 0; c < C; ++c)
     {
         // ---- request the tile's tokens for chunk c (asynchronous: the decode below runs while they arrive)
-#pragma unroll
-        for (int u = 0; u < TG; ++u)
-        {
-            if (16 * u >= nrows) break;                          // block-uniform
-            const int row = 16 * u + srow, grow = row < nrows ? row : nrows - 1;
-            const char* src = (const char*)A + ((size_t)(row0 + grow) * K + c * 128) * 2 + scol;
-            __builtin_amdgcn_global_load_lds((gvp)src, (lvp)(smem + (16 * u + 4 * warp) * PF_ROW), 16, 0, 0);
-        }
+        pf_stage_tokens<TG>(A, K, row0, nrows, c, smem, warp, srow, scol);
         // ---- decode this wave's unit pair of chunk c into A operands; prefetch chunk c + 1
         uint32_t wb[6], wr[NW + 2];
         wb[0] = nb.x; wb[1] = nb.y; wb[2] = nb.z; wb[3] = nb.w;
@@ -481,55 +648,7 @@ __device__ __forceinline__ void pf_chunks(const Planes& P, const LaneCtx& L, int
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");         // this wavefront's share of the tile has landed
         __syncthreads();
         __builtin_amdgcn_s_setprio(3);                           // MFMA phase first: see below
-        // ---- TG x 8 MFMAs: tokens 16 tg + n as the N dimension (row groups beyond the tile multiply stale LDS rows whose
-        // results are never stored). Two row groups are interleaved so that four different accumulators separate an MFMA
-        // from the next one that depends on it.
-        constexpr int TS = TG >= 2 ? 2 : 1, NGRP = TG / TS * 4, PD = 1;      // read-ahead depth in groups
-        if constexpr (PD == 0)
-        {
-#pragma unroll
-            for (int tg = 0; tg < TG; tg += TS)
-            {
-#pragma unroll
-                for (int mm = 0; mm < 4; ++mm)
-                {
-#pragma unroll
-                    for (int u = 0; u < TS; ++u)
-                    {
-                        const half8_t b = *(const half8_t*)(smem + boff[mm] + (tg + u) * 16 * PF_ROW);
-                        acc[tg + u][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aop[mm][0], b, acc[tg + u][0], 0, 0, 0);
-                        acc[tg + u][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aop[mm][1], b, acc[tg + u][1], 0, 0, 0);
-                    }
-                }
-            }
-        }
-        else
-        {
-            // operand reads run PD groups ahead of the MFMAs that use them (a group = one mm of TS row groups)
-            half8_t bq[PD + 1][TS];
-            auto bread = [&](int grp, half8_t* dst) {
-                const int tg = grp / 4 * TS, mm = grp % 4;
-#pragma unroll
-                for (int u = 0; u < TS; ++u) dst[u] = *(const half8_t*)(smem + boff[mm] + (tg + u) * 16 * PF_ROW);
-            };
-#pragma unroll
-            for (int gq = 0; gq < PD; ++gq) bread(gq, bq[gq]);
-#pragma unroll
-            for (int gq = 0; gq < NGRP; ++gq)
-            {
-                if (gq + PD < NGRP) bread(gq + PD, bq[(gq + PD) % (PD + 1)]);
-                __builtin_amdgcn_sched_barrier(0);
-                const int tg = gq / 4 * TS, mm = gq % 4;
-#pragma unroll
-                for (int u = 0; u < TS; ++u)
-                {
-                    const half8_t b = bq[gq % (PD + 1)][u];
-                    acc[tg + u][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aop[mm][0], b, acc[tg + u][0], 0, 0, 0);
-                    acc[tg + u][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aop[mm][1], b, acc[tg + u][1], 0, 0, 0);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
+        pf_mfmas<TG>(aop, smem, boff, acc);
         __builtin_amdgcn_s_setprio(0);
         __syncthreads();                                         // every wavefront has read chunk c before chunk c + 1 overwrites it
     }
@@ -546,7 +665,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) n
     extern __shared__ __align__(16) char smem[];
     const int lane = threadIdx.x & 63, warp = threadIdx.x >> 6;
     const int32_t* tile = a.tiles + 4 * blockIdx.y;
-    const int e = tile[0], row0 = tile[1], nrows = tile[2];
+    const int e = tile[0], row0 = tile[1], nrows = tile[2], slot = tile[3] - 1;
     if (e < 0 || e >= a.E || nrows <= 0) return;
     const int64_t* ent = a.table + (size_t)e * TBL_W;
     const int lv = (int)ent[0];
@@ -576,7 +695,11 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) n
     for (int tg = 0; tg < TG; ++tg) { acc[tg][0] = float4_t{0.f, 0.f, 0.f, 0.f}; acc[tg][1] = float4_t{0.f, 0.f, 0.f, 0.f}; }
     if constexpr (!MASKED)
     {
-        if (lv == 2) pf_chunks<TG, false, 0, false>(P, L, C, A, K, row0, nrows, smem, acc);
+        // a hot expert (several tiles): its weights were decoded once into the scratch by nq_pf_wdecode_k (block-uniform)
+        const bool pre = a.Wop != nullptr && slot >= 0 && P.flags == nullptr;
+        if (pre && a.skip_hot) return;                           // nq_pf_dense_k has this tile
+        if (pre) pf_chunks_pre<TG>(a.Wop + wop_base(slot, a.mode, a.H, a.I) + (size_t)sp * C * 8 * 64, C, A, K, row0, nrows, smem, acc);
+        else if (lv == 2) pf_chunks<TG, false, 0, false>(P, L, C, A, K, row0, nrows, smem, acc);
         else dispatch_code(P.code, [&](auto tag) { pf_chunks<TG, true, decltype(tag)::value, false>(P, L, C, A, K, row0, nrows, smem, acc); });
     }
     else
@@ -646,10 +769,10 @@ static int launch_gemm_tg(const PfGemm& a, int ntiles, int N, hipStream_t st)
 }
 
 int launch_pf_gemm(const int64_t* table, const int32_t* tiles, int ntiles, int bm, int mode, const void* A0, const void* A1, float* C,
-                   int E, int H, int I, hipStream_t st)
+                   int E, int H, int I, const void* Wop, hipStream_t st)
 {
     if (!ntiles) return 0;
-    PfGemm a{table, tiles, (const _Float16*)A0, (const _Float16*)A1, C, mode & 1, E, H, I, (mode & 4) != 0};
+    PfGemm a{table, tiles, (const _Float16*)A0, (const _Float16*)A1, C, mode & 1, E, H, I, (mode & 4) != 0, (const u32x4*)Wop, 0};
     const int N = (mode & 1) == 0 ? 2 * I : H;
     const bool masked = (mode & 2) != 0;
     switch (bm)

@@ -187,7 +187,13 @@ struct Engine
         ok = ok && hip_ok(hipMemcpyAsync(o->seqp, seqs + o->ring, 4, hipMemcpyHostToDevice, st), "hipMemcpyAsync(seq)");
         o->copy_failed = !ok;                                    // the chain stops at the first failure, so seq is never written after one
         o->ev = get_event();
-        if (o->ev) hip_ok(hipEventRecord(o->ev, st), "hipEventRecord");
+        if (!o->ev || !hip_ok(hipEventRecord(o->ev, st), "hipEventRecord"))
+        {
+            // no event to watch: the op may not be retired (its pinned row, seq and host entry handed to the next op) while its
+            // copies can still be in flight, so wait for the stream here, once, instead
+            if (o->ev) { evpool.push_back(o->ev); o->ev = nullptr; }
+            if (!hip_ok(hipStreamSynchronize(st), "hipStreamSynchronize")) o->copy_failed = true;
+        }
         copying.push_back(o); n_copying++;
     }
     void retire_copies()
@@ -195,8 +201,13 @@ struct Engine
         for (size_t i = 0; i < copying.size();)
         {
             Op* o = copying[i];
-            if (o->ev && hipEventQuery(o->ev) == hipErrorNotReady) { ++i; continue; }
-            if (o->ev) evpool.push_back(o->ev);
+            if (o->ev)
+            {
+                const hipError_t q = hipEventQuery(o->ev);
+                if (q == hipErrorNotReady) { ++i; continue; }
+                if (q != hipSuccess) { hip_ok(q, "hipEventQuery"); o->copy_failed = true; }   // a real error is a failed op, not a landed one
+                evpool.push_back(o->ev);
+            }
             ring_free.push_back(o->ring);
             if (o->tier_src) tier_users--;
             else if (o->read) ent_users[o->entry]--;
@@ -527,6 +538,8 @@ int64_t nq_stream_tier_load(NqStream* s, const int64_t* recs, int64_t n)
     Engine& e = s->e;
     if (e.tier_state.load() != 0) { nq::set_error("nq_stream_tier_load: tier already loaded / dropped"); return -1; }
     if (n <= 0) return 0;
+    if (e.nd == 0 || e.rb == 0) { nq::set_error("nq_stream_tier_load: this engine was opened without a record file (uploads and row-only ops only)"); return -1; }
+    if (!recs) { nq::set_error("nq_stream_tier_load: null record list"); return -1; }
     hipError_t he = hipSetDevice(e.dev);
     uint8_t* m = nullptr;
     if (he == hipSuccess) he = hipHostMalloc((void**)&m, (size_t)n * e.rb, hipHostMallocPortable);

@@ -261,21 +261,28 @@ class MoELayer:
 
 _PF = {}
 PF_TILES = (16, 32, 64, 128, 256)            # token-tile heights the grouped GEMM is compiled for
+# An expert with at least PF_HOT_MIN pair rows in a chunk (more than one 256-row tile) is decoded once per call into a scratch of
+# decoded weights (at most PF_HOT_SLOTS experts at 6 H I bytes each) instead of once per tile; see nq_pf_wdecode.
+PF_HOT_MIN, PF_HOT_SLOTS = 257, 32
 
 
 def pf_bytes(H, I, R, G=0):
-    """bytes of prefill scratch for R pair rows (G is accepted for signature compatibility: no decoded-weight scratch exists)"""
-    return R * (2 * H * 2 + 2 * I * 4 + I * 2 + H * 4 + 32)
+    """bytes of prefill scratch for R pair rows (G is accepted for signature compatibility: the decoded-weight scratch is sized
+    by the rows, not by a group of experts)"""
+    return R * (2 * H * 2 + 2 * I * 4 + I * 2 + H * 4 + 32) + max(0, min(PF_HOT_SLOTS, R // PF_HOT_MIN)) * 6 * H * I
 
 
 def pf_scratch(dev, H, I, R, G=0):
     """Prefill scratch shared by every layer on `dev`, allocated on first use: xg | xu fp16 [R, H], acc_gu fp32 [R, 2I],
-    h fp16 [R, I], y fp32 [R, H]. Unlike the reference (sm120/moe.py:263-274) there is no dense-weight scratch: the
-    grouped GEMM decodes weights in registers."""
+    h fp16 [R, I], y fp32 [R, H], and wop: decoded weights of up to PF_HOT_SLOTS hot experts. Unlike the reference
+    (sm120/moe.py:263-274), which decodes every expert of a group into dense scratch, only experts with more than one tile go
+    through scratch; the others are decoded in registers inside the grouped GEMM."""
     k = (str(dev), H, I, R)
     if k not in _PF:
         f16, f32 = torch.float16, torch.float32
-        _PF[k] = dict(xg=torch.empty(R, H, dtype=f16, device=dev), xu=torch.empty(R, H, dtype=f16, device=dev),
+        slots = max(0, min(PF_HOT_SLOTS, R // PF_HOT_MIN))
+        _PF[k] = dict(wop=torch.empty(slots, 3 * H * I, dtype=f16, device=dev) if slots else None,
+                      xg=torch.empty(R, H, dtype=f16, device=dev), xu=torch.empty(R, H, dtype=f16, device=dev),
                       acc=torch.empty(R, 2 * I, dtype=f32, device=dev), h=torch.empty(R, I, dtype=f16, device=dev),
                       y=torch.empty(R, H, dtype=f32, device=dev),
                       zg=torch.zeros(R, 4, dtype=f32, device=dev), zd=torch.zeros(R, 4, dtype=f32, device=dev))
@@ -299,7 +306,7 @@ _PF_SIDE = {}
 _PF_STREAM_OF = {256: 0, 128: 1, 64: 2, 32: 3, 16: 3}          # stream 0 = the caller's
 
 
-def _pf_chains(Lb, tb, lists, variants, S, x, pts, pes, n, tiles, cap, E, H, I):
+def _pf_chains(Lb, tb, lists, variants, S, x, pts, pes, n, tiles, cap, E, H, I, wop=None):
     """Everything between the tile plan and the post kernel of one row chunk: rotation of the activations, gate|up GEMM, SwiGLU
     kernel and down GEMM of every tile height. The heights work on disjoint pair rows, so each is a chain of its own. A GEMM
     launch ends with the GPU partly idle while its last workgroups drain (a workgroup runs the whole K loop, ~75 us, so a
@@ -320,7 +327,7 @@ def _pf_chains(Lb, tb, lists, variants, S, x, pts, pes, n, tiles, cap, E, H, I):
         for bm, t, nt in lists:
             stp = C.c_void_p(streams[_PF_STREAM_OF[bm]].cuda_stream)
             for v in variants:
-                _lib.check(Lb.nq_pf_gemm(tb.data_ptr(), t.data_ptr(), nt, bm, mode | v, A0, A1, Cm, E, H, I, stp))
+                _lib.check(Lb.nq_pf_gemm(tb.data_ptr(), t.data_ptr(), nt, bm, mode | v, A0, A1, Cm, E, H, I, wop, stp))
 
     masks = [sum(bm // 16 for bm, _, _ in lists if _PF_STREAM_OF[bm] == i) for i in range(len(streams))]    # bit k = height 16 << k
     for st, heights in zip(streams, masks):
@@ -375,10 +382,18 @@ def prefill(s, x, sel, rw, out=None, R=None, G=None, table=None):
         # tile lists of the chunk, built on the device from the expert counts: list i = tiles of height 16 << i, entries
         # without a tile are skipped by the GEMM (no host synchronisation anywhere in the call)
         tiles = torch.empty(5, cap, 4, dtype=torch.int32, device=dev)
-        _lib.check(Lb.nq_pf_plan(cnt.data_ptr(), E, c, n, tiles.data_ptr(), cap, st))
+        # experts with several tiles are decoded once into scratch (rows of the common kind only: the variant kernel of the
+        # others decodes in the GEMM); the side streams of _pf_chains start after these launches
+        wop = S["wop"] if (S["wop"] is not None and n >= PF_HOT_MIN and not s.rare_rows and table is None) else None
+        hot = torch.empty(E, dtype=torch.int32, device=dev) if wop is not None else None
+        _lib.check(Lb.nq_pf_plan(cnt.data_ptr(), E, c, n, tiles.data_ptr(), cap, None if hot is None else hot.data_ptr(), PF_HOT_MIN,
+                                 0 if wop is None else wop.shape[0], st))
+        if wop is not None:
+            for mode in (0, 1):
+                _lib.check(Lb.nq_pf_wdecode(tb.data_ptr(), hot.data_ptr(), E, mode, wop.data_ptr(), wop.numel() * 2, wop.shape[0], H, I, st))
         lists = [(16 << i, tiles[i], E if i < 4 else cap) for i in (4, 3, 2, 1, 0)]          # tallest first
         pts, pes = pt[c:d], pe[c:d]
-        _pf_chains(Lb, tb, lists, variants, S, x, pts, pes, n, tiles, cap, E, H, I)
+        _pf_chains(Lb, tb, lists, variants, S, x, pts, pes, n, tiles, cap, E, H, I, None if wop is None else wop.data_ptr())
         _lib.check(Lb.nq_pf_post(S["y"].data_ptr(), pos.data_ptr(), selc.data_ptr(), rwc.data_ptr(), T, k, c, n, tb.data_ptr(),
                                  out.data_ptr(), S["zd"].data_ptr(), E, H, I, st))
     return out

@@ -110,10 +110,12 @@ def test_argument_checks_run_before_any_device_work():
     a.mb_table = None; a.G = 3
     a.G = 0; a.common_rows = 2
     assert L.nq_moe_forward(C.byref(a), None) != 0 and "common_rows" in err()
-    assert L.nq_pf_plan(base, 256, 0, 1024, base, 256, None) != 0 and "cap" in err()
-    assert L.nq_pf_plan(base, 256, 0, 1024, base + 4, 512, None) != 0 and "aligned" in err()
-    assert L.nq_pf_gemm(base, base, 1, 48, 0, base, base, base, 4, 256, 256, None) != 0 and "tile height" in err()
-    assert L.nq_pf_gemm(base, base, 1, 16, 0, base + 8, base, base, 4, 256, 256, None) != 0 and "aligned" in err()
+    assert L.nq_pf_plan(base, 256, 0, 1024, base, 256, None, 0, 0, None) != 0 and "cap" in err()
+    assert L.nq_pf_plan(base, 256, 0, 1024, base + 4, 512, None, 0, 0, None) != 0 and "aligned" in err()
+    assert L.nq_pf_gemm(base, base, 1, 48, 0, base, base, base, 4, 256, 256, None, None) != 0 and "tile height" in err()
+    assert L.nq_pf_gemm(base, base, 1, 16, 0, base + 8, base, base, 4, 256, 256, None, None) != 0 and "aligned" in err()
+    assert L.nq_pf_plan(base, 256, 0, 1024, base, 512, base, 0, 4, None) != 0 and "hot_min" in err()
+    assert L.nq_pf_wdecode(base, base, 4, 0, base, 100, 2, 256, 256, None) != 0 and "scratch" in err()
     assert L.nq_pf_pre(base + 2, base, base, 1, base, base, base, None, 4, 256, 256, None) != 0 and "aligned" in err()
     assert L.nq_pf_pre_rows(base, base, base, 1, base, base, base, None, 4, 256, 256, base, 3, 1, None) != 0 and "cap" in err()
     assert L.nq_pf_pre_rows(base, base, base, 1, base, base, base, None, 4, 256, 256, base, 4, 32, None) != 0 and "heights" in err()

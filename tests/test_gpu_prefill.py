@@ -96,7 +96,7 @@ def test_prefill_argument_errors_and_empty():
         t = torch.tensor([[0, 0, 4, 0]], dtype=torch.int32, device=DEV)
         buf = torch.zeros(8, 512, dtype=torch.float16, device=DEV); c = torch.zeros(8, 512, device=DEV)
         from nestquant_amd import _lib
-        _lib.check(_lib.lib().nq_pf_gemm(tb.data_ptr(), t.data_ptr(), 1, 48, 0, buf.data_ptr(), buf.data_ptr(), c.data_ptr(), 4, 256, 256, None))
+        _lib.check(_lib.lib().nq_pf_gemm(tb.data_ptr(), t.data_ptr(), 1, 48, 0, buf.data_ptr(), buf.data_ptr(), c.data_ptr(), 4, 256, 256, None, None))
     x = torch.zeros(12, 256, dtype=torch.float16, device=DEV)
     sel = torch.zeros(12, 2, dtype=torch.int64, device=DEV); sel[:, 1] = 1
     rw = torch.full((12, 2), 0.5, dtype=torch.float16, device=DEV)
@@ -126,7 +126,7 @@ def test_device_tile_planner_matches_host_lists():
             want = {bm: sorted(map(tuple, t.tolist())) for bm, t in M.pf_tiles(segs).items()}
             cap = E + n // 256 + 1
             tiles = torch.full((5, cap, 4), 77, dtype=torch.int32, device=DEV)
-            _lib.check(_lib.lib().nq_pf_plan(cnt.to(DEV).data_ptr(), E, lo, n, tiles.data_ptr(), cap, None))
+            _lib.check(_lib.lib().nq_pf_plan(cnt.to(DEV).data_ptr(), E, lo, n, tiles.data_ptr(), cap, None, 0, 0, None))
             torch.cuda.synchronize()
             t = tiles.cpu()
             for i in range(5):
@@ -138,7 +138,7 @@ def test_device_tile_planner_matches_host_lists():
             total = sum(int(t[i, : (E if i < 4 else cap)][t[i, : (E if i < 4 else cap), 0] >= 0][:, 2].sum()) for i in range(5))
             assert total == n
     with pytest.raises(RuntimeError, match="cap"):
-        _lib.check(_lib.lib().nq_pf_plan(cnt.to(DEV).data_ptr(), 64, 0, 1024, tiles.data_ptr(), 64, None))
+        _lib.check(_lib.lib().nq_pf_plan(cnt.to(DEV).data_ptr(), 64, 0, 1024, tiles.data_ptr(), 64, None, 0, 0, None))
 
 
 def test_prefill_on_a_side_stream_matches_the_default_stream():
@@ -188,7 +188,7 @@ def test_row_restricted_pre_and_mid_cover_the_rows_of_their_heights_exactly():
     pe_d, pt_d = pe.to(DEV), pt.to(DEV)
     cap = E + n // 256 + 1
     tiles = torch.empty(5, cap, 4, dtype=torch.int32, device=DEV)
-    _lib.check(Lb.nq_pf_plan(cnt.int().to(DEV).data_ptr(), E, 0, n, tiles.data_ptr(), cap, None))
+    _lib.check(Lb.nq_pf_plan(cnt.int().to(DEV).data_ptr(), E, 0, n, tiles.data_ptr(), cap, None, 0, 0, None))
     # height class of every row from the host lists
     start = torch.cumsum(cnt, 0) - cnt
     cls = torch.full((n,), 4)

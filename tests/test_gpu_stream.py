@@ -280,6 +280,8 @@ def test_uploads_from_pinned_memory_on_an_engine_without_a_file():
         assert (st["uploads"], st["upload_bytes"], st["posts"], st["upgrades"], st["drives"]) == (1, 8192 + 4096 + RB - 32768, 1, 0, 0)
         with pytest.raises(RuntimeError, match="without a record file"):
             b.upgrade(eng, 0, 0)
+        with pytest.raises(RuntimeError, match="without a record file"):
+            eng.tier_load([0, 1])                                         # no drive to read a tier from (once a division by zero)
         with pytest.raises(RuntimeError, match="spans"):
             eng.upload(3, [(src.data_ptr(), b.slots[0].data_ptr(), 16)] * 9, b.stage[0].data_ptr(), row, b.seq.data_ptr(), 6)
         with pytest.raises(RuntimeError, match="span 0"):
