@@ -247,6 +247,63 @@ __device__ __forceinline__ uint32_t weight_pair(const uint32_t* wb, const uint32
     return pk_fma(code_pair<RES, CODE, JA, JB, BK>(wb, wr, k), k.A2, k.C2);
 }
 
+// ---- two pairs at once, stage by stage --------------------------------------------------------------------------------
+// A wavefront issues an instruction that depends on the one before it only every second or third issue slot, and a SIMD that
+// holds two to four wavefronts then idles part of the time. The decode of one weight is a chain of five to seven dependent
+// instructions, but the weights are independent of each other: here the four weights (JA, JA + 8, JB, JB + 8) go through the
+// chain side by side, each stage for all four before the next, so that four independent instructions separate an instruction
+// from the one that needs its result. The hash multiplies are volatile asm: the compiler keeps them in this order and fits
+// the rest around them. Values and roundings are those of weight_pair.
+template <int O> __device__ __forceinline__ uint32_t window_reg(const uint32_t* w)
+{
+    constexpr int o = (O & 31) >= 16 ? O - 16 : O, i = o >> 5, s = o & 31;
+    if constexpr (s == 0) return w[i]; else return __builtin_amdgcn_alignbit(w[i + 1], w[i], s);
+}
+template <int O> __device__ __forceinline__ uint32_t hash_lo(uint32_t r)
+{
+    uint32_t y;
+    const uint32_t klo = HASH_LO;
+    if constexpr ((O & 31) < 16) asm volatile("v_mad_u32_u16 %0, %1, %2, 0" : "=v"(y) : "v"(r), "s"(klo));
+    else asm volatile("v_mad_u32_u16 %0, %1, %2, 0 op_sel:[1,0,0,0]" : "=v"(y) : "v"(r), "s"(klo));
+    return y;
+}
+template <int O> __device__ __forceinline__ uint32_t hash_hi(uint32_t r, uint32_t y)
+{
+    uint32_t x;
+    const uint32_t khi = HASH_HI_SHL;
+    if constexpr ((O & 31) < 16) asm volatile("v_pk_mad_u16 %0, %1, %2, %3 op_sel:[0,0,0] op_sel_hi:[0,1,1]" : "=v"(x) : "v"(r), "s"(khi), "v"(y));
+    else asm volatile("v_pk_mad_u16 %0, %1, %2, %3 op_sel:[1,0,0] op_sel_hi:[1,1,1]" : "=v"(x) : "v"(r), "s"(khi), "v"(y));
+    return x;
+}
+template <bool RES, int CODE, int JA, int JB, int BK = 0>
+__device__ __forceinline__ void weight_pairs2(const uint32_t* wb, const uint32_t* wr, const FoldK& k, uint32_t& ua, uint32_t& ub)
+{
+    constexpr int B0 = Rec<BK>::off(JA), B1 = Rec<BK>::off(JA + 8), B2 = Rec<BK>::off(JB), B3 = Rec<BK>::off(JB + 8);
+    const uint32_t r0 = window_reg<B0>(wb), r1 = window_reg<B1>(wb), r2 = window_reg<B2>(wb), r3 = window_reg<B3>(wb);
+    const uint32_t y0 = hash_lo<B0>(r0), y1 = hash_lo<B1>(r1), y2 = hash_lo<B2>(r2), y3 = hash_lo<B3>(r3);
+    if constexpr (!RES)
+    {
+        const uint32_t x0 = hash_hi<B0>(r0, y0), x1 = hash_hi<B1>(r1, y1), x2 = hash_hi<B2>(r2, y2), x3 = hash_hi<B3>(r3, y3);
+        const uint32_t ta = __builtin_amdgcn_sad_u8(x0, 0u, 0x64006400u), tb = __builtin_amdgcn_sad_u8(x2, 0u, 0x64006400u);
+        const uint32_t ca = __builtin_amdgcn_sad_hi_u8(x1, 0u, ta), cb = __builtin_amdgcn_sad_hi_u8(x3, 0u, tb);
+        ua = pk_fma(ca, k.A2, k.C2); ub = pk_fma(cb, k.A2, k.C2);
+    }
+    else
+    {
+        constexpr int R0 = Rec<CODE>::off(JA), R1 = Rec<CODE>::off(JA + 8), R2 = Rec<CODE>::off(JB), R3 = Rec<CODE>::off(JB + 8);
+        const uint32_t q0 = window_reg<R0>(wr), q1 = window_reg<R1>(wr), q2 = window_reg<R2>(wr), q3 = window_reg<R3>(wr);
+        const uint32_t z0 = hash_lo<R0>(q0), z1 = hash_lo<R1>(q1), z2 = hash_lo<R2>(q2), z3 = hash_lo<R3>(q3);
+        const uint32_t x0 = hash_hi<B0>(r0, y0), x1 = hash_hi<B1>(r1, y1), x2 = hash_hi<B2>(r2, y2), x3 = hash_hi<B3>(r3, y3);
+        const uint32_t v0 = hash_hi<R0>(q0, z0), v1 = hash_hi<R1>(q1, z1), v2 = hash_hi<R2>(q2, z2), v3 = hash_hi<R3>(q3, z3);
+        uint32_t t0 = __builtin_amdgcn_udot4(x0, k.Mrep, 0x640080u, false), t1 = __builtin_amdgcn_udot4(x1, k.Mrep, 0x640080u, false);
+        uint32_t t2 = __builtin_amdgcn_udot4(x2, k.Mrep, 0x640080u, false), t3 = __builtin_amdgcn_udot4(x3, k.Mrep, 0x640080u, false);
+        t0 = __builtin_amdgcn_udot4(v0, k.Nrep, t0, false); t1 = __builtin_amdgcn_udot4(v1, k.Nrep, t1, false);
+        t2 = __builtin_amdgcn_udot4(v2, k.Nrep, t2, false); t3 = __builtin_amdgcn_udot4(v3, k.Nrep, t3, false);
+        const uint32_t ca = __builtin_amdgcn_perm(t1, t0, 0x06050201u), cb = __builtin_amdgcn_perm(t3, t2, 0x06050201u);
+        ua = pk_fma(ca, k.A2, k.C2); ub = pk_fma(cb, k.A2, k.C2);
+    }
+}
+
 // ---- table row ------------------------------------------------------------------------------------------------------
 // int64[20] per expert (reference sm120/moe.py:216-229, sm120/nqmoe.cu:26-45):
 //   [0] level 0/2/3/4  [1..4] gate|up base, residual plane, block words, flags (mask mode, 0 = dense)  [5..8] down  [9] sign/scale vector
