@@ -260,19 +260,14 @@ template <int O> __device__ __forceinline__ uint32_t window_reg(const uint32_t* 
     if constexpr (s == 0) return w[i]; else return __builtin_amdgcn_alignbit(w[i + 1], w[i], s);
 }
 template <int O> __device__ __forceinline__ uint32_t hash_lo(uint32_t r)
-{
-    uint32_t y;
-    const uint32_t klo = HASH_LO;
-    if constexpr ((O & 31) < 16) asm volatile("v_mad_u32_u16 %0, %1, %2, 0" : "=v"(y) : "v"(r), "s"(klo));
-    else asm volatile("v_mad_u32_u16 %0, %1, %2, 0 op_sel:[1,0,0,0]" : "=v"(y) : "v"(r), "s"(klo));
-    return y;
+{   // the clean 16-bit state (an and / a shift: double-rate instructions on gfx950)
+    if constexpr ((O & 31) < 16) return r & 0xFFFFu; else return r >> 16;
 }
-template <int O> __device__ __forceinline__ uint32_t hash_hi(uint32_t r, uint32_t y)
+template <int O> __device__ __forceinline__ uint32_t hash_hi(uint32_t, uint32_t st)
 {
     uint32_t x;
-    const uint32_t khi = HASH_HI_SHL;
-    if constexpr ((O & 31) < 16) asm volatile("v_pk_mad_u16 %0, %1, %2, %3 op_sel:[0,0,0] op_sel_hi:[0,1,1]" : "=v"(x) : "v"(r), "s"(khi), "v"(y));
-    else asm volatile("v_pk_mad_u16 %0, %1, %2, %3 op_sel:[1,0,0] op_sel_hi:[1,1,1]" : "=v"(x) : "v"(r), "s"(khi), "v"(y));
+    const uint32_t hc = HASH_LO | HASH_HI_SHL;
+    asm volatile("v_mul_lo_u32 %0, %1, %2" : "=v"(x) : "v"(st), "s"(hc));
     return x;
 }
 template <bool RES, int CODE, int JA, int JB, int BK = 0>
