@@ -522,18 +522,29 @@ __device__ __forceinline__ void pf_mfmas(const half8_t (*aop)[2], const char* sm
 // picks which 16-byte column of its row it fetches: column (lane & 15) ^ (row & 15) goes to slot lane & 15, and the MFMA reads
 // undo the XOR, which spreads the 16 tokens of an operand read over all banks without padding. Rows beyond the tile re-read
 // its last row: their products are never stored.
-template <int TG>
+// PART = 0 .. 3 issues a quarter of the loads (all of them in part 0 when there are fewer than four): the decode-fused body
+// spreads them over its decode, because the texture path takes 16 clocks per 1 KB load and a wavefront that issues sixteen in
+// a row stalls behind its own requests (measured: 1450 clocks per chunk at 256 rows) with the record loads queued after them.
+template <int TG, int PART = -1>
 __device__ __forceinline__ void pf_stage_tokens(const _Float16* A, int K, int row0, int nrows, int c, char* smem, int warp, int srow, uint32_t scol)
 {
     typedef const __attribute__((address_space(1))) void* gvp;
     typedef __attribute__((address_space(3))) void* lvp;
+    constexpr int U0 = PART < 0 ? 0 : (TG >= 4 ? PART * (TG / 4) : 0), U1 = PART < 0 ? TG : (TG >= 4 ? U0 + TG / 4 : (PART == 0 ? TG : 0));
+    // uniform base of the tile's chunk (scalar registers) + a 32-bit lane offset inside the tile; the offset passes through an
+    // empty asm so that the addresses of a part are formed when the part is issued, not sixteen of them ahead of the decode
+    const char* base = (const char*)A + ((size_t)row0 * K + c * 128) * 2;
+    uint32_t lane_off = (uint32_t)(srow * K * 2) + scol;
+    asm volatile("" : "+v"(lane_off));
+    const uint32_t ustep = (uint32_t)(16 * K * 2);
+    const uint32_t last_off = (uint32_t)((nrows - 1) * K * 2) + scol;
 #pragma unroll
-    for (int u = 0; u < TG; ++u)
+    for (int u = U0; u < U1; ++u)
     {
-        if (16 * u >= nrows) break;                              // block-uniform
-        const int row = 16 * u + srow, grow = row < nrows ? row : nrows - 1;
-        const char* src = (const char*)A + ((size_t)(row0 + grow) * K + c * 128) * 2 + scol;
-        __builtin_amdgcn_global_load_lds((gvp)src, (lvp)(smem + (16 * u + 4 * warp) * PF_ROW), 16, 0, 0);
+        if constexpr (PART < 0) { if (16 * u >= nrows) break; }  // block-uniform; the spread parts stay free of branches
+        uint32_t off = lane_off + (uint32_t)u * ustep;
+        off = 16 * u + srow < nrows ? off : last_off;
+        __builtin_amdgcn_global_load_lds((gvp)(base + off), (lvp)(smem + (16 * u + 4 * warp) * PF_ROW), 16, 0, 0);
     }
 }
 
@@ -598,9 +609,8 @@ __device__ __forceinline__ void pf_chunks(const Planes& P, const LaneCtx& L, int
     typedef __attribute__((address_space(3))) void* lvp;
     for (int c = 0; c < C; ++c)
     {
-        // ---- request the tile's tokens for chunk c (asynchronous: the decode below runs while they arrive)
-        pf_stage_tokens<TG>(A, K, row0, nrows, c, smem, warp, srow, scol);
-        // ---- decode this wave's unit pair of chunk c into A operands; prefetch chunk c + 1
+        // ---- decode this wave's unit pair of chunk c into A operands; prefetch chunk c + 1; request the tile's tokens for chunk c
+        // a quarter at a time between the decode stages (asynchronous: they arrive while the decode runs)
         uint32_t wb[6], wr[NW + 2];
         wb[0] = nb.x; wb[1] = nb.y; wb[2] = nb.z; wb[3] = nb.w;
 #pragma unroll
@@ -631,6 +641,7 @@ __device__ __forceinline__ void pf_chunks(const Planes& P, const LaneCtx& L, int
                 const FoldK k = consts_fold(dw, sgm);
                 static_for<4>([&](auto mm) {
                     constexpr int MM = decltype(mm)::value;
+                    pf_stage_tokens<TG, MM>(A, K, row0, nrows, c, smem, warp, srow, scol);
                     aop[MM][0] = a_operand<RES, CODE, MM, 0, BK>(wb, wr, k);
                     aop[MM][1] = a_operand<RES, CODE, MM, 1, BK>(wb, wr, k);
                 });
@@ -641,6 +652,7 @@ __device__ __forceinline__ void pf_chunks(const Planes& P, const LaneCtx& L, int
             const FoldK k = consts_l2(sgm);
             static_for<4>([&](auto mm) {
                 constexpr int MM = decltype(mm)::value;
+                pf_stage_tokens<TG, MM>(A, K, row0, nrows, c, smem, warp, srow, scol);
                 aop[MM][0] = a_operand<false, 0, MM, 0, BK>(wb, wr, k);
                 aop[MM][1] = a_operand<false, 0, MM, 1, BK>(wb, wr, k);
             });
