@@ -22,8 +22,7 @@
 namespace nq {
 
 constexpr int TBL_W = 20;                       // int64 words per table row (reference sm120/moe.py:6)
-constexpr uint32_t HASH_LO = 0xD12Du;           // 0x83DCD12D = HASH_HI << 16 | HASH_LO
-constexpr uint32_t HASH_HI_SHL = 0x83DC0000u;   // high multiplier in the upper half, zero in the lower half
+constexpr uint32_t HASH_MUL = 0x83DCD12Du;      // state -> 32-bit hash (reference sm120/moe.py:115, sm120/nqmoe.cu:79)
 constexpr uint32_t MUL1_A2 = 0x1eee1eeeu;       // fp16 A twice
 constexpr uint32_t MUL1_B2 = 0xc931c931u;       // fp16 B twice
 constexpr int CODE_L3 = 10, CODE_L4N = 11;      // nested planes of this build: K=1 plane; P3 record || P4 record
@@ -160,34 +159,28 @@ __device__ __forceinline__ void ext_words(uint32_t* w, uint32_t nb)
 }
 
 // ---- hash -----------------------------------------------------------------------------------------------------------
-// x = st * 0x83DCD12D mod 2^32 with st = the low (HI = false) or high (HI = true) 16 bits of r; other bits ignored.
-template <bool HI>
-__device__ __forceinline__ uint32_t hash16(uint32_t r)
+// x = st * 0x83DCD12D mod 2^32 for the 16-bit window st at bit offset O of the extended record w[]. Windows O and O + 16 share
+// one register (window_reg); state() takes the low or the high half of it (an and / a shift, which the compiler merges with
+// the funnel shift into one bit-field extract where the window lies inside a word), times_hash() is the 32-bit multiply
+// (on gfx950 it issues at the rate of the 16-bit multiply-adds it replaces, two per weight before). The
+// multiply is volatile asm so that code which lays several weights side by side keeps that order (weight_pairs2).
+template <int O> __device__ __forceinline__ uint32_t window_reg(const uint32_t* w)
 {
-    uint32_t y, x;
-    const uint32_t klo = HASH_LO, khi = HASH_HI_SHL;
-    if constexpr (!HI)
-    {
-        asm("v_mad_u32_u16 %0, %1, %2, 0" : "=v"(y) : "v"(r), "s"(klo));
-        asm("v_pk_mad_u16 %0, %1, %2, %3 op_sel:[0,0,0] op_sel_hi:[0,1,1]" : "=v"(x) : "v"(r), "s"(khi), "v"(y));
-    }
-    else
-    {
-        asm("v_mad_u32_u16 %0, %1, %2, 0 op_sel:[1,0,0,0]" : "=v"(y) : "v"(r), "s"(klo));
-        asm("v_pk_mad_u16 %0, %1, %2, %3 op_sel:[1,0,0] op_sel_hi:[1,1,1]" : "=v"(x) : "v"(r), "s"(khi), "v"(y));
-    }
+    constexpr int o = (O & 31) >= 16 ? O - 16 : O, i = o >> 5, s = o & 31;
+    if constexpr (s == 0) return w[i]; else return __builtin_amdgcn_alignbit(w[i + 1], w[i], s);
+}
+template <int O> __device__ __forceinline__ uint32_t state(uint32_t r)
+{
+    if constexpr ((O & 31) < 16) return r & 0xFFFFu; else return r >> 16;
+}
+__device__ __forceinline__ uint32_t times_hash(uint32_t st)
+{
+    uint32_t x;
+    const uint32_t hc = HASH_MUL;
+    asm volatile("v_mul_lo_u32 %0, %1, %2" : "=v"(x) : "v"(st), "s"(hc));
     return x;
 }
-// hash of the 16-bit window at bit offset O of the extended record w[]. Windows O and O + 16 share one register.
-template <int O>
-__device__ __forceinline__ uint32_t hash_at(const uint32_t* w)
-{
-    constexpr bool HI = (O & 31) >= 16;
-    constexpr int o = HI ? O - 16 : O, i = o >> 5, s = o & 31;
-    uint32_t r;
-    if constexpr (s == 0) r = w[i]; else r = __builtin_amdgcn_alignbit(w[i + 1], w[i], s);
-    return hash16<HI>(r);
-}
+template <int O> __device__ __forceinline__ uint32_t hash_at(const uint32_t* w) { return times_hash(state<O>(window_reg<O>(w))); }
 
 // ---- per-unit constants ---------------------------------------------------------------------------------------------
 struct FoldK { uint32_t Mrep, Nrep, A2, C2; };      // Mb and N replicated into 4 bytes; fp16 A', C replicated twice
@@ -248,37 +241,22 @@ __device__ __forceinline__ uint32_t weight_pair(const uint32_t* wb, const uint32
 }
 
 // ---- two pairs at once, stage by stage --------------------------------------------------------------------------------
-// A wavefront issues an instruction that depends on the one before it only every second or third issue slot, and a SIMD that
-// holds two to four wavefronts then idles part of the time. The decode of one weight is a chain of five to seven dependent
-// instructions, but the weights are independent of each other: here the four weights (JA, JA + 8, JB, JB + 8) go through the
+// A wavefront cannot issue an instruction right behind the one whose result it needs, and a SIMD that holds only two to four
+// wavefronts then idles part of the time. The decode of one weight is a chain of five to seven dependent instructions, but
+// the weights are independent of each other: here the four weights (JA, JA + 8, JB, JB + 8) go through the
 // chain side by side, each stage for all four before the next, so that four independent instructions separate an instruction
 // from the one that needs its result. The hash multiplies are volatile asm: the compiler keeps them in this order and fits
-// the rest around them. Values and roundings are those of weight_pair.
-template <int O> __device__ __forceinline__ uint32_t window_reg(const uint32_t* w)
-{
-    constexpr int o = (O & 31) >= 16 ? O - 16 : O, i = o >> 5, s = o & 31;
-    if constexpr (s == 0) return w[i]; else return __builtin_amdgcn_alignbit(w[i + 1], w[i], s);
-}
-template <int O> __device__ __forceinline__ uint32_t hash_lo(uint32_t r)
-{   // the clean 16-bit state (an and / a shift: double-rate instructions on gfx950)
-    if constexpr ((O & 31) < 16) return r & 0xFFFFu; else return r >> 16;
-}
-template <int O> __device__ __forceinline__ uint32_t hash_hi(uint32_t, uint32_t st)
-{
-    uint32_t x;
-    const uint32_t hc = HASH_LO | HASH_HI_SHL;
-    asm volatile("v_mul_lo_u32 %0, %1, %2" : "=v"(x) : "v"(st), "s"(hc));
-    return x;
-}
+// the rest around them (measured at two wavefronts per SIMD: 2.39 -> 2.02 ns per instruction; at four 2.03 -> 1.85). Values
+// and roundings are those of weight_pair.
 template <bool RES, int CODE, int JA, int JB, int BK = 0>
 __device__ __forceinline__ void weight_pairs2(const uint32_t* wb, const uint32_t* wr, const FoldK& k, uint32_t& ua, uint32_t& ub)
 {
     constexpr int B0 = Rec<BK>::off(JA), B1 = Rec<BK>::off(JA + 8), B2 = Rec<BK>::off(JB), B3 = Rec<BK>::off(JB + 8);
     const uint32_t r0 = window_reg<B0>(wb), r1 = window_reg<B1>(wb), r2 = window_reg<B2>(wb), r3 = window_reg<B3>(wb);
-    const uint32_t y0 = hash_lo<B0>(r0), y1 = hash_lo<B1>(r1), y2 = hash_lo<B2>(r2), y3 = hash_lo<B3>(r3);
+    const uint32_t y0 = state<B0>(r0), y1 = state<B1>(r1), y2 = state<B2>(r2), y3 = state<B3>(r3);
     if constexpr (!RES)
     {
-        const uint32_t x0 = hash_hi<B0>(r0, y0), x1 = hash_hi<B1>(r1, y1), x2 = hash_hi<B2>(r2, y2), x3 = hash_hi<B3>(r3, y3);
+        const uint32_t x0 = times_hash(y0), x1 = times_hash(y1), x2 = times_hash(y2), x3 = times_hash(y3);
         const uint32_t ta = __builtin_amdgcn_sad_u8(x0, 0u, 0x64006400u), tb = __builtin_amdgcn_sad_u8(x2, 0u, 0x64006400u);
         const uint32_t ca = __builtin_amdgcn_sad_hi_u8(x1, 0u, ta), cb = __builtin_amdgcn_sad_hi_u8(x3, 0u, tb);
         ua = pk_fma(ca, k.A2, k.C2); ub = pk_fma(cb, k.A2, k.C2);
@@ -287,9 +265,9 @@ __device__ __forceinline__ void weight_pairs2(const uint32_t* wb, const uint32_t
     {
         constexpr int R0 = Rec<CODE>::off(JA), R1 = Rec<CODE>::off(JA + 8), R2 = Rec<CODE>::off(JB), R3 = Rec<CODE>::off(JB + 8);
         const uint32_t q0 = window_reg<R0>(wr), q1 = window_reg<R1>(wr), q2 = window_reg<R2>(wr), q3 = window_reg<R3>(wr);
-        const uint32_t z0 = hash_lo<R0>(q0), z1 = hash_lo<R1>(q1), z2 = hash_lo<R2>(q2), z3 = hash_lo<R3>(q3);
-        const uint32_t x0 = hash_hi<B0>(r0, y0), x1 = hash_hi<B1>(r1, y1), x2 = hash_hi<B2>(r2, y2), x3 = hash_hi<B3>(r3, y3);
-        const uint32_t v0 = hash_hi<R0>(q0, z0), v1 = hash_hi<R1>(q1, z1), v2 = hash_hi<R2>(q2, z2), v3 = hash_hi<R3>(q3, z3);
+        const uint32_t z0 = state<R0>(q0), z1 = state<R1>(q1), z2 = state<R2>(q2), z3 = state<R3>(q3);
+        const uint32_t x0 = times_hash(y0), x1 = times_hash(y1), x2 = times_hash(y2), x3 = times_hash(y3);
+        const uint32_t v0 = times_hash(z0), v1 = times_hash(z1), v2 = times_hash(z2), v3 = times_hash(z3);
         uint32_t t0 = __builtin_amdgcn_udot4(x0, k.Mrep, 0x640080u, false), t1 = __builtin_amdgcn_udot4(x1, k.Mrep, 0x640080u, false);
         uint32_t t2 = __builtin_amdgcn_udot4(x2, k.Mrep, 0x640080u, false), t3 = __builtin_amdgcn_udot4(x3, k.Mrep, 0x640080u, false);
         t0 = __builtin_amdgcn_udot4(v0, k.Nrep, t0, false); t1 = __builtin_amdgcn_udot4(v1, k.Nrep, t1, false);

@@ -402,7 +402,6 @@ struct PfGemm
     float* C; int mode, E, H, I;
     int solo;                                       // the other kernel variant will not be launched on these tiles: a tile that is its kind comes out NaN
     const u32x4* Wop;                               // decoded weights of hot experts in A-operand order (nq_pf_wdecode_k), or null
-    int skip_hot;                                   // leave the 256-row tiles of hot experts to nq_pf_dense_k
 };
 
 // ---- decoded-weight scratch of hot experts --------------------------------------------------------------------------------
@@ -709,7 +708,6 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) n
     {
         // a hot expert (several tiles): its weights were decoded once into the scratch by nq_pf_wdecode_k (block-uniform)
         const bool pre = a.Wop != nullptr && slot >= 0 && P.flags == nullptr;
-        if (pre && a.skip_hot) return;                           // nq_pf_dense_k has this tile
         if (pre) pf_chunks_pre<TG>(a.Wop + wop_base(slot, a.mode, a.H, a.I) + (size_t)sp * C * 8 * 64, C, A, K, row0, nrows, smem, acc);
         else if (lv == 2) pf_chunks<TG, false, 0, false>(P, L, C, A, K, row0, nrows, smem, acc);
         else dispatch_code(P.code, [&](auto tag) { pf_chunks<TG, true, decltype(tag)::value, false>(P, L, C, A, K, row0, nrows, smem, acc); });
@@ -784,7 +782,7 @@ int launch_pf_gemm(const int64_t* table, const int32_t* tiles, int ntiles, int b
                    int E, int H, int I, const void* Wop, hipStream_t st)
 {
     if (!ntiles) return 0;
-    PfGemm a{table, tiles, (const _Float16*)A0, (const _Float16*)A1, C, mode & 1, E, H, I, (mode & 4) != 0, (const u32x4*)Wop, 0};
+    PfGemm a{table, tiles, (const _Float16*)A0, (const _Float16*)A1, C, mode & 1, E, H, I, (mode & 4) != 0, (const u32x4*)Wop};
     const int N = (mode & 1) == 0 ? 2 * I : H;
     const bool masked = (mode & 2) != 0;
     switch (bm)

@@ -66,24 +66,13 @@ __device__ __forceinline__ int bop_index(int c)
 }
 
 // A operand of MFMA (MM, RHO): rows g + 8 RHO, columns of t = 2 MM and 2 MM + 1
-// WIDE = false decodes pair by pair (fewer registers in flight, for the kernel that has none to spare)
-template <bool RES, int CODE, int MM, int RHO, int BK = 0, bool WIDE = true>
+template <bool RES, int CODE, int MM, int RHO, int BK = 0>
 __device__ __forceinline__ half8_t a_operand(const uint32_t* wb, const uint32_t* wr, const FoldK& k)
 {
     constexpr int J = 16 * MM + 2 * RHO;
     uint32_t u[4];
-    if constexpr (WIDE)
-    {
-        weight_pairs2<RES, CODE, J + 0, J + 1, BK>(wb, wr, k, u[0], u[1]);
-        weight_pairs2<RES, CODE, J + 4, J + 5, BK>(wb, wr, k, u[2], u[3]);
-    }
-    else
-    {
-        u[0] = weight_pair<RES, CODE, J + 0, J + 8, BK>(wb, wr, k);
-        u[1] = weight_pair<RES, CODE, J + 1, J + 9, BK>(wb, wr, k);
-        u[2] = weight_pair<RES, CODE, J + 4, J + 12, BK>(wb, wr, k);
-        u[3] = weight_pair<RES, CODE, J + 5, J + 13, BK>(wb, wr, k);
-    }
+    weight_pairs2<RES, CODE, J + 0, J + 1, BK>(wb, wr, k, u[0], u[1]);
+    weight_pairs2<RES, CODE, J + 4, J + 5, BK>(wb, wr, k, u[2], u[3]);
     return __builtin_bit_cast(half8_t, *(u32x4*)u);
 }
 
