@@ -29,7 +29,7 @@ HBM_PEAK_GBS = 8000.0
 MFMA_PEAK_TFLOPS = 2500.0            # dense fp16 / bf16 MFMA peak of MI355X
 # HBM bytes per gate|up launch / algorithmic bytes, from rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a 256 MiB copy kernel
 # (profiles/decode_gemv_hbm_traffic_pmc.txt)
-TRAFFIC_RATIO = 1.029
+TRAFFIC_RATIO = 1.038
 
 
 def build_layer(dev, seed=0, Bmax=4):
@@ -237,6 +237,7 @@ def prefill_leg(L, ex, dev, T=4096, reps=3):
     want = O.moe_forward(dense, [4] * E, signs, x[toks].cpu().numpy(), sel[toks].cpu().numpy(), rw[toks].cpu().numpy(), dtype=np.float64)
     rel = float(np.linalg.norm(y[toks].cpu().numpy() - want) / np.linalg.norm(want))
     assert rel < 1e-3, f"prefill output of tokens {toks} is {rel:.2e} from the oracle"
+    parts = prefill_parts(L, x, sel, dev)
     L.table.copy_(saved)
     flops = T * TOPK * 6 * H * I
     cnt = torch.bincount(sel.flatten().cpu(), minlength=E)
@@ -244,7 +245,59 @@ def prefill_leg(L, ex, dev, T=4096, reps=3):
                          f"rows per expert max {int(cnt.max())} / median {int(cnt.median())}",
                 ms=round(dt * 1e3, 3), tflops=round(flops / dt / 1e12, 1), flop=flops, mfma_peak_tflops=MFMA_PEAK_TFLOPS,
                 mfma_frac=round(flops / dt / 1e12 / MFMA_PEAK_TFLOPS, 4), rel_err_vs_oracle=float(f"{rel:.2e}"), checked_tokens=toks,
-                note="whole prefill() call: sort, pre, 2 decode-fused grouped GEMMs, mid, post; bound by the VALU trellis decode")
+                launches_alone=parts,
+                note="whole prefill() call: sort, plan, hot-expert decode, then per tile height pre, gate|up GEMM, mid, down GEMM on "
+                     "concurrent streams, post; the GEMMs decode their weights in the kernel and are bound by the issue rate of the "
+                     "decode's vector instructions")
+
+
+def prefill_parts(L, x, sel, dev):
+    """the grouped-GEMM launches of one prefill() call timed one at a time on one stream (inside the call they overlap on four
+    streams and their durations stretch): per tile height the tiles, pair rows, us of the gate|up and the down launch, and
+    the MFMA fraction of that height alone; plus the two launches that decode the hot experts into the operand scratch"""
+    from nestquant_amd import _lib
+    T = x.shape[0]
+    Lb, tb, P = L.M, L.table, T * TOPK
+    flat = sel.reshape(-1)
+    order = torch.argsort(flat, stable=True)
+    pe, pt = flat[order].int(), (order // TOPK).int()
+    cnt = torch.zeros(E, dtype=torch.int32, device=dev).scatter_add_(0, flat, torch.ones_like(flat, dtype=torch.int32))
+    S = M.pf_scratch(dev, H, I, P)
+    cap, st, wop = E + P // 256 + 1, _lib.stream_ptr(), S["wop"]
+    tiles = torch.empty(5, cap, 4, dtype=torch.int32, device=dev)
+    hot = torch.empty(E, dtype=torch.int32, device=dev)
+    nslot, wptr = (wop.shape[0], wop.data_ptr()) if wop is not None else (0, None)
+    hot.fill_(-1)
+    _lib.check(Lb.nq_pf_plan(cnt.data_ptr(), E, 0, P, tiles.data_ptr(), cap, hot.data_ptr() if nslot else None, M.PF_HOT_MIN, nslot, st))
+    _lib.check(Lb.nq_pf_pre(x.data_ptr(), pt.data_ptr(), pe.data_ptr(), P, tb.data_ptr(), S["xg"].data_ptr(), S["xu"].data_ptr(),
+                            S["zg"].data_ptr(), E, H, I, st))
+
+    def us(fn, reps=3):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / reps
+    rec = dict(hot_experts=int((hot >= 0).sum()), wdecode_us=[round(us(lambda m=m: _lib.check(Lb.nq_pf_wdecode(
+        tb.data_ptr(), hot.data_ptr(), E, m, wptr, wop.numel() * 2, nslot, H, I, st))), 0) for m in (0, 1)] if nslot else [])
+    tl, tot = tiles.cpu(), 0.0
+    for i in (4, 3, 2, 1, 0):
+        bm, nt = 16 << i, (E if i < 4 else cap)
+        valid = tl[i, :nt, 0] >= 0
+        rows = int(tl[i, :nt, 2][valid].sum())
+        gu = us(lambda: _lib.check(Lb.nq_pf_gemm(tb.data_ptr(), tiles[i].data_ptr(), nt, bm, 4, S["xg"].data_ptr(), S["xu"].data_ptr(),
+                                                 S["acc"].data_ptr(), E, H, I, wptr, st)))
+        dn = us(lambda: _lib.check(Lb.nq_pf_gemm(tb.data_ptr(), tiles[i].data_ptr(), nt, bm, 5, S["h"].data_ptr(), None,
+                                                 S["y"].data_ptr(), E, H, I, wptr, st)))
+        tot += gu + dn
+        rec[f"height_{bm}"] = dict(tiles=int(valid.sum()), hot_tiles=int((tl[i, :nt, 3][valid] > 0).sum()), rows=rows, gate_up_us=round(gu, 0),
+                                   down_us=round(dn, 0), mfma_frac=round(rows * 6 * H * I / (gu + dn) / 1e6 / MFMA_PEAK_TFLOPS, 3))
+    rec["sum_us"] = round(tot, 0)
+    return rec
 
 
 def batch_leg(L, MB, ex, levels, dev, R=32, blocks=8):

@@ -158,7 +158,7 @@ int main(int argc, char** argv)
     for (int st = 0; st < steps; ++st) { a.sel = sel + (size_t)st * S; NQCHK(nq_moe_forward(&a, nullptr)); }
     HIPCHK(hipEventRecord(e1, nullptr)); HIPCHK(hipEventSynchronize(e1));
     float ms; HIPCHK(hipEventElapsedTime(&ms, e0, e1));
-    printf("nq_bench_native: E=%d B=%d steps=%d  %.2f us per layer call (eager launches, 2 kernels per call); resident planes %.1f MB\n",
+    printf("nq_bench_native: E=%d B=%d steps=%d  %.2f us per layer call (eager launches, 3 kernels per call); resident planes %.1f MB\n",
            E, B, steps, ms * 1e3 / steps, plane_bytes / 1e6);
     return 0;
 }
