@@ -12,6 +12,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libnq_moe_hip.so")
 NATIVE = os.path.join(HERE, "nq_bench_native")
+PROBE = os.path.join(HERE, "nq_issue_probe")
 OBJ = os.path.join(HERE, "build")
 ARCH = "gfx950"
 FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-ffp-contract=off",
@@ -49,6 +50,9 @@ def build(verbose=False, jobs=None):
     # torch-free driver of the C ABI (timing cross-check and the program rocprofv3 counter passes wrap)
     _run([hipcc, "-O2", "-std=c++17", f"--offload-arch={ARCH}", "-x", "hip", os.path.join(CSRC, "nq_bench_native.cpp"),
           "-o", NATIVE, "-L" + HERE, "-lnq_moe_hip", "-Wl,-rpath,$ORIGIN", "-Wno-unused-command-line-argument", "-Wno-unused-result"])
+    # stand-alone probe of the vector-instruction issue rates the decoder's design rests on (no library, no inputs)
+    _run([hipcc, "-O3", "-std=c++17", f"--offload-arch={ARCH}", "-x", "hip", os.path.join(CSRC, "nq_issue_probe.cpp"),
+          "-o", PROBE, "-Wno-unused-command-line-argument"])
     return LIB
 
 
