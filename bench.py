@@ -238,6 +238,20 @@ def prefill_leg(L, ex, dev, T=4096, reps=3):
     rel = float(np.linalg.norm(y[toks].cpu().numpy() - want) / np.linalg.norm(want))
     assert rel < 1e-3, f"prefill output of tokens {toks} is {rel:.2e} from the oracle"
     parts = prefill_parts(L, x, sel, dev)
+    # the same call with the operand scratch for experts of several tiles switched on (32 slots; off by default)
+    M.PF_HOT_SLOTS = 32
+    try:
+        yh = L.prefill(x, sel, rw)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            L.prefill(x, sel, rw)
+        torch.cuda.synchronize()
+        hot_ms = (time.perf_counter() - t0) / reps * 1e3
+        assert torch.equal(yh, y), "the hot-expert scratch changed the result"
+        hot_parts = prefill_parts(L, x, sel, dev)
+    finally:
+        M.PF_HOT_SLOTS = 0
     L.table.copy_(saved)
     flops = T * TOPK * 6 * H * I
     cnt = torch.bincount(sel.flatten().cpu(), minlength=E)
@@ -246,6 +260,8 @@ def prefill_leg(L, ex, dev, T=4096, reps=3):
                 ms=round(dt * 1e3, 3), tflops=round(flops / dt / 1e12, 1), flop=flops, mfma_peak_tflops=MFMA_PEAK_TFLOPS,
                 mfma_frac=round(flops / dt / 1e12 / MFMA_PEAK_TFLOPS, 4), rel_err_vs_oracle=float(f"{rel:.2e}"), checked_tokens=toks,
                 launches_alone=parts,
+                with_hot_scratch=dict(ms=round(hot_ms, 3), result="bitwise equal", hot_experts=hot_parts["hot_experts"],
+                                      wdecode_us=hot_parts["wdecode_us"], height_256=hot_parts["height_256"], sum_us=hot_parts["sum_us"]),
                 note="whole prefill() call: sort, plan, hot-expert decode, then per tile height pre, gate|up GEMM, mid, down GEMM on "
                      "concurrent streams, post; the GEMMs decode their weights in the kernel and are bound by the issue rate of the "
                      "decode's vector instructions")

@@ -261,9 +261,11 @@ class MoELayer:
 
 _PF = {}
 PF_TILES = (16, 32, 64, 128, 256)            # token-tile heights the grouped GEMM is compiled for
-# An expert with at least PF_HOT_MIN pair rows in a chunk (more than one 256-row tile) is decoded once per call into a scratch of
-# decoded weights (at most PF_HOT_SLOTS experts at 6 H I bytes each) instead of once per tile; see nq_pf_wdecode.
-PF_HOT_MIN, PF_HOT_SLOTS = 257, 32
+# An expert with at least PF_HOT_MIN pair rows in a chunk (more than one 256-row tile) can be decoded once per call into a scratch
+# of decoded weights (at most PF_HOT_SLOTS experts at 6 H I bytes each) instead of once per tile; see nq_pf_wdecode. Off by
+# default (0 slots): a tile then reads 75 MB of fp16 operands from HBM where the decode-fused kernel reads 12.6 MB of codes, and
+# on the 4096-token benchmark the call takes 6.7 ms with 32 slots against 6.6 ms without. Same bits either way.
+PF_HOT_MIN, PF_HOT_SLOTS = 257, 0
 
 
 def pf_bytes(H, I, R, G=0):
@@ -277,7 +279,7 @@ def pf_scratch(dev, H, I, R, G=0):
     h fp16 [R, I], y fp32 [R, H], and wop: decoded weights of up to PF_HOT_SLOTS hot experts. Unlike the reference
     (sm120/moe.py:263-274), which decodes every expert of a group into dense scratch, only experts with more than one tile go
     through scratch; the others are decoded in registers inside the grouped GEMM."""
-    k = (str(dev), H, I, R)
+    k = (str(dev), H, I, R, PF_HOT_SLOTS)
     if k not in _PF:
         f16, f32 = torch.float16, torch.float32
         slots = max(0, min(PF_HOT_SLOTS, R // PF_HOT_MIN))

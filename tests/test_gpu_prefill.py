@@ -89,6 +89,37 @@ def test_full_shape_prefill_vs_decode_slices():
     assert rel_err(y[idx].cpu().numpy(), want) < 5e-5
 
 
+def test_hot_expert_scratch_gives_the_same_bits():
+    """experts with more than one 256-row tile decoded once into the operand scratch (nq_pf_wdecode, off by default): the
+    grouped GEMM multiplies the same operands in the same order, so the result is bitwise the one of the decode-fused tiles"""
+    H, I, NE, T = 1024, 512, 6, 700
+    levels = [4, 2, 3, 4, 2, 4]
+    ex = to_dev(experts_on_gpu(H, I, NE, 900, nested_ids=(0, 2, 4)))
+    L = M.MoELayer(NE, H, I, Bmax=8)
+    for e in range(NE):
+        L.set(e, ex[e], levels[e])
+    sel, rw = gumbel_topk(T, NE, 2, seed=5)
+    g = torch.Generator().manual_seed(6)
+    x = (torch.randn(T, H, generator=g) * 0.05).half().to(DEV)
+    assert M.PF_HOT_SLOTS == 0
+    y0 = L.prefill(x, sel, rw)
+    torch.cuda.synchronize()
+    cnt = torch.bincount(sel.flatten().cpu(), minlength=NE)
+    assert int((cnt >= M.PF_HOT_MIN).sum()) >= 2                  # several experts qualify
+    try:
+        M.PF_HOT_SLOTS = 1                                       # fewer slots than hot experts: the rest keep decoding per tile
+        y1 = L.prefill(x, sel, rw)
+        M.PF_HOT_SLOTS = 4
+        y2 = L.prefill(x, sel, rw)
+        torch.cuda.synchronize()
+    finally:
+        M.PF_HOT_SLOTS = 0
+    assert torch.equal(y0, y1) and torch.equal(y0, y2)
+    ys = sliced_decode(L, x, sel, rw)
+    torch.cuda.synchronize()
+    assert rel_err(y0.cpu().numpy(), ys.cpu().numpy()) < 5e-5
+
+
 def test_prefill_argument_errors_and_empty():
     L = M.MoELayer(4, 256, 256, Bmax=2, topk=2)
     tb = L.table
