@@ -264,7 +264,8 @@ PF_TILES = (16, 32, 64, 128, 256)            # token-tile heights the grouped GE
 # An expert with at least PF_HOT_MIN pair rows in a chunk (more than one 256-row tile) can be decoded once per call into a scratch
 # of decoded weights (at most PF_HOT_SLOTS experts at 6 H I bytes each) instead of once per tile; see nq_pf_wdecode. Off by
 # default (0 slots): a tile then reads 75 MB of fp16 operands from HBM where the decode-fused kernel reads 12.6 MB of codes, and
-# on the 4096-token benchmark the call takes 6.7 ms with 32 slots against 6.6 ms without. Same bits either way.
+# on the 4096-token benchmark the call takes 6.59-6.65 ms with 32 slots against 6.58-6.61 ms without (the tiles save 0.4 ms, the
+# decode launches cost 0.57 ms) plus 2.4 GB of scratch. Same bits either way.
 PF_HOT_MIN, PF_HOT_SLOTS = 257, 0
 
 
