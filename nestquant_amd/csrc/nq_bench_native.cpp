@@ -117,7 +117,7 @@ int main(int argc, char** argv)
         return 0;
     }
 
-    const int cfg_gu[4] = {1, 4, 12, 0}, cfg_dn[4] = {1, 4, 8, 0};
+    const int cfg_gu[4] = {1, 4, 12, 0}, cfg_dn[4] = {1, 4, 4, 0};
     const int ny_gu = H / 128 / (cfg_gu[0] * cfg_gu[2]), ny_dn = I / 128 / (cfg_dn[0] * cfg_dn[2]);
     uint16_t *x, *rw, *h; int64_t* sel; float *out, *acc_gu, *acc_d, *zd; int32_t *cnt_gu, *cnt_d, *cnt_h;
     HIPCHK(hipMalloc(&x, (size_t)B * H * 2)); fill_half<<<64, 256>>>(x, (size_t)B * H, 0x2A66);   // 0.05

@@ -158,7 +158,7 @@ class MoELayer:
     # k-slice lengths (chunks) per token count 1..8 at the full shape H = 6144, I = 2048, top-8 over 256 experts, measured on
     # an MI355X with the routing of the layer benchmark; the reference keeps such tables for its GPUs
     # (sm120/serve/nq_vllm.py:32-33). Index = tokens of the call; other shapes use default_cfg for every count.
-    TUNED_NST = {(6144, 2048): ([12, 12, 24, 12, 24, 24, 24, 24, 24], [4, 4, 16, 16, 16, 16, 16, 16, 16])}
+    TUNED_NST = {(6144, 2048): ([12, 12, 24, 24, 24, 24, 24, 24, 24], [4, 4, 4, 4, 4, 4, 4, 4, 4])}
 
     def cfg_for(s, T):
         """(cfg_gu, cfg_dn) for a decode call of T tokens: the layer's defaults, with the tuned k-slice length for T where this
