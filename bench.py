@@ -675,31 +675,27 @@ def main():
     dt = time.perf_counter() - t0
     nbytes = sum(code_bytes(ex, levels, routes[i % R][2]) for i in range(K))
     gbs = nbytes / dt / 1e9
-    # spread of the same measurement, after the reference's method (median and minimum over blocks of replays, each between two
-    # events, sm120/timing.py:2-29): 12 blocks of one 64-step graph
-    blocks = []
-    with torch.cuda.stream(s):
-        for _ in range(12):
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record(s); g_full.replay(); e1.record(s)
-            blocks.append((e0, e1))
-    torch.cuda.synchronize()
-    blocks = sorted(e0.elapsed_time(e1) * 1e3 / R for e0, e1 in blocks)
-    # the layer call alone, as the reference quotes its per-layer figures (mailbox kernel listed separately,
-    # threads/13-moe-layer-kernel/INTEGRATION.md:241): the same 64 steps without the mailbox launch
+    # spread of the same measurement with the reference's method (sm120/timing.py:2-29): the graphs under comparison are replayed
+    # in a seeded shuffled order per block, each one twice back to back with the second replay between two events; median and
+    # minimum over the blocks. The two graphs: the 64 steps with the mailbox in the call, and the layer call alone, as the
+    # reference quotes its per-layer figures (mailbox listed separately, threads/13-moe-layer-kernel/INTEGRATION.md:241)
+    import random
     g_call = torch.cuda.CUDAGraph()
     with torch.cuda.graph(g_call, stream=s):
         for i in range(R):
             L(xs[i], routes[i][0], routes[i][1], out=outs[i])
-    call_blocks = []
+    graphs, rows = {"step": g_full, "call": g_call}, {"step": [], "call": []}
     with torch.cuda.stream(s):
         g_call.replay()
-        for _ in range(12):
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record(s); g_call.replay(); e1.record(s)
-            call_blocks.append((e0, e1))
-    torch.cuda.synchronize()
-    call_blocks = sorted(e0.elapsed_time(e1) * 1e3 / R for e0, e1 in call_blocks)
+        for seed in range(24):
+            order = list(graphs)
+            random.Random(seed).shuffle(order)
+            for name in order:
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                graphs[name].replay(); e0.record(s); graphs[name].replay(); e1.record(s)
+                e1.synchronize()
+                rows[name].append(e0.elapsed_time(e1) * 1e3 / R)
+    blocks, call_blocks = sorted(rows["step"]), sorted(rows["call"])
 
     # dominant kernel alone: gate|up decode-GEMV (which = 1: the launch with its SwiGLU finisher); one graph of R launches, replayed
     # between two events recorded on the launch stream (eager launches from Python would measure the host, not the kernel). Every
