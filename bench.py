@@ -718,26 +718,37 @@ def main():
     with torch.cuda.graph(gk, stream=s):
         for i in range(R):
             gu_only(i, 5)
+    # the same launch as it runs inside a layer call (which = 1 | 4 | 8: the SwiGLU is left to the down launch's staging)
+    gk_in = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(gk_in, stream=s):
+        for i in range(R):
+            gu_only(i, 13)
     L.route, L.xrot = ws_main
     nrep = max(1, (K + R - 1) // R)
-    with torch.cuda.stream(s):
-        gk.replay()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record(s)
-        for _ in range(nrep):
-            gk.replay()
-        e1.record(s)
-    torch.cuda.synchronize()
-    kdt = e0.elapsed_time(e1) / 1e3 / (nrep * R)
+
+    def timed_graph(gr):
+        with torch.cuda.stream(s):
+            gr.replay()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(s)
+            for _ in range(nrep):
+                gr.replay()
+            e1.record(s)
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / 1e3 / (nrep * R)
+    kdt, kdt_in = timed_graph(gk), timed_graph(gk_in)
     kbytes = sum(code_bytes(ex, levels, routes[i][2], "gu") for i in range(R)) / R
     achieved = kbytes / kdt / 1e9
     roofline = dict(bound="hbm", kernel="nq_gemv_k<0, false> (gate|up decode+GEMV)", achieved=round(achieved, 1), peak=HBM_PEAK_GBS, unit="GB/s",
                     frac=round(achieved / HBM_PEAK_GBS, 4), traffic=int(kbytes * TRAFFIC_RATIO), us_per_launch=round(kdt * 1e6, 2),
-                    algorithmic_bytes_per_launch=int(kbytes),
+                    algorithmic_bytes_per_launch=int(kbytes), us_per_launch_inside_layer_call=round(kdt_in * 1e6, 2),
+                    frac_inside_layer_call=round(kbytes / kdt_in / 1e9 / HBM_PEAK_GBS, 4),
                     traffic_source=f"algorithmic bytes x {TRAFFIC_RATIO}: rocprofv3 FETCH_SIZE + WRITE_SIZE of this kernel, scaled by a 256 MiB copy "
                                    "(profiles/decode_gemv_hbm_traffic_pmc.txt), not a counter read in this run",
                     timed="the gate|up projection launch alone (which = 1 | 4: with its SwiGLU finisher, routing and rotated activations "
-                          "prepared beforehand), 64 routings in one graph, HIP events on the launch stream")
+                          "prepared beforehand), 64 routings in one graph, HIP events on the launch stream; "
+                          "us_per_launch_inside_layer_call is the same launch as the timed layer steps run it (which = 1 | 4 | 8: the "
+                          "SwiGLU is formed by the down launch), the variant a kernel trace of this command mostly shows")
     cpu = None
     if not a.no_cpu:
         cpu, y0, yt0 = cpu_baseline(ex, levels, routes, xs)

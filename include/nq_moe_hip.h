@@ -62,7 +62,9 @@ int nq_pf_decode(const int64_t* table, const int32_t* experts, int G, void* Wgu_
  * reference's workspace contract, sm120/nqmoe.cu:855-857). Picks with rw == 0, level <= 0 or an expert id outside
  * [0, E) contribute nothing. which: bit 0 = gate|up launch, bit 1 = down launch; bit 2 = skip the call's first launch (routing
  * and rotation of the activations) because route_ws and xrot still hold what an earlier call with the same x, sel, rw and table
- * rows left there (what a benchmark of one projection launch alone uses). hits: optional int32[E] pick counters
+ * rows left there (what a benchmark of one projection launch alone uses); bit 3 = the two launches come as two calls but with the
+ * arithmetic of one: the gate|up call (which = 1 | 8) leaves h to the down call (which = 2 | 4 | 8), which forms it from the gate|up
+ * partial sums exactly as a which = 3 call does (same bits). hits: optional int32[E] pick counters
  * (device or host-mapped memory), incremented once per pick with rw != 0 (reference :784-787). */
 /* Element types of the caller's tensors. The casts the reference's caller launches around the call (x.half(), ids.long(),
  * w.half(), out.to(x.dtype): sm120/serve/nq_vllm.py:522,560,573; fusing them is the open item of

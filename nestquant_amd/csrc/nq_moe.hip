@@ -663,6 +663,7 @@ int launch_moe(const MoeArgs& a, const int* cfg_gu, const int* cfg_dn, int which
 {
     const int S = a.B * a.topk;
     const bool reuse = (which & 4) != 0;                          // the routing launch of an earlier call left route_ws / xrot as this call needs them
+    const bool defer = (which & 8) != 0;                          // two-call form of the one-call arithmetic: h is formed by the down launch
     which &= 3;
     if (!reuse)
     {
@@ -682,7 +683,7 @@ int launch_moe(const MoeArgs& a, const int* cfg_gu, const int* cfg_dn, int which
         const int shm = std::max(a.B * (NC * 256 + 16) + 256, SB * 512);
         const bool any = a.common_rows != 1;
         MoeArgs b = a;
-        b.fuse = which == 3;                                      // both launches belong to this call
+        b.fuse = which == 3 || defer;                             // both launches belong to this call (or the caller says the other one follows)
         b.ny_gu = (a.H / 128) / (cfg_gu[0] * cfg_gu[2]);
         b.mb_apply = mb_todo; mb_todo = false;                    // the call's first projection launch carries the mailbox block
         auto kern = mode == 0 ? (any ? nq_gemv_k<0, true> : nq_gemv_k<0, false>) : (any ? nq_gemv_k<1, true> : nq_gemv_k<1, false>);

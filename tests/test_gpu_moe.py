@@ -490,5 +490,10 @@ def test_finisher_in_the_down_launch_gives_the_same_bits(golden_dir):
         y3 = L(xb, sb, wb).clone()
         L(xb, sb, wb, which=1)
         y12 = L(xb, sb, wb, which=2).clone()
+        # two calls with the arithmetic of one (which bit 3): the gate|up call leaves h to the down call, which reuses the routing
+        L.h.fill_(float("nan"))
+        L(xb, sb, wb, which=1 | 8)
+        y18 = L(xb, sb, wb, which=2 | 4 | 8).clone()
         torch.cuda.synchronize()
-        assert torch.isfinite(y3).all() and y3.abs().max() > 0 and torch.equal(y3, y12), B
+        assert torch.isfinite(y3).all() and y3.abs().max() > 0 and torch.equal(y3, y12) and torch.equal(y3, y18), B
+        assert not L.cnt_gu.any() and not L.cnt_d.any() and not L.cnt_h.any()
