@@ -158,20 +158,20 @@ def all_MbN():
 
 def _block_words(nb, gen, mbn, dev):
     """'rand': realistic delta = N / Mb ~ 0.1-0.8 plus 5% random extremes; ('exh', offset): cycle through all_MbN()"""
-    if mbn == "rand":
-        kw = dict(generator=gen, device=dev)
-        Mb = torch.randint(120, 256, (nb,), **kw)
-        Nn = (torch.rand(nb, **kw) * 0.8 * Mb).round().long()
-        ext = torch.rand(nb, **kw) < 0.05
-        Mb2 = torch.randint(1, 256, (nb,), **kw)
-        N2 = (torch.rand(nb, **kw) * (torch.clamp(257 - Mb2, max=255) + 1)).floor().long()
-        Mb = torch.where(ext, Mb2, Mb)
-        Nn = torch.minimum(torch.where(ext, N2, Nn), 257 - Mb)
-    else:
-        L = all_MbN().to(dev)
-        idx = (torch.arange(nb, device=dev) + mbn[1]) % len(L)
-        Mb, Nn = L[idx, 0], L[idx, 1]
-    return Mb, Nn
+    if mbn != "rand":
+        table = all_MbN().to(dev)
+        pick = table[(torch.arange(nb, device=dev) + mbn[1]) % len(table)]
+        return pick[:, 0], pick[:, 1]
+    # five draws in the reference's order (sm120/moe.py:93-97), so that the same seed gives the same block words
+    uniform = lambda: torch.rand(nb, generator=gen, device=dev)
+    integer = lambda lo: torch.randint(lo, 256, (nb,), generator=gen, device=dev)
+    m_usual = integer(120)
+    n_usual = (uniform() * 0.8 * m_usual).round().long()
+    extreme = uniform() < 0.05
+    m_any = integer(1)
+    n_any = (uniform() * (torch.clamp(257 - m_any, max=255) + 1)).floor().long()
+    Mb = torch.where(extreme, m_any, m_usual)
+    return Mb, torch.minimum(torch.where(extreme, n_any, n_usual), 257 - Mb)
 
 
 class Proj:
@@ -193,32 +193,32 @@ class Proj:
         R = C if nm is None else nm                      # residual records and block words exist for R chunks per strip
         nr, nb = S * C * 32, S * R
         bits = rbits(rk); nw = (bits + 31) // 32
-        if bk == 0:
+        def record_words(nrec, nbits):
+            """random records of nbits bits as 32-bit words in int64 [nrec, ceil(nbits / 32)], the unused top bits cleared"""
+            words = torch.randint(0, 2**32, (nrec, (nbits + 31) // 32), generator=gen, dtype=torch.int64, device=dev)
+            if nbits % 32:
+                words[:, -1] &= (1 << (nbits % 32)) - 1
+            return words
+        block = lambda Mb, N: (Mb | (N << 8)).to(torch.int32)
+        s.bw = None
+        if bk:                                          # record words of the base code, stored in the sub-array layout
+            s.bw = record_words(nr, rbits(bk))
+            s.base = pack_words(s.bw, rbits(bk))
+        else:
             s.base = torch.randint(-2**31, 2**31 - 1, (nr * 4,), generator=gen, dtype=torch.int32, device=dev)
-            s.bw = None
-        else:                                           # record words of the base code, stored in the sub-array layout
-            bb = rbits(bk)
-            s.bw = torch.randint(0, 2**32, (nr, (bb + 31) // 32), generator=gen, dtype=torch.int64, device=dev)
-            if bb % 32:
-                s.bw[:, -1] &= (1 << (bb % 32)) - 1
-            s.base = pack_words(s.bw, bb)
-        w = torch.randint(0, 2**32, (nb * 32, nw), generator=gen, dtype=torch.int64, device=dev)
-        if bits % 32:
-            w[:, -1] &= (1 << (bits % 32)) - 1
-        s.p4w, s.p4 = w, pack_words(w, bits)
+        s.p4w = record_words(nb * 32, bits)
+        s.p4 = pack_words(s.p4w, bits)
         s.Mb, s.Nn = _block_words(nb, gen, mbn, dev)
-        s.d4 = (s.Mb | (s.Nn << 8)).to(torch.int32)
+        s.d4 = block(s.Mb, s.Nn)
         s.var = torch.randint(0, 256, (S * C,), generator=gen, dtype=torch.int64, device=dev).to(torch.uint8) if var else None
         s.flags, s.fl = (None, None) if nm is None else make_flags(S, C, nm, gen)
         s.p3 = s.d3 = s.p4n = s.d4n = s.p3w = s.p4nw = None
         if nested:
-            s.p3w = torch.randint(0, 2**32, (nr, 2), generator=gen, dtype=torch.int64, device=dev)
-            s.p4nw = torch.randint(0, 2**32, (nr, 2), generator=gen, dtype=torch.int64, device=dev)
+            s.p3w, s.p4nw = record_words(nr, 64), record_words(nr, 64)
             s.p3, s.p4n = pack_words(s.p3w, 64), pack_words(s.p4nw, 64)
             s.Mb3, s.N3 = _block_words(S * C, gen, "rand", dev)
             s.Mb4n, s.N4n = _block_words(S * C, gen, "rand", dev)
-            s.d3 = (s.Mb3 | (s.N3 << 8)).to(torch.int32)
-            s.d4n = (s.Mb4n | (s.N4n << 8)).to(torch.int32)
+            s.d3, s.d4n = block(s.Mb3, s.N3), block(s.Mb4n, s.N4n)
 
     _TENSORS = ["base", "bw", "p4", "d4", "flags", "fl", "p4w", "Mb", "Nn", "var", "p3", "d3", "p4n", "d4n", "p3w", "p4nw"]
 
@@ -248,25 +248,22 @@ class Expert:
         mbn_dn = mbn if mbn == "rand" else ("exh", mbn[1] + (2 * I // 16) * (H // 128))
         s.gu = Proj(2 * I, H, gen, nm_gu, rk_gu, mbn, var, bk_gu, nested).to(dev)
         s.dn = Proj(H, I, gen, nm_dn, rk_dn, mbn_dn, var, bk_dn, nested).to(dev)
-        sg = torch.randint(0, 2, (2 * H + 3 * I,), generator=gen, device=gen_dev) * 2 - 1
-        su_u = torch.randint(0, 2, (H,), generator=gen, device=gen_dev) * 2 - 1
-        s.signs = torch.cat([sg, su_u]).half().to(dev)
+        signs = lambda n: torch.randint(0, 2, (n,), generator=gen, device=gen_dev) * 2 - 1
+        s.signs = torch.cat([signs(2 * H + 3 * I), signs(H)]).half().to(dev)     # five vectors in one draw, then su_u
         s.H, s.I, s.nested = H, I, nested
-        s.lr = s.lr4 = None
-        s.rg = s.rd = 0
+        s.lr, s.lr4, s.rg, s.rd = None, None, 0, 0
         if nested:                                       # slot image: [P3 | P4] per projection, contiguous
             s.gu.slot = s.gu.nested_plane(); s.dn.slot = s.dn.nested_plane()
 
     def set_lr(s, Vg, U2g, U2u, U4g, U4u, Vd, U2d, U4d):
         """low-rank plane (fp16; reference sm120/moe.py:184-189): Vg [rg, H], U2g / U2u / U4g / U4u [rg, I], Vd [rd, I],
         U2d / U4d [rd, H] -> the two buffers of table words 14 / 15: lr = Vg | U2g | U2u | Vd | U2d, lr4 = U4g | U4u | U4d"""
-        f = lambda *t: torch.cat([x.reshape(-1) for x in t]).half().contiguous()
-        s.rg, s.rd = Vg.shape[0], Vd.shape[0]
         s.lrT = (Vg, U2g, U2u, U4g, U4u, Vd, U2d, U4d)
-        if s.rg + s.rd == 0:
-            s.lr = s.lr4 = None
-            return s
-        s.lr = f(Vg, U2g, U2u, Vd, U2d).to(s.signs.device); s.lr4 = f(U4g, U4u, U4d).to(s.signs.device)
+        s.rg, s.rd = Vg.shape[0], Vd.shape[0]
+        s.lr = s.lr4 = None
+        if s.rg or s.rd:
+            flat = lambda parts: torch.cat([t.reshape(-1) for t in parts]).half().contiguous().to(s.signs.device)
+            s.lr, s.lr4 = flat((Vg, U2g, U2u, Vd, U2d)), flat((U4g, U4u, U4d))
         return s
 
     def compact(s):

@@ -118,7 +118,7 @@ def test_prefill_soak(seed):
 
 
 def test_config3_full_table_one_to_four_tokens():
-    """BASELINE config 3 as the benchmark builds it: 256 experts at the full shape (26 at level 4, 51 at level 3 or 4 by seed, 179
+    """The full decode layer as the benchmark builds it: 256 experts at the full shape (26 at level 4, 51 at level 3 or 4 by seed, 179
     at level 2), seeded softmax top-8 routing, 1-4 tokens, against the oracle's layer math in float64 over the HIP-decoded dense
     weights of the routed experts (the decoder is proved bit-exact in test_gpu_dequant): 5e-5, and 1e-3 against the fp32 pipeline
     without activation rounding."""
