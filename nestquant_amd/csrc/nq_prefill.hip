@@ -604,8 +604,6 @@ __device__ __forceinline__ void pf_chunks(const Planes& P, const LaneCtx& L, int
     uint32_t boff[4];                                            // B-operand read offsets of this lane for mm = 0..3
 #pragma unroll
     for (int mm = 0; mm < 4; ++mm) boff[mm] = (uint32_t)(n * PF_ROW + (((4 * mm + t4) ^ n) << 4));
-    typedef const __attribute__((address_space(1))) void* gvp;
-    typedef __attribute__((address_space(3))) void* lvp;
     for (int c = 0; c < C; ++c)
     {
         // ---- decode this wave's unit pair of chunk c into A operands; prefetch chunk c + 1; request the tile's tokens for chunk c
