@@ -278,8 +278,11 @@ __global__ void __launch_bounds__(256) nq_prep_k(MoeArgs a)
     const int lane = threadIdx.x & 63;
     if (threadIdx.x < 64) route(a, a.route, lane, blockIdx.x == 0, &Q);
     __syncthreads();
-    const int C = a.H / 128, ntask = Q.nq * 2 * C;
-    for (int t = blockIdx.x * 4 + (threadIdx.x >> 6); t < ntask; t += gridDim.x * 4)
+    // workgroup 0 has the result to write (it ends ~1 us after the others' routing): with more than one workgroup in the grid the
+    // rotation tasks go to the others, so that it is not also the last to finish
+    const int C = a.H / 128, ntask = Q.nq * 2 * C, nrot = gridDim.x > 1 ? gridDim.x - 1 : 1, rot = gridDim.x > 1 ? (int)blockIdx.x - 1 : 0;
+    if (rot < 0) return;
+    for (int t = rot * 4 + (threadIdx.x >> 6); t < ntask; t += nrot * 4)
     {
         const int q = t / (2 * C), r = t - q * 2 * C, up = r / C, c = r - up * C, kk = c * 128 + 2 * lane;
         const _Float16* su = Q.signs[q] + (up ? 2 * a.H + 3 * a.I : 0);
@@ -668,7 +671,7 @@ int launch_moe(const MoeArgs& a, const int* cfg_gu, const int* cfg_dn, int which
     if (!reuse)
     {
         const int ntask = S * 2 * (a.H / 128);                   // upper bound: every pick active
-        nq_prep_k<<<std::min((ntask + 3) / 4, 1024), 256, 0, st>>>(a);
+        nq_prep_k<<<std::min((ntask + 3) / 4, 1023) + 1, 256, 0, st>>>(a);       // one workgroup per four rotation tasks, plus the writer
         NQ_LAUNCH_CHECK("moe_forward (routing)");
     }
     if (a.mb_table && which == 0) return launch_mailbox(a.mb_table, a.mb_stage, a.mb_seq, a.mb_applied, a.mb_applied_host, a.E, st);
