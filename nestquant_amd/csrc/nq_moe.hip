@@ -198,6 +198,7 @@ __device__ __forceinline__ void route(const MoeArgs& a, RouteWs* W, int lane, bo
     const int tok = lane / a.topk, sh = tok * a.topk;
     const unsigned long long mytok = sh < 64 ? (a.topk >= 64 ? ~0ull : ((1ull << a.topk) - 1ull)) << sh : 0ull;
     int r = 0, cum = 0;
+    int my_run = -1, my_pos = 0, my_ntok = 0, my_q0 = 0;         // the run this lane's pick went into, its place there; for the first lane of a run: its size
     for (int pass = 0; pass < 2; ++pass)
     {
         unsigned long long rem = pass == 0 ? heavy : okm & ~heavy;
@@ -209,35 +210,36 @@ __device__ __forceinline__ void route(const MoeArgs& a, RouteWs* W, int lane, bo
             const unsigned long long m = __ballot(((same >> lane) & 1ull) && (same & mytok & below) == 0ull);   // first pick per token
             if ((m >> lane) & 1ull)
             {
-                const int pos = __popcll(m & below);
-                Q->tok[cum + pos] = (unsigned char)tok; Q->signs[cum + pos] = (const _Float16*)f[9];
-            }
-            if (writer && ((m >> lane) & 1ull))
-            {
-                const int pos = __popcll(m & below);
-                W->run[0][r].slot[pos] = (unsigned char)lane; W->run[1][r].slot[pos] = (unsigned char)lane;
-                if (pos == 0)
-                {
-#pragma unroll
-                    for (int mode = 0; mode < 2; ++mode)
-                    {
-                        RunHdr& R = W->run[mode][r];
-                        const int o = mode == 0 ? 1 : 5;
-                        R.P.base = (gp_u4)f[o]; R.P.res = (gp_u8)f[o + 1]; R.P.dw = (gp_u32)f[o + 2]; R.P.flags = (gp_u64)f[o + 3];
-                        R.P.var = (gp_u8)f[12 + mode]; R.P.code = (int)f[10 + mode]; R.P.bcode = (int)((f[19] >> (8 * mode)) & 0xFF);
-                        R.signs = (const _Float16*)f[9];
-                        R.level = level;
-                        R.had = f[18] == 512 ? 512 : 128;
-                        R.lr = (const _Float16*)f[14]; R.lr4 = (const _Float16*)f[15]; R.rg = (int)f[16]; R.rd = (int)f[17];
-                        R.ntok = __popcll(m); R.q0 = cum;
-                    }
-                }
+                my_run = r; my_pos = __popcll(m & below); my_ntok = __popcll(m); my_q0 = cum;
+                Q->tok[cum + my_pos] = (unsigned char)tok; Q->signs[cum + my_pos] = (const _Float16*)f[9];
             }
             rem &= ~m; ++r; cum += __popcll(m);
         }
     }
     if (lane == 0) Q->nq = cum;
     if (!writer) return;
+    // the headers, after the numbering: every lane holds its own pick's row, so the first lanes of all runs write their runs'
+    // headers side by side (inside the loop above the same stores would be issued once per run, one lane at a time)
+    if (my_run >= 0)
+    {
+        W->run[0][my_run].slot[my_pos] = (unsigned char)lane; W->run[1][my_run].slot[my_pos] = (unsigned char)lane;
+        if (my_pos == 0)
+        {
+#pragma unroll
+            for (int mode = 0; mode < 2; ++mode)
+            {
+                RunHdr& R = W->run[mode][my_run];
+                const int o = mode == 0 ? 1 : 5;
+                R.P.base = (gp_u4)f[o]; R.P.res = (gp_u8)f[o + 1]; R.P.dw = (gp_u32)f[o + 2]; R.P.flags = (gp_u64)f[o + 3];
+                R.P.var = (gp_u8)f[12 + mode]; R.P.code = (int)f[10 + mode]; R.P.bcode = (int)((f[19] >> (8 * mode)) & 0xFF);
+                R.signs = (const _Float16*)f[9];
+                R.level = level;
+                R.had = f[18] == 512 ? 512 : 128;
+                R.lr = (const _Float16*)f[14]; R.lr4 = (const _Float16*)f[15]; R.rg = (int)f[16]; R.rd = (int)f[17];
+                R.ntok = my_ntok; R.q0 = my_q0;
+            }
+        }
+    }
     PickInfo& K = W->picks;
     K.w[lane] = ok ? rw_at(a, lane) : 0.f; K.signs[lane] = (const _Float16*)f[9];
     K.lr[lane] = (const _Float16*)f[14]; K.lr4[lane] = (const _Float16*)f[15];
