@@ -1,4 +1,5 @@
-"""Minimal level-2 encoder: dense weight [N, K] -> 2-bit trellis base plane + fp16 sign/scale vectors.
+"""Minimal encoder: dense weight [N, K] -> 2-bit trellis base plane + fp16 sign/scale vectors (encode_level2), and on top
+of it the refinement planes of levels 3 and 4 fitted to the base plane's residual (encode_nested).
 
 It exists to produce honest planes for the CPU-plumbing configuration (one 512 x 256 weight, encode -> decode -> GEMV);
 it is not the reference's production encoder. What it restates, in plain torch that runs on CPU or GPU:
@@ -9,14 +10,22 @@ it is not the reference's production encoder. What it restates, in plain torch t
     threads/05-exl3-harness/harness.py:297-364: pass 1 rolled by half a ring finds the state entering step 0, pass 2 is
     constrained to start from and end in it), Viterbi step i <-> ring position p = (-i) mod 256
     (threads/12-reference-encoder/nq_encode.py:54-58);
-  * the LSB-first packing of ring states into lane records (threads/12-reference-encoder/nq_decode.py:101-109).
+  * the LSB-first packing of ring states into lane records (threads/12-reference-encoder/nq_decode.py:101-109);
+  * the greedy refinement stage with identity Hessian (threads/12-reference-encoder/nq_encode.py:286-316 without the LDLQ
+    feedback terms; threads/03-nested-trellis-code/exp3.py:20-26,55-60): the residual of the frozen base plane, divided by
+    its rms per unit and by the input scale the reference found best on Gaussian data (1.1 at one bit per weight, 1.0 at
+    two), goes through the same Viterbi with K = 1 or 2 bits per step; the least-squares step size delta = N / Mb is then
+    searched over the reference's twelve block-word candidates (nq_encode.py:186-198, nq_decode.py:158-163) with the
+    integer fold itself (sm120/ref15_spec.py:79-90) as the cost, so the chosen word is the best of them for the values
+    the decoder really produces.
 The reference's encoder depends on exllamav3 1.5.1, which is not available here, so bit parity with it is not claimed;
 the tests pin this encoder by brute force on a small trellis, by decode(encode) self-consistency and by the Gaussian
-distortion the reference reports for this code (MSE 0.068 at 2 bits, threads/03-nested-trellis-code/REPORT.md:21).
+distortion the reference reports for this code (MSE 0.068 at 2 bits, threads/03-nested-trellis-code/REPORT.md:21; base +
+one-bit refinement 0.018747, base + two-bit refinement 0.004729, threads/03-nested-trellis-code/exp3_mul1L.log:3-4).
 """
 import torch
 
-from .format import Proj, proj_sizes
+from .format import Proj, pack_words, proj_sizes
 
 HC = 0x83DCD12D
 
@@ -101,6 +110,47 @@ def blocked_had(X, dim):
     return Y.movedim(-1, dim)
 
 
+def to_rings(M):
+    """[N, K] -> [units * 8, 256] in ring position order (unit = strip * C + chunk)"""
+    N, K = M.shape
+    S, C = N // 16, K // 128
+    units = M.reshape(S, 16, C, 128).permute(0, 2, 3, 1).reshape(S * C, 2048)        # [unit, column * 16 + row]
+    return units[:, ring_index(M.device).reshape(-1)].reshape(S * C * 8, 256)
+
+
+def from_rings(R, N, K):
+    """inverse of to_rings"""
+    S, C = N // 16, K // 128
+    U = torch.empty(S * C, 2048, dtype=R.dtype, device=R.device)
+    U[:, ring_index(R.device).reshape(-1)] = R.reshape(S * C, 2048)
+    return U.reshape(S, C, 128, 16).permute(0, 3, 1, 2).reshape(N, K)
+
+
+def viterbi_rings(rings, K=2, chunk=64):
+    """rings [T, 256] in ring position order -> states int64 [T, 256] in the same order.
+    Viterbi step i <-> position p = (-i) mod 256, a permutation that is its own inverse."""
+    dev = rings.device
+    ip = (-torch.arange(256, device=dev)) % 256
+    lut = codebook(dev)
+    st = torch.empty(rings.shape, dtype=torch.int64, device=dev)
+    for a in range(0, rings.shape[0], chunk):
+        st[a:a + chunk] = viterbi_ring(rings[a:a + chunk][:, ip].contiguous(), lut, K)[:, ip]
+    return st
+
+
+def lane_records(st, K):
+    """ring states [T, 256] (position order) of a K-bits-per-step stream -> record words int64 [T * 4, 2 K] (uint32 values).
+    Stream bit K p + b = bit b of state(p): the low K bits of each state are the new bits of its step; lane t4 of a ring
+    holds the stream's bits [64 K t4, 64 K (t4 + 1)), so records come out in (unit, ring, lane) order."""
+    dev = st.device
+    bits = torch.stack([(st >> b) & 1 for b in range(K)], -1).reshape(-1, 256 * K)
+    sym = (bits.reshape(-1, 256, K) << torch.arange(K, device=dev)).sum(-1)
+    n = 16 // K
+    idx = (torch.arange(256, device=dev)[:, None] + torch.arange(n, device=dev)[None]) % 256
+    assert torch.equal((sym[:, idx] << (K * torch.arange(n, device=dev))).sum(-1), st), "ring states are not tail-biting"
+    return (bits.reshape(-1, 8 * K, 32) << torch.arange(32, device=dev)).sum(-1).reshape(-1, 2 * K)
+
+
 def encode_level2(W, seed=0, chunk=64):
     """W [N, K] float (N % 16 == 0, K % 128 == 0; N % 128 == 0 for the output rotation) ->
     dict(base int32 [nrec*4], su fp16 [K], sv fp16 [N], states int64 [units, 8, 256] (ring position order), Q fp32 [N, K])
@@ -119,38 +169,140 @@ def encode_level2(W, seed=0, chunk=64):
     # the decoder applies the fp16-rounded scales, so the target is built from them
     Wn = Wd / su.double()[None, :] / sv.double()[:, None]
     target = blocked_had(blocked_had(Wn, 1), 0).float()          # B_N Wn B_K
-    S, C = N // 16, K // 128
-    RI = ring_index(dev)
-    units = target.reshape(S, 16, C, 128).permute(0, 2, 3, 1).reshape(S * C, 2048)   # [unit, column * 16 + row]
-    rings = units[:, RI.reshape(-1)].reshape(S * C * 8, 256)     # ring position order
-    ip = (-torch.arange(256, device=dev)) % 256                  # Viterbi step i <-> position p = (-i) mod 256
-    lut = codebook(dev)
-    st = torch.empty(rings.shape, dtype=torch.int64, device=dev)
-    for a in range(0, rings.shape[0], chunk):
-        sv_i = viterbi_ring(rings[a:a + chunk][:, ip].contiguous(), lut)
-        st[a:a + chunk] = sv_i[:, ip]                            # back to position order (ip is its own inverse)
-    # stream bit 2p + b = bit b of state(p): the low 2 bits of each state are the 2 new bits of its step
-    bits = torch.stack([st & 1, (st >> 1) & 1], -1).reshape(-1, 512)
-    chk = (bits.reshape(-1, 256, 2) * torch.tensor([1, 2], device=dev)).sum(-1)
-    idx = (torch.arange(256, device=dev)[:, None] + torch.arange(8, device=dev)[None]) % 256
-    assert torch.equal((chk[:, idx] << (2 * torch.arange(8, device=dev))).sum(-1), st), "ring states are not tail-biting"
-    words = (bits.reshape(-1, 16, 32) << torch.arange(32, device=dev)).sum(-1)       # [rings, 16 words]; lane t4 = words 4 t4..
-    base = words.reshape(S * C, 8, 4, 4).reshape(-1)                                  # record = (unit, lane 4 g + t4): 4 words
+    st = viterbi_rings(to_rings(target), 2, chunk)
+    base = lane_records(st, 2).reshape(-1)                       # record = (unit, lane 4 g + t4): 4 words
     base = torch.where(base >= 2**31, base - 2**32, base).to(torch.int32)
-    Qr = lut[st]                                                 # decoded values, ring position order
-    Qu = torch.empty(S * C, 2048, device=dev)
-    Qu[:, RI.reshape(-1)] = Qr.reshape(S * C, 2048)
-    Q = Qu.reshape(S, C, 128, 16).permute(0, 3, 1, 2).reshape(N, K)
-    return dict(base=base, su=su, sv=sv, states=st.reshape(S * C, 8, 256), Q=Q, target=target)
+    Q = from_rings(codebook(dev)[st], N, K)                      # decoded values
+    return dict(base=base, su=su, sv=sv, states=st.reshape(-1, 8, 256), Q=Q, target=target)
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# refinement planes (levels 3 and 4)
+A_ = float(torch.tensor([0x1EEE], dtype=torch.int16).view(torch.float16))
+K0 = 1024.0 * A_ + float(torch.tensor([0xC931 - 65536], dtype=torch.int16).view(torch.float16))
+RES_SCALE = {1: 1.1, 2: 1.0}     # best input scale of the refinement stage on Gaussian data (reference exp3_mul1L.log:3-4)
+
+
+def hash_sum(st):
+    """byte sum S of state * HC mod 2^32 (reference sm120/ref15_spec.py:64-70)"""
+    x = (st * HC) & 0xFFFFFFFF
+    return (x & 255) + ((x >> 8) & 255) + ((x >> 16) & 255) + (x >> 24)
+
+
+def round_f16(v):
+    """float64 -> fp16 with one rounding. Going through fp32 rounds twice; rounding to odd at 24 bits first (truncate, then
+    set the last bit if anything was cut off) makes the second rounding see on which side of a tie the value lies."""
+    f = v.float()
+    cut = f.double() != v
+    bits = f.view(torch.int32) - (f.double().abs() > v.abs()).to(torch.int32)      # one step towards zero where fp32 rounded away
+    return (bits | cut.to(torch.int32)).view(torch.float32).half()
+
+
+_FOLD = None
+
+
+def fold_table():
+    """fp16 constants (A', C) of the integer fold for every block word, as fp32 [256, 258, 2] indexed by (Mb, N): fp32
+    operations in the spec's order, none contracted (reference sm120/ref15_spec.py:79-86). Built once on the CPU, whose
+    fp32 division and products are correctly rounded."""
+    global _FOLD
+    if _FOLD is None:
+        Mb = torch.arange(256, dtype=torch.float32).clamp_min(1)[:, None]
+        N = torch.arange(258, dtype=torch.float32)[None, :]
+        rcp = torch.ones(1) / Mb
+        Ah = (torch.tensor(1.732421875) * rcp).half()
+        t = (N * rcp) * torch.tensor(K0, dtype=torch.float32)
+        t = t + torch.tensor(K0, dtype=torch.float32)
+        Ch = (t - torch.tensor(1024.0) * Ah.float()).half()
+        _FOLD = torch.stack([Ah.float().expand(256, 258), Ch.float()], -1).contiguous()
+    return _FOLD
+
+
+def fold_value(Sb, Sr, Mb, N):
+    """levels 3 / 4: F = (Mb Sb + N Sr + 128) >> 8, value = fp16(A' (1024 + F) + C) with one rounding
+    (reference sm120/ref15_spec.py:87-90, sm120/moe.py:128-134). Sb, Sr int64 [U, ...]; Mb, N int64 [U]. -> fp16"""
+    shape = (-1,) + (1,) * (Sb.dim() - 1)
+    Mb_, N_ = Mb.view(shape), N.view(shape)
+    c = fold_table().to(Sb.device)[Mb, N].double()
+    F = (Mb_ * Sb + N_ * Sr + 128) >> 8
+    return round_f16(c[:, 0].view(shape) * (1024 + F).double() + c[:, 1].view(shape))
+
+
+def block_word_candidates(delta):
+    """[U] step sizes -> (Mb, N) int64 [U, 12]: the largest-Mb rational N / Mb nearest to delta with Mb + N <= 257,
+    Mb <= 255, and its neighbours Mb - 0..3, N - 1..N + 1; a candidate outside the valid range is replaced by the first
+    (reference nq_decode.py:158-163, nq_encode.py:186-198)."""
+    d = delta.double().clamp_min(0)
+    Mb0 = torch.floor(257 / (1 + d)).clamp(1, 255).long()
+    N0 = torch.minimum(torch.round(d * Mb0).long(), 257 - Mb0)
+    Ms, Ns = [], []
+    for dm in range(4):
+        Mb = (Mb0 - dm).clamp(1, 255)
+        Nr = torch.round(d * Mb).long()
+        for dn in (-1, 0, 1):
+            Ms.append(Mb); Ns.append(Nr + dn)
+    Mb, N = torch.stack(Ms, 1), torch.stack(Ns, 1)
+    ok = (N >= 0) & (N <= 255) & (Mb + N <= 257)
+    return torch.where(ok, Mb, Mb0[:, None]), torch.where(ok, N, N0[:, None].clamp_max(255))
+
+
+def encode_residual(target, st_base, K, chunk=64, scale=None):
+    """One refinement stage on the frozen base plane. target fp32 [U, 8, 256] and st_base int64 [U, 8, 256] in ring position
+    order, K = 1 or 2 bits per weight -> dict(states [U, 8, 256], Mb [U], N [U], Q fp32 [U, 8, 256], delta [U])."""
+    U = target.shape[0]
+    dev = target.device
+    lut = codebook(dev)
+    Sb = hash_sum(st_base)
+    r = target.double() - lut[st_base].double()
+    rms = r.square().mean((1, 2)).sqrt().clamp_min(1e-12)
+    s0 = rms / (RES_SCALE[K] if scale is None else scale)
+    st = viterbi_rings((r / s0[:, None, None]).float().reshape(U * 8, 256), K, chunk).reshape(U, 8, 256)
+    Sr = hash_sum(st)
+    a = A_ * Sr.double() + K0                                    # unrounded value of the refinement code
+    delta = ((a * r).sum((1, 2)) / a.square().sum((1, 2)).clamp_min(1e-30)).clamp_min(0)
+    Mbs, Ns = block_word_candidates(delta)
+    best = None
+    for ci in range(Mbs.shape[1]):
+        q = fold_value(Sb, Sr, Mbs[:, ci], Ns[:, ci]).float()
+        c = (target - q).double().square().sum((1, 2))
+        if best is None:
+            best = dict(c=c, Q=q, Mb=Mbs[:, ci].clone(), N=Ns[:, ci].clone())
+        else:
+            w = c < best["c"]
+            best["c"] = torch.where(w, c, best["c"]); best["Q"][w] = q[w]
+            best["Mb"][w] = Mbs[w, ci]; best["N"][w] = Ns[w, ci]
+    return dict(states=st, Mb=best["Mb"], N=best["N"], Q=best["Q"], delta=delta)
+
+
+def encode_nested(W, seed=0, chunk=64):
+    """encode_level2 plus the two refinement planes, each fitted to the residual of the same frozen base plane:
+    p3 / d3 (one bit per weight, 64-bit records; level 3 = base + P3) and p4 / d4 (two bits per weight, 128-bit records of
+    window code 0; level 4 = base + the wide plane). Adds p3, d3, Q3, p4, d4, Q4 (Q3 / Q4 fp32 [N, K]: the matrices the
+    decoder reproduces bit for bit at levels 3 / 4) to encode_level2's dict."""
+    N, K = W.shape
+    r = encode_level2(W, seed, chunk)
+    tr = to_rings(r["target"]).reshape(-1, 8, 256)
+    i32 = lambda t: torch.where(t >= 2**31, t - 2**32, t).to(torch.int32)
+    for lvl, bits_per_weight in ((3, 1), (4, 2)):
+        e = encode_residual(tr, r["states"], bits_per_weight, chunk)
+        r["p%d" % lvl] = pack_words(lane_records(e["states"].reshape(-1, 256), bits_per_weight), 64 * bits_per_weight)
+        r["d%d" % lvl] = i32(e["Mb"] | (e["N"] << 8))
+        r["Q%d" % lvl] = from_rings(e["Q"].reshape(-1, 256), N, K)
+        r["states%d" % lvl] = e["states"]
+    return r
 
 
 class EncodedProj(Proj):
-    """a Proj (nestquant_amd.format) holding an encoded level-2 base plane; the residual planes are absent"""
+    """a Proj (nestquant_amd.format) holding encoded planes: the level-2 base plane and, when given, the refinement planes
+    p3 / d3 (level 3, the one-bit nested plane) and p4 / d4 (level 4, wide plane of window code 0)"""
 
-    def __init__(s, N, K, base):
+    def __init__(s, N, K, base, p3=None, d3=None, p4=None, d4=None):
         s.z = proj_sizes(N, K)
         s.N, s.K, s.rk, s.bk, s.nested = N, K, 0, 0, False
         s.base = base
-        s.p4 = torch.zeros(1, dtype=torch.int32, device=base.device); s.d4 = torch.zeros(1, dtype=torch.int32, device=base.device)
+        zero = lambda: torch.zeros(1, dtype=torch.int32, device=base.device)
+        s.p4 = zero() if p4 is None else p4
+        s.d4 = zero() if d4 is None else d4
         s.p4w = s.Mb = s.Nn = s.var = s.flags = s.fl = None
-        s.p3 = s.d3 = s.p4n = s.d4n = s.p3w = s.p4nw = None
+        s.p3, s.d3 = p3, d3
+        s.p4n = s.d4n = s.p3w = s.p4nw = None

@@ -35,27 +35,32 @@ def H128(dev="cuda", n=128):
 
 
 def entry(ex, level):
-    """table row int64[TBL_W] of expert `ex` at `level` (0, 2, 3, 4). Level 3 and, for experts built with nested=True,
-    level 4 point at the nested planes (codes 10 / 11); otherwise level 4 points at the wide residual plane p4 (code rk)."""
+    """table row int64[TBL_W] of expert `ex` at `level` (0, 2, 3, 4). Level 3 points at the one-bit plane p3 (code 10); level 4
+    points, for experts built with nested=True, at the record P3 || P4 (code 11), otherwise at the wide residual plane p4
+    (code rk)."""
     e = torch.zeros(TBL_W, dtype=torch.int64)
     e[0] = level
     nested = bool(getattr(ex, "nested", False))
-    if level == 3 and not nested:
-        raise ValueError("level 3 needs an expert with nested planes")
+    l3 = level == 3
+    if l3 and not nested and any(getattr(p, "p3", None) is None for p in (ex.gu, ex.dn)):
+        raise ValueError("level 3 needs an expert with the one-bit planes p3 / d3")
     for off, p in ((1, ex.gu), (5, ex.dn)):
         e[off] = p.base.data_ptr()
         if nested:
             slot = p.slot
             e[off + 1] = slot.data_ptr()
-            e[off + 2] = (p.d3 if level == 3 else p.d4n).data_ptr()
+            e[off + 2] = (p.d3 if l3 else p.d4n).data_ptr()
+        elif l3:
+            e[off + 1] = p.p3.data_ptr()
+            e[off + 2] = p.d3.data_ptr()
         else:
             e[off + 1] = 0 if p.p4 is None else p.p4.data_ptr()      # None: resident-only expert, a record slot supplies them
             e[off + 2] = 0 if p.d4 is None else p.d4.data_ptr()
         if getattr(p, "flags", None) is not None:
             e[off + 3] = p.flags.data_ptr()
     e[9] = ex.signs.data_ptr()
-    if nested:
-        e[10] = e[11] = CODE_L3 if level == 3 else CODE_L4N
+    if nested or l3:
+        e[10] = e[11] = CODE_L3 if l3 else CODE_L4N
     else:
         e[10], e[11] = ex.gu.rk, ex.dn.rk
     for i, p in ((12, ex.gu), (13, ex.dn)):
