@@ -1,5 +1,6 @@
 """Minimal encoder: dense weight [N, K] -> 2-bit trellis base plane + fp16 sign/scale vectors (encode_level2), and on top
-of it the refinement planes of levels 3 and 4 fitted to the base plane's residual (encode_nested).
+of it the refinement planes of levels 3 and 4 fitted to the base plane's residual (encode_nested), optionally with the
+errors of later column chunks fed forward through the block LDL factor of the input Hessian (encode_ldlq).
 
 It exists to produce honest planes for the CPU-plumbing configuration (one 512 x 256 weight, encode -> decode -> GEMV);
 it is not the reference's production encoder. What it restates, in plain torch that runs on CPU or GPU:
@@ -151,10 +152,9 @@ def lane_records(st, K):
     return (bits.reshape(-1, 8 * K, 32) << torch.arange(32, device=dev)).sum(-1).reshape(-1, 2 * K)
 
 
-def encode_level2(W, seed=0, chunk=64):
-    """W [N, K] float (N % 16 == 0, K % 128 == 0; N % 128 == 0 for the output rotation) ->
-    dict(base int32 [nrec*4], su fp16 [K], sv fp16 [N], states int64 [units, 8, 256] (ring position order), Q fp32 [N, K])
-    with  W ~= D(sv) B_N Q B_K D(su)  and Q the matrix the decoder reproduces bit for bit from `base`."""
+def prepare(W, seed=0):
+    """signs, scales and rotations: W [N, K] -> (su fp16 [K], sv fp16 [N], target fp32 [N, K]) with
+    W = D(sv) B_N target B_K D(su) up to the fp16 rounding of the scales, B the 128-blocked orthonormal Hadamard"""
     N, K = W.shape
     assert N % 128 == 0 and K % 128 == 0
     dev = W.device
@@ -168,11 +168,23 @@ def encode_level2(W, seed=0, chunk=64):
     su = (sgn_u * c_in).half(); sv = (sgn_v * r_out).half()
     # the decoder applies the fp16-rounded scales, so the target is built from them
     Wn = Wd / su.double()[None, :] / sv.double()[:, None]
-    target = blocked_had(blocked_had(Wn, 1), 0).float()          # B_N Wn B_K
+    return su, sv, blocked_had(blocked_had(Wn, 1), 0).float()    # B_N Wn B_K
+
+
+def signed32(w):
+    """uint32 values held in int64 -> int32 with the same bits"""
+    return torch.where(w >= 2**31, w - 2**32, w).to(torch.int32)
+
+
+def encode_level2(W, seed=0, chunk=64):
+    """W [N, K] float (N % 16 == 0, K % 128 == 0; N % 128 == 0 for the output rotation) ->
+    dict(base int32 [nrec*4], su fp16 [K], sv fp16 [N], states int64 [units, 8, 256] (ring position order), Q fp32 [N, K])
+    with  W ~= D(sv) B_N Q B_K D(su)  and Q the matrix the decoder reproduces bit for bit from `base`."""
+    N, K = W.shape
+    su, sv, target = prepare(W, seed)
     st = viterbi_rings(to_rings(target), 2, chunk)
-    base = lane_records(st, 2).reshape(-1)                       # record = (unit, lane 4 g + t4): 4 words
-    base = torch.where(base >= 2**31, base - 2**32, base).to(torch.int32)
-    Q = from_rings(codebook(dev)[st], N, K)                      # decoded values
+    base = signed32(lane_records(st, 2).reshape(-1))             # record = (unit, lane 4 g + t4): 4 words
+    Q = from_rings(codebook(W.device)[st], N, K)                 # decoded values
     return dict(base=base, su=su, sv=sv, states=st.reshape(-1, 8, 256), Q=Q, target=target)
 
 
@@ -246,12 +258,14 @@ def block_word_candidates(delta):
     return torch.where(ok, Mb, Mb0[:, None]), torch.where(ok, N, N0[:, None].clamp_max(255))
 
 
-def encode_residual(target, st_base, K, chunk=64, scale=None):
+def encode_residual(target, st_base, K, chunk=64, scale=None, cost=None):
     """One refinement stage on the frozen base plane. target fp32 [U, 8, 256] and st_base int64 [U, 8, 256] in ring position
-    order, K = 1 or 2 bits per weight -> dict(states [U, 8, 256], Mb [U], N [U], Q fp32 [U, 8, 256], delta [U])."""
+    order, K = 1 or 2 bits per weight -> dict(states [U, 8, 256], Mb [U], N [U], Q fp32 [U, 8, 256], delta [U]).
+    cost: error fp64 [U, 8, 256] -> [U], what the block-word search minimises (default: the squared error)."""
     U = target.shape[0]
     dev = target.device
     lut = codebook(dev)
+    cost = cost or (lambda E: E.square().sum((1, 2)))
     Sb = hash_sum(st_base)
     r = target.double() - lut[st_base].double()
     rms = r.square().mean((1, 2)).sqrt().clamp_min(1e-12)
@@ -264,7 +278,7 @@ def encode_residual(target, st_base, K, chunk=64, scale=None):
     best = None
     for ci in range(Mbs.shape[1]):
         q = fold_value(Sb, Sr, Mbs[:, ci], Ns[:, ci]).float()
-        c = (target - q).double().square().sum((1, 2))
+        c = cost((target - q).double())
         if best is None:
             best = dict(c=c, Q=q, Mb=Mbs[:, ci].clone(), N=Ns[:, ci].clone())
         else:
@@ -274,21 +288,109 @@ def encode_residual(target, st_base, K, chunk=64, scale=None):
     return dict(states=st, Mb=best["Mb"], N=best["N"], Q=best["Q"], delta=delta)
 
 
+def pack_planes(r, N, K, st2, fits):
+    """ring states of the base plane [units, 8, 256] and the refinement fits {3: e3, 4: e4} (encode_residual's dicts over all
+    units) -> r gains base, states, Q and p3 / d3 / Q3 / states3, p4 / d4 / Q4 / states4"""
+    dev = st2.device
+    r["states"] = st2
+    r["base"] = signed32(lane_records(st2.reshape(-1, 256), 2).reshape(-1))
+    r["Q"] = from_rings(codebook(dev)[st2].reshape(-1, 256), N, K)
+    for lvl, e in fits.items():
+        bpw = lvl - 2
+        r["p%d" % lvl] = pack_words(lane_records(e["states"].reshape(-1, 256), bpw), 64 * bpw)
+        r["d%d" % lvl] = signed32(e["Mb"] | (e["N"] << 8))
+        r["Q%d" % lvl] = from_rings(e["Q"].reshape(-1, 256), N, K)
+        r["states%d" % lvl] = e["states"]
+    return r
+
+
 def encode_nested(W, seed=0, chunk=64):
     """encode_level2 plus the two refinement planes, each fitted to the residual of the same frozen base plane:
     p3 / d3 (one bit per weight, 64-bit records; level 3 = base + P3) and p4 / d4 (two bits per weight, 128-bit records of
     window code 0; level 4 = base + the wide plane). Adds p3, d3, Q3, p4, d4, Q4 (Q3 / Q4 fp32 [N, K]: the matrices the
     decoder reproduces bit for bit at levels 3 / 4) to encode_level2's dict."""
     N, K = W.shape
-    r = encode_level2(W, seed, chunk)
-    tr = to_rings(r["target"]).reshape(-1, 8, 256)
-    i32 = lambda t: torch.where(t >= 2**31, t - 2**32, t).to(torch.int32)
-    for lvl, bits_per_weight in ((3, 1), (4, 2)):
-        e = encode_residual(tr, r["states"], bits_per_weight, chunk)
-        r["p%d" % lvl] = pack_words(lane_records(e["states"].reshape(-1, 256), bits_per_weight), 64 * bits_per_weight)
-        r["d%d" % lvl] = i32(e["Mb"] | (e["N"] << 8))
-        r["Q%d" % lvl] = from_rings(e["Q"].reshape(-1, 256), N, K)
-        r["states%d" % lvl] = e["states"]
+    su, sv, target = prepare(W, seed)
+    tr = to_rings(target).reshape(-1, 8, 256)
+    st2 = viterbi_rings(tr.reshape(-1, 256), 2, chunk).reshape(-1, 8, 256)
+    fits = {lvl: encode_residual(tr, st2, lvl - 2, chunk) for lvl in (3, 4)}
+    return pack_planes(dict(su=su, sv=sv, target=target), N, K, st2, fits)
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# Hessian-aware fit: block LDL feedback (LDLQ) with one error state per level
+def block_ldl(H, b=128):
+    """H = L D L^T with L unit block lower triangular (identity diagonal blocks of size b) and D block diagonal:
+    from the Cholesky factor C, L = C diag(C_ii)^-1 and D_i = C_ii C_ii^T (reference nq_encode.py:115-132).
+    -> (L [n, n], D [n / b, b, b]), float64"""
+    n = H.shape[0]
+    m = n // b
+    C = torch.linalg.cholesky(H.double())
+    Cd = torch.stack([C[i * b:(i + 1) * b, i * b:(i + 1) * b] for i in range(m)])
+    L = torch.cat([C[:, i * b:(i + 1) * b] @ torch.linalg.inv(Cd[i]) for i in range(m)], 1)
+    return L, Cd @ Cd.transpose(1, 2)
+
+
+def rotated_hessian(H, su, sigma=0.01):
+    """second moment of the activations the quantised matrix multiplies: y = D(sv) B Q (B D(su) x), so
+    H' = B D(su) H D(su) B; then sigma * mean(diag) on the diagonal (reference nq_encode.py:141-147, which rotates with the
+    signs only and folds the scale into the weights instead)"""
+    Hs = H.double() * su.double()[:, None] * su.double()[None, :]
+    Hr = blocked_had(blocked_had(Hs, 0), 1)
+    return Hr + sigma * Hr.diagonal().mean() * torch.eye(H.shape[0], dtype=torch.float64, device=H.device)
+
+
+def proxy_loss(Q, target, Hr):
+    """tr((Q - T) H' (Q - T)^T) / tr(T H' T^T): the expected squared output error relative to the output's energy"""
+    E = Q.double() - target.double()
+    return float(((E @ Hr) * E).sum() / ((target.double() @ Hr) * target.double()).sum())
+
+
+def encode_ldlq(W, H, seed=0, chunk=64, lam=0.3, sigma=0.01):
+    """encode_nested for a layer whose input second moment H [K, K] is known: the 128-column chunks are fitted from the last
+    to the first, and each chunk's target is the weight plus the errors of the chunks already fitted, carried over by the
+    block LDL factor of H', T_a = W_a + sum_{b > a} E_b L[b, a] (reference nq_encode.py:206-339, its one-sided schedule).
+    Then tr(E H' E^T) = sum_a tr(eta_a D_a eta_a^T) with eta_a = T_a - Q_a the chunk's own fitting error. One error state
+    per level (the reference keeps two, for levels 2 and 4): the base plane is fitted to (1 - lam) T_2 + lam T_4, the refinement
+    planes to T_3 - Q_2 and T_4 - Q_2, their block words costed with D_a.
+    Adds Hr, D (the block diagonal factor), eta = {2, 3, 4: fp64 [N, K]} and proxy = {2, 3, 4: proxy_loss} to encode_nested's dict."""
+    N, K = W.shape
+    S, C = N // 16, K // 128
+    dev = W.device
+    su, sv, target = prepare(W, seed)
+    Hr = rotated_hessian(H.to(dev), su, sigma)
+    L, D = block_ldl(Hr)
+    Tg = target.double()
+    err = {lvl: torch.zeros(N, K, dtype=torch.float64, device=dev) for lvl in (2, 3, 4)}
+    eta = {lvl: torch.zeros(N, K, dtype=torch.float64, device=dev) for lvl in (2, 3, 4)}
+    st2 = torch.empty(S, C, 8, 256, dtype=torch.int64, device=dev)
+    fit = {lvl: dict(states=torch.empty(S, C, 8, 256, dtype=torch.int64, device=dev), Q=torch.empty(S, C, 8, 256, device=dev),
+                     Mb=torch.empty(S, C, dtype=torch.int64, device=dev), N=torch.empty(S, C, dtype=torch.int64, device=dev))
+           for lvl in (3, 4)}
+    rings = lambda M: to_rings(M.float()).reshape(S, 8, 256)     # a chunk [N, 128] is one unit per strip
+    for a in range(C - 1, -1, -1):
+        cols = slice(a * 128, (a + 1) * 128)
+        T = {lvl: Tg[:, cols] + err[lvl] @ L[:, cols] for lvl in (2, 3, 4)}      # later chunks only: the others' errors are still zero
+        tb = (1 - lam) * T[2] + lam * T[4]
+        sa = viterbi_rings(rings(tb).reshape(-1, 256), 2, chunk).reshape(S, 8, 256)
+        st2[:, a] = sa
+        q2 = from_rings(codebook(dev)[sa].reshape(-1, 256), N, 128).double()
+        err[2][:, cols], eta[2][:, cols] = Tg[:, cols] - q2, T[2] - q2
+        Da = D[a]
+
+        def cost(E):                                             # ring order -> [strip, 16 rows, 128 columns]
+            Eu = from_rings(E.reshape(-1, 256), N, 128).reshape(S, 16, 128)
+            return ((Eu @ Da) * Eu).sum((1, 2))
+        for lvl in (3, 4):
+            e = encode_residual(rings(T[lvl]), sa, lvl - 2, chunk, cost=cost)
+            for k in ("states", "Q", "Mb", "N"):
+                fit[lvl][k][:, a] = e[k]
+            q = from_rings(e["Q"].reshape(-1, 256), N, 128).double()
+            err[lvl][:, cols], eta[lvl][:, cols] = Tg[:, cols] - q, T[lvl] - q
+    flat = {lvl: dict(states=f["states"].reshape(-1, 8, 256), Q=f["Q"].reshape(-1, 8, 256), Mb=f["Mb"].reshape(-1), N=f["N"].reshape(-1))
+            for lvl, f in fit.items()}
+    r = pack_planes(dict(su=su, sv=sv, target=target, Hr=Hr, D=D, eta=eta), N, K, st2.reshape(-1, 8, 256), flat)
+    r["proxy"] = {2: proxy_loss(r["Q"], target, Hr), 3: proxy_loss(r["Q3"], target, Hr), 4: proxy_loss(r["Q4"], target, Hr)}
     return r
 
 
