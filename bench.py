@@ -601,6 +601,73 @@ def stream_leg(dev, nrec=48, nslot=32, nup=192, n_host=16, qd=8):
                 tier_GBps=round(nup * rb / dt_tier / 1e9, 2), tier_load_GBps=round(nrec * rb / dt_load / 1e9, 2))
 
 
+def dense_decode_leg(L, ex, dev, R=32, reps=4):
+    """the dense decoder on its own (planes -> rotated-domain fp16 matrices of one expert, gate|up [2I, H] and down [H, I]):
+    a graph of R experts in turn at each level, event-timed; bound by the fp16 it writes (2 bytes per weight against 0.25-0.5
+    read). fill_GBps is what torch's fill kernel reaches on the same two buffers: the write rate to compare with."""
+    from nestquant_amd import _lib
+    saved = L.table.clone()
+    picks = [(53 * i + 7) % E for i in range(R)]
+    bufs = [torch.empty(2 * I, H, dtype=torch.float16, device=dev), torch.empty(H, I, dtype=torch.float16, device=dev)]
+    s = torch.cuda.Stream()
+    written = 2 * 3 * H * I
+
+    def timed(body):
+        with torch.cuda.stream(s):
+            body()
+        torch.cuda.synchronize()
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr, stream=s):
+            body()
+        with torch.cuda.stream(s):
+            gr.replay()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(s)
+            for _ in range(reps):
+                gr.replay()
+            e1.record(s)
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / (reps * R)
+
+    out = {}
+    for lv in (2, 3, 4):
+        for e in picks:
+            L.set(e, ex[e], lv)
+        rows = [L.table[e] for e in picks]
+
+        def body():
+            for row in rows:
+                for proj in (0, 1):
+                    M.dequant(row, proj, H, I, out=bufs[proj])
+        us = timed(body)
+        out[f"L{lv}"] = dict(us_per_expert=round(us, 2), write_GBps=round(written / us / 1e3, 1), hbm_frac=round(written / us / 1e3 / HBM_PEAK_GBS, 4))
+
+        # the grouped form (the reference's pf_decode over a group of 16 experts): one launch, 1.2 GB written
+        G = 16
+        if "Wg" not in out:
+            out["Wg"] = (torch.empty(G, 2 * I, H, dtype=torch.float16, device=dev), torch.empty(G, H, I, dtype=torch.float16, device=dev))
+        ids = torch.tensor(picks[:G], dtype=torch.int32, device=dev)
+        Wg, Wd = out["Wg"]
+
+        def grouped():
+            for _ in range(R // G):
+                _lib.check(_lib.lib().nq_pf_decode(L.table.data_ptr(), ids.data_ptr(), G, Wg.data_ptr(), Wd.data_ptr(), H, I, _lib.stream_ptr()))
+        us = timed(grouped)
+        out[f"L{lv}"].update(grouped16_us_per_expert=round(us, 2), grouped16_write_GBps=round(written / us / 1e3, 1),
+                              grouped16_hbm_frac=round(written / us / 1e3 / HBM_PEAK_GBS, 4))
+    del out["Wg"]
+
+    def fill():
+        for _ in range(R):
+            bufs[0].fill_(1.0); bufs[1].fill_(1.0)
+    us = timed(fill)
+    out["fill_GBps"] = round(written / us / 1e3, 1)
+    L.table.copy_(saved)
+    out["workload"] = (f"{R} experts in turn in one graph, both projections of each (nq_dequant: 2 launches per expert, {written / 1e6:.1f} MB of fp16 "
+                       "written per expert); grouped16: nq_pf_decode, 16 experts and both projections in one launch")
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -611,6 +678,7 @@ def main():
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill (4096 tokens) leg")
     ap.add_argument("--no-churn", action="store_true", help="skip the plane-churn leg")
     ap.add_argument("--no-config2", action="store_true", help="skip the single-projection leg (per-level GB/s at 1 / 4 / 8 tokens)")
+    ap.add_argument("--no-dense", action="store_true", help="skip the dense-decode leg (planes -> fp16 matrices of one expert)")
     ap.add_argument("--no-stream", action="store_true", help="skip the record upgrade engine leg (file -> pinned -> slot)")
     ap.add_argument("--no-caller", action="store_true", help="skip the caller-dtype leg (bf16 / fp32 / int32 tensors)")
     ap.add_argument("--no-batches", action="store_true", help="skip the 1-4 token table (mixed levels, all 2 bit, all 4 bit)")
@@ -767,6 +835,7 @@ def main():
         churn["torch_copies"] = {k: t[k] for k in ("step_us_churn", "ops", "refused", "h2d_GBps", "lag_steps_median", "lag_steps_max")}
     stream = None if a.no_stream else stream_leg(dev)
     config2 = None if a.no_config2 else config2_leg(L, ex, levels, dev)
+    dense = None if a.no_dense else dense_decode_leg(L, ex, dev)
     print(json.dumps({
         "metric": "MoE layer us + HBM GB/s (decode bs1 top-8); prefill grouped-GEMM TFLOP/s",
         "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": W,
@@ -777,7 +846,7 @@ def main():
         "config": {"workload": f"decode MoE layer: E=256 top-8 B={B}, H=6144 I=2048, levels 2/3/4 = "
                                f"{lv_counts[2]}/{lv_counts[3]}/{lv_counts[4]} experts, seeded softmax routing avoiding the previous step",
                    "code_MB_per_step": round(nbytes / K / 1e6, 2), "hbm_frac_layer": round(gbs / HBM_PEAK_GBS, 4)},
-        "roofline": roofline, "cpu_baseline": cpu, "prefill": prefill, "batches": batches, "caller_dtypes": caller, "churn": churn, "stream": stream, "config2": config2}))
+        "roofline": roofline, "cpu_baseline": cpu, "prefill": prefill, "batches": batches, "caller_dtypes": caller, "churn": churn, "stream": stream, "config2": config2, "dense_decode": dense}))
 
 
 if __name__ == "__main__":
