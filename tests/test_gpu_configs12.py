@@ -66,6 +66,34 @@ def test_config1_encode_decode_gemv():
         print("config 1 level %d: dequant bit-exact, GEMV rel err %.1e, vs unquantised W x %.3f" % (level, rel_err(y, want), rel_err(y, exact)))
 
 
+def test_hessian_aware_fit_on_the_gpu_decodes_bit_for_bit():
+    """encode_ldlq run on the GPU (256 x 256 weight, activations with shared strong directions): its three matrices are what
+    the HIP decoder reproduces from its planes, and the expected output error is below the H-agnostic fit's at every level"""
+    N, K = 256, 256
+    g = torch.Generator().manual_seed(5)
+    W = torch.randn(N, K, generator=g)
+    V = torch.randn(4, K, generator=g)
+    X = torch.randn(4096, 4, generator=g) @ V * 1.5 + torch.randn(4096, K, generator=g)
+    Hx = (X.T @ X / 4096).double()
+    r = EN.encode_ldlq(W.to(DEV), Hx.to(DEV), seed=3)
+    r0 = EN.encode_nested(W.to(DEV), seed=3)
+    H, I = K, N // 2
+    ex = _Ex()
+    ex.H, ex.I, ex.nested, ex.lr = H, I, False, None
+    ex.gu = EN.EncodedProj(N, K, r["base"], r["p3"], r["d3"], r["p4"], r["d4"])
+    zd = F.proj_sizes(H, I)
+    zeros = lambda n: torch.zeros(n, dtype=torch.int32, device=DEV)
+    unit_words = torch.ones(zd["S"] * zd["C"], dtype=torch.int32, device=DEV)
+    ex.dn = EN.EncodedProj(H, I, zeros(zd["base"] // 4), zeros(zd["nrec_r"] * 2), unit_words, zeros(zd["nrec_r"] * 4), unit_words)
+    ex.signs = torch.ones(2 * H + 3 * I + H, dtype=torch.float16, device=DEV)
+    for level, key in ((2, "Q"), (3, "Q3"), (4, "Q4")):
+        assert same_f16(M.dense_W(ex, 0, level).cpu().numpy(), r[key].half().cpu().numpy()) == 0
+        plain = EN.proxy_loss(r0[key], r["target"], r["Hr"])
+        assert r["proxy"][level] < 0.8 * plain, (level, r["proxy"][level], plain)
+    print("LDLQ fit: expected output error %s against %s without H" % (
+        {k: round(v, 4) for k, v in r["proxy"].items()}, [round(EN.proxy_loss(r0[k], r["target"], r["Hr"]), 4) for k in ("Q", "Q3", "Q4")]))
+
+
 @pytest.mark.parametrize("level", [2, 3, 4])
 def test_config2_single_projection(level):
     """6144 -> 2048 as the gate|up projection of an expert with I = 1024 (2I = 2048 rows), B = 1 / 4 / 8"""
