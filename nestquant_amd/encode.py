@@ -258,16 +258,35 @@ def block_word_candidates(delta):
     return torch.where(ok, Mb, Mb0[:, None]), torch.where(ok, N, N0[:, None].clamp_max(255))
 
 
-def encode_residual(target, st_base, K, chunk=64, scale=None, cost=None):
+def base_rings(rings, chunk=64, var=False):
+    """base plane of rings [T, 256] (ring position order) -> (states int64 [T, 256], sign fp32 [T, 1]): with var, each ring is
+    fitted as it is and negated, and keeps the better of the two by its squared error (the reference's 'sign' base variant,
+    nq_encode.py:87-113; the decoder negates the ring's values, table words 12 / 13)"""
+    T = rings.shape[0]
+    st = viterbi_rings(torch.cat([rings, -rings]) if var else rings, 2, chunk)
+    sign = torch.ones(T, 1, device=rings.device)
+    if var:
+        lut = codebook(rings.device)
+        e_pos = (lut[st[:T]] - rings).square().sum(1)
+        e_neg = (lut[st[T:]] + rings).square().sum(1)
+        neg = e_neg < e_pos
+        st = torch.where(neg[:, None], st[T:], st[:T])
+        sign[neg] = -1.0
+    return st, sign
+
+
+def encode_residual(target, st_base, K, chunk=64, scale=None, cost=None, sign=None):
     """One refinement stage on the frozen base plane. target fp32 [U, 8, 256] and st_base int64 [U, 8, 256] in ring position
     order, K = 1 or 2 bits per weight -> dict(states [U, 8, 256], Mb [U], N [U], Q fp32 [U, 8, 256], delta [U]).
-    cost: error fp64 [U, 8, 256] -> [U], what the block-word search minimises (default: the squared error)."""
+    cost: error fp64 [U, 8, 256] -> [U], what the block-word search minimises (default: the squared error).
+    sign [U, 8, 1] (+-1): rings whose decoded values are negated, base and refinement alike."""
     U = target.shape[0]
     dev = target.device
     lut = codebook(dev)
     cost = cost or (lambda E: E.square().sum((1, 2)))
+    sign = torch.ones(U, 8, 1, device=dev) if sign is None else sign
     Sb = hash_sum(st_base)
-    r = target.double() - lut[st_base].double()
+    r = (target * sign).double() - lut[st_base].double()         # in the ring's own orientation
     rms = r.square().mean((1, 2)).sqrt().clamp_min(1e-12)
     s0 = rms / (RES_SCALE[K] if scale is None else scale)
     st = viterbi_rings((r / s0[:, None, None]).float().reshape(U * 8, 256), K, chunk).reshape(U, 8, 256)
@@ -277,7 +296,7 @@ def encode_residual(target, st_base, K, chunk=64, scale=None, cost=None):
     Mbs, Ns = block_word_candidates(delta)
     best = None
     for ci in range(Mbs.shape[1]):
-        q = fold_value(Sb, Sr, Mbs[:, ci], Ns[:, ci]).float()
+        q = fold_value(Sb, Sr, Mbs[:, ci], Ns[:, ci]).float() * sign
         c = cost((target - q).double())
         if best is None:
             best = dict(c=c, Q=q, Mb=Mbs[:, ci].clone(), N=Ns[:, ci].clone())
@@ -288,13 +307,19 @@ def encode_residual(target, st_base, K, chunk=64, scale=None, cost=None):
     return dict(states=st, Mb=best["Mb"], N=best["N"], Q=best["Q"], delta=delta)
 
 
-def pack_planes(r, N, K, st2, fits):
-    """ring states of the base plane [units, 8, 256] and the refinement fits {3: e3, 4: e4} (encode_residual's dicts over all
-    units) -> r gains base, states, Q and p3 / d3 / Q3 / states3, p4 / d4 / Q4 / states4"""
+def pack_planes(r, N, K, st2, fits, sign=None):
+    """ring states of the base plane [units, 8, 256], the refinement fits {3: e3, 4: e4} (encode_residual's dicts over all
+    units) and the ring signs [units, 8, 1] (None: all +1) -> r gains base, states, Q and p3 / d3 / Q3 / states3,
+    p4 / d4 / Q4 / states4, and with signs var (uint8 per unit, bit g = ring g negated)"""
     dev = st2.device
     r["states"] = st2
     r["base"] = signed32(lane_records(st2.reshape(-1, 256), 2).reshape(-1))
-    r["Q"] = from_rings(codebook(dev)[st2].reshape(-1, 256), N, K)
+    q2 = codebook(dev)[st2]
+    r["var"] = None
+    if sign is not None:
+        q2 = q2 * sign
+        r["var"] = ((sign.reshape(-1, 8) < 0).long() << torch.arange(8, device=dev)).sum(1).to(torch.uint8)
+    r["Q"] = from_rings(q2.reshape(-1, 256), N, K)
     for lvl, e in fits.items():
         bpw = lvl - 2
         r["p%d" % lvl] = pack_words(lane_records(e["states"].reshape(-1, 256), bpw), 64 * bpw)
@@ -304,17 +329,19 @@ def pack_planes(r, N, K, st2, fits):
     return r
 
 
-def encode_nested(W, seed=0, chunk=64):
+def encode_nested(W, seed=0, chunk=64, var=False):
     """encode_level2 plus the two refinement planes, each fitted to the residual of the same frozen base plane:
     p3 / d3 (one bit per weight, 64-bit records; level 3 = base + P3) and p4 / d4 (two bits per weight, 128-bit records of
     window code 0; level 4 = base + the wide plane). Adds p3, d3, Q3, p4, d4, Q4 (Q3 / Q4 fp32 [N, K]: the matrices the
-    decoder reproduces bit for bit at levels 3 / 4) to encode_level2's dict."""
+    decoder reproduces bit for bit at levels 3 / 4) to encode_level2's dict. var: also fit every ring negated and keep the
+    better orientation (adds the sign plane `var`)."""
     N, K = W.shape
     su, sv, target = prepare(W, seed)
     tr = to_rings(target).reshape(-1, 8, 256)
-    st2 = viterbi_rings(tr.reshape(-1, 256), 2, chunk).reshape(-1, 8, 256)
-    fits = {lvl: encode_residual(tr, st2, lvl - 2, chunk) for lvl in (3, 4)}
-    return pack_planes(dict(su=su, sv=sv, target=target), N, K, st2, fits)
+    st2, sign = base_rings(tr.reshape(-1, 256), chunk, var)
+    st2, sign = st2.reshape(-1, 8, 256), sign.reshape(-1, 8, 1)
+    fits = {lvl: encode_residual(tr, st2, lvl - 2, chunk, sign=sign) for lvl in (3, 4)}
+    return pack_planes(dict(su=su, sv=sv, target=target), N, K, st2, fits, sign if var else None)
 
 
 # ----------------------------------------------------------------------------------------------------------------------
@@ -346,7 +373,7 @@ def proxy_loss(Q, target, Hr):
     return float(((E @ Hr) * E).sum() / ((target.double() @ Hr) * target.double()).sum())
 
 
-def encode_ldlq(W, H, seed=0, chunk=64, lam=0.3, sigma=0.01):
+def encode_ldlq(W, H, seed=0, chunk=64, lam=0.3, sigma=0.01, var=False):
     """encode_nested for a layer whose input second moment H [K, K] is known: the 128-column chunks are fitted from the last
     to the first, and each chunk's target is the weight plus the errors of the chunks already fitted, carried over by the
     block LDL factor of H', T_a = W_a + sum_{b > a} E_b L[b, a] (reference nq_encode.py:206-339, its one-sided schedule).
@@ -364,6 +391,7 @@ def encode_ldlq(W, H, seed=0, chunk=64, lam=0.3, sigma=0.01):
     err = {lvl: torch.zeros(N, K, dtype=torch.float64, device=dev) for lvl in (2, 3, 4)}
     eta = {lvl: torch.zeros(N, K, dtype=torch.float64, device=dev) for lvl in (2, 3, 4)}
     st2 = torch.empty(S, C, 8, 256, dtype=torch.int64, device=dev)
+    sign = torch.ones(S, C, 8, 1, device=dev)
     fit = {lvl: dict(states=torch.empty(S, C, 8, 256, dtype=torch.int64, device=dev), Q=torch.empty(S, C, 8, 256, device=dev),
                      Mb=torch.empty(S, C, dtype=torch.int64, device=dev), N=torch.empty(S, C, dtype=torch.int64, device=dev))
            for lvl in (3, 4)}
@@ -372,9 +400,10 @@ def encode_ldlq(W, H, seed=0, chunk=64, lam=0.3, sigma=0.01):
         cols = slice(a * 128, (a + 1) * 128)
         T = {lvl: Tg[:, cols] + err[lvl] @ L[:, cols] for lvl in (2, 3, 4)}      # later chunks only: the others' errors are still zero
         tb = (1 - lam) * T[2] + lam * T[4]
-        sa = viterbi_rings(rings(tb).reshape(-1, 256), 2, chunk).reshape(S, 8, 256)
-        st2[:, a] = sa
-        q2 = from_rings(codebook(dev)[sa].reshape(-1, 256), N, 128).double()
+        sa, sg = base_rings(rings(tb).reshape(-1, 256), chunk, var)
+        sa, sg = sa.reshape(S, 8, 256), sg.reshape(S, 8, 1)
+        st2[:, a] = sa; sign[:, a] = sg
+        q2 = from_rings((codebook(dev)[sa] * sg).reshape(-1, 256), N, 128).double()
         err[2][:, cols], eta[2][:, cols] = Tg[:, cols] - q2, T[2] - q2
         Da = D[a]
 
@@ -382,29 +411,31 @@ def encode_ldlq(W, H, seed=0, chunk=64, lam=0.3, sigma=0.01):
             Eu = from_rings(E.reshape(-1, 256), N, 128).reshape(S, 16, 128)
             return ((Eu @ Da) * Eu).sum((1, 2))
         for lvl in (3, 4):
-            e = encode_residual(rings(T[lvl]), sa, lvl - 2, chunk, cost=cost)
+            e = encode_residual(rings(T[lvl]), sa, lvl - 2, chunk, cost=cost, sign=sg)
             for k in ("states", "Q", "Mb", "N"):
                 fit[lvl][k][:, a] = e[k]
             q = from_rings(e["Q"].reshape(-1, 256), N, 128).double()
             err[lvl][:, cols], eta[lvl][:, cols] = Tg[:, cols] - q, T[lvl] - q
     flat = {lvl: dict(states=f["states"].reshape(-1, 8, 256), Q=f["Q"].reshape(-1, 8, 256), Mb=f["Mb"].reshape(-1), N=f["N"].reshape(-1))
             for lvl, f in fit.items()}
-    r = pack_planes(dict(su=su, sv=sv, target=target, Hr=Hr, D=D, eta=eta), N, K, st2.reshape(-1, 8, 256), flat)
+    r = pack_planes(dict(su=su, sv=sv, target=target, Hr=Hr, D=D, eta=eta), N, K, st2.reshape(-1, 8, 256), flat,
+                    sign.reshape(-1, 8, 1) if var else None)
     r["proxy"] = {2: proxy_loss(r["Q"], target, Hr), 3: proxy_loss(r["Q3"], target, Hr), 4: proxy_loss(r["Q4"], target, Hr)}
     return r
 
 
 class EncodedProj(Proj):
     """a Proj (nestquant_amd.format) holding encoded planes: the level-2 base plane and, when given, the refinement planes
-    p3 / d3 (level 3, the one-bit nested plane) and p4 / d4 (level 4, wide plane of window code 0)"""
+    p3 / d3 (level 3, the one-bit nested plane), p4 / d4 (level 4, wide plane of window code 0) and the sign plane var"""
 
-    def __init__(s, N, K, base, p3=None, d3=None, p4=None, d4=None):
+    def __init__(s, N, K, base, p3=None, d3=None, p4=None, d4=None, var=None):
         s.z = proj_sizes(N, K)
         s.N, s.K, s.rk, s.bk, s.nested = N, K, 0, 0, False
         s.base = base
         zero = lambda: torch.zeros(1, dtype=torch.int32, device=base.device)
         s.p4 = zero() if p4 is None else p4
         s.d4 = zero() if d4 is None else d4
-        s.p4w = s.Mb = s.Nn = s.var = s.flags = s.fl = None
+        s.p4w = s.Mb = s.Nn = s.flags = s.fl = None
+        s.var = var
         s.p3, s.d3 = p3, d3
         s.p4n = s.d4n = s.p3w = s.p4nw = None

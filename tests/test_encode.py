@@ -117,11 +117,19 @@ def test_encode_decode_round_trip_through_the_oracle():
     g = torch.Generator().manual_seed(2)
     N, K = 128, 128
     W = torch.randn(N, K, generator=g) * torch.linspace(0.5, 2.0, K)[None]        # uneven input channels
-    r = EN.encode_nested(W, seed=3)
+    r = EN.encode_nested(W, seed=3, var=True)                    # with the sign plane: every ring in its better orientation
     nrec = (N // 16) * (K // 128) * 32
     p = O.Plane(N, K, u32(r["base"]).reshape(-1, 4), rk=0,
                 res=O.unpack_words(r["p4"].numpy(), nrec, 128), d4=u32(r["d4"]),
-                p3=O.unpack_words(r["p3"].numpy(), nrec, 64), d3=u32(r["d3"]))
+                p3=O.unpack_words(r["p3"].numpy(), nrec, 64), d3=u32(r["d3"]), var=r["var"].numpy())
+    negated = int(((r["var"].long()[:, None] >> torch.arange(8)) & 1).sum())
+    assert 16 <= negated <= 48                                    # of 64 rings: about half are better negated
+    # a negated ring is at least as good as the ring fitted as it is
+    tr = EN.to_rings(r["target"])
+    plain = EN.viterbi_rings(tr, 2)
+    e_plain = (EN.codebook()[plain] - tr).square().sum(1)
+    e_var = (EN.to_rings(r["Q"]) - tr).square().sum(1)
+    assert bool((e_var <= e_plain + 1e-6).all()) and float(e_var.sum()) < float(e_plain.sum())
     B = lambda X, d: EN.blocked_had(X, d)
     # W ~= D(sv) B Q B D(su): relative error of the code on Gaussian data is sqrt(0.068), sqrt(0.0187), sqrt(0.0047)
     for level, key, lo, hi in ((2, "Q", 0.22, 0.30), (3, "Q3", 0.12, 0.155), (4, "Q4", 0.06, 0.078)):

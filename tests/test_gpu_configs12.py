@@ -75,12 +75,13 @@ def test_hessian_aware_fit_on_the_gpu_decodes_bit_for_bit():
     V = torch.randn(4, K, generator=g)
     X = torch.randn(4096, 4, generator=g) @ V * 1.5 + torch.randn(4096, K, generator=g)
     Hx = (X.T @ X / 4096).double()
-    r = EN.encode_ldlq(W.to(DEV), Hx.to(DEV), seed=3)
+    r = EN.encode_ldlq(W.to(DEV), Hx.to(DEV), seed=3, var=True)  # with the sign plane: rings the decoder negates
     r0 = EN.encode_nested(W.to(DEV), seed=3)
+    assert 0 < int(r["var"].count_nonzero()) <= r["var"].numel()
     H, I = K, N // 2
     ex = _Ex()
     ex.H, ex.I, ex.nested, ex.lr = H, I, False, None
-    ex.gu = EN.EncodedProj(N, K, r["base"], r["p3"], r["d3"], r["p4"], r["d4"])
+    ex.gu = EN.EncodedProj(N, K, r["base"], r["p3"], r["d3"], r["p4"], r["d4"], var=r["var"])
     zd = F.proj_sizes(H, I)
     zeros = lambda n: torch.zeros(n, dtype=torch.int32, device=DEV)
     unit_words = torch.ones(zd["S"] * zd["C"], dtype=torch.int32, device=DEV)
