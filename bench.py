@@ -313,6 +313,15 @@ def prefill_parts(L, x, sel, dev):
         rec[f"height_{bm}"] = dict(tiles=int(valid.sum()), hot_tiles=int((tl[i, :nt, 3][valid] > 0).sum()), rows=rows, gate_up_us=round(gu, 0),
                                    down_us=round(dn, 0), mfma_frac=round(rows * 6 * H * I / (gu + dn) / 1e6 / MFMA_PEAK_TFLOPS, 3))
     rec["sum_us"] = round(tot, 0)
+    # the two memory-bound kernels either side of the gate|up GEMM, over all pair rows at once (inside the call they run per
+    # tile height under the GEMMs of other heights): rotation of the tokens, and SwiGLU between the projections
+    pre = us(lambda: _lib.check(Lb.nq_pf_pre(x.data_ptr(), pt.data_ptr(), pe.data_ptr(), P, tb.data_ptr(), S["xg"].data_ptr(), S["xu"].data_ptr(),
+                                             S["zg"].data_ptr(), E, H, I, st)))
+    mid = us(lambda: _lib.check(Lb.nq_pf_mid(S["acc"].data_ptr(), pe.data_ptr(), P, tb.data_ptr(), S["h"].data_ptr(), S["zg"].data_ptr(),
+                                             S["zd"].data_ptr(), E, H, I, st)))
+    rec["pre_us"], rec["mid_us"] = round(pre, 0), round(mid, 0)
+    rec["pre_GBps"] = round((T * H * 2 + 2 * P * H * 2) / pre / 1e3, 0)
+    rec["mid_GBps"] = round((P * 2 * I * 4 + P * I * 2) / mid / 1e3, 0)
     return rec
 
 
