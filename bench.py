@@ -504,7 +504,9 @@ def config2_leg(L, ex, levels, dev, R=64, reps=4):
     """config 2: one expert's fused gate|up projection (6144 -> 2 x 2048, decode + GEMV without the layer around it) at each
     level for 1 / 4 / 8 tokens: a graph of R calls over R different experts (cold weights), event-timed; GB/s of the code
     bytes the launch reads at that level. us = the call (routing launch + projection launch with its SwiGLU finisher);
-    us_projection_launch = the projection launch with its finisher alone, routing prepared beforehand"""
+    us_projection_launch = the projection launch with its finisher alone, routing prepared beforehand; us_to_partial_sums =
+    the same launch in the form the layer call runs it (which = 1 | 4 | 8): decode + GEMV into k-slice partial sums, which the
+    down launch adds up while it forms h, no arrival counter and no finisher in this launch"""
     saved = L.table.clone()
     g = torch.Generator().manual_seed(2)
     s = torch.cuda.Stream()
@@ -544,36 +546,42 @@ def config2_leg(L, ex, levels, dev, R=64, reps=4):
                     best = (us, nst)
             # the projection launch by itself: each expert's routing and rotated activations prepared beforehand in workspaces
             # of its own (which = 0, then which = 1 | 4), so the graph holds R projection launches and nothing else
-            cfg = [1, L.cfg_gu[1], best[1]]
             own, keep = [], (L.route, L.xrot)
             for q in sels:
                 L.route, L.xrot = torch.zeros_like(keep[0]), torch.zeros_like(keep[1])
                 own.append((L.route, L.xrot))
                 with torch.cuda.stream(s):
-                    L(x, q, rw, which=0, cfg_gu=cfg)
+                    L(x, q, rw, which=0)
 
-            def launches():
-                for q, (ro, xr) in zip(sels, own):
-                    L.route, L.xrot = ro, xr
-                    L(x, q, rw, which=1 | 4, cfg_gu=cfg)
-            with torch.cuda.stream(s):
-                launches()
-            torch.cuda.synchronize()
-            gr = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(gr, stream=s):
-                launches()
-            with torch.cuda.stream(s):
-                gr.replay()
-                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                e0.record(s)
-                for _ in range(reps):
+            def alone(which, nst):
+                cfg = [1, L.cfg_gu[1], nst]
+
+                def launches():
+                    for q, (ro, xr) in zip(sels, own):
+                        L.route, L.xrot = ro, xr
+                        L(x, q, rw, which=which, cfg_gu=cfg)
+                with torch.cuda.stream(s):
+                    launches()
+                torch.cuda.synchronize()
+                gr = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(gr, stream=s):
+                    launches()
+                with torch.cuda.stream(s):
                     gr.replay()
-                e1.record(s)
-            torch.cuda.synchronize()
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record(s)
+                    for _ in range(reps):
+                        gr.replay()
+                    e1.record(s)
+                torch.cuda.synchronize()
+                return e0.elapsed_time(e1) * 1e3 / (reps * R)
+            fin = alone(1 | 4, best[1])
+            part = min((alone(1 | 4 | 8, nst), nst) for nst in (6, 3, 2))      # as the layer runs it: ends with the k-slice partial sums
             L.route, L.xrot = keep
-            alone = e0.elapsed_time(e1) * 1e3 / (reps * R)
             out[f"L{lv}_B{B}"] = dict(us=round(best[0], 2), GBps=round(nbytes / best[0] / 1e3, 1), k_slice_chunks=best[1],
-                                      us_projection_launch=round(alone, 2), GBps_projection_launch=round(nbytes / alone / 1e3, 1))
+                                      us_projection_launch=round(fin, 2), GBps_projection_launch=round(nbytes / fin / 1e3, 1),
+                                      us_to_partial_sums=round(part[0], 2), GBps_to_partial_sums=round(nbytes / part[0] / 1e3, 1),
+                                      k_slice_chunks_to_partial_sums=part[1])
     L.table.copy_(saved)
     out["workload"] = ("one expert's gate|up projection per launch (N=4096, K=6144), 64 experts in turn, best k-slice of 12 / 6 / 3 / 2 chunks; "
                        "code bytes per launch: " + ", ".join(f"L{lv} {int(sum(code_bytes(ex, [lv] * E, [e], which='gu') for e in picks) / R)}" for lv in (2, 3, 4)))
