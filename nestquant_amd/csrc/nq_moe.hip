@@ -76,7 +76,7 @@ __device__ __forceinline__ void sum_partials(const float* const* p, size_t strid
 // ---- caller dtypes: the casts a caller would otherwise launch as separate kernels (x.half(), ids.long(), w.half(),
 // out.to(x.dtype); reference sm120/serve/nq_vllm.py:522,560,573) happen at the loads and the final store, with the same
 // roundings: activations and routing weights pass through fp16, the fp32 result is rounded once to the output type.
-constexpr int DT_DEFAULT = 0, DT_BF16 = 1, DT_F32 = 2, DT_I32 = 1, DT_OUT_F16 = 1, DT_OUT_BF16 = 2;
+constexpr int DT_BF16 = 1, DT_F32 = 2, DT_I32 = 1, DT_OUT_F16 = 1, DT_OUT_BF16 = 2;   // 0 = the default type of each argument (fp16, int64, fp32 out)
 __device__ __forceinline__ float bf16_to_f(uint16_t v) { return __builtin_bit_cast(float, (uint32_t)v << 16); }
 __device__ __forceinline__ uint16_t f_to_bf16(float f)           // round to nearest even; NaN stays NaN
 {
