@@ -20,7 +20,7 @@ extern "C" {
 #endif
 
 #define NQ_TBL_W 20
-#define NQ_ABI_VERSION 2
+#define NQ_ABI_VERSION 3
 
 /* library identification; no counterpart in the reference (its module is rebuilt per process by sm120/build.py:7-12) */
 int nq_abi_version(void);
@@ -64,7 +64,8 @@ int nq_pf_decode(const int64_t* table, const int32_t* experts, int G, void* Wgu_
  * and rotation of the activations) because route_ws and xrot still hold what an earlier call with the same x, sel, rw and table
  * rows left there (what a benchmark of one projection launch alone uses); bit 3 = the two launches come as two calls but with the
  * arithmetic of one: the gate|up call (which = 1 | 8) leaves h to the down call (which = 2 | 4 | 8), which forms it from the gate|up
- * partial sums exactly as a which = 3 call does (same bits). hits: optional int32[E] pick counters
+ * partial sums exactly as a which = 3 call does (same bits). Calls that share a routing (bits 2 / 3) must agree in B, topk, x, sel,
+ * rw and cfg_gu's sb; the number of gate|up k-slices is taken from what the gate|up launch recorded in route_ws. hits: optional int32[E] pick counters
  * (device or host-mapped memory), incremented once per pick with rw != 0 (reference :784-787). */
 /* Element types of the caller's tensors. The casts the reference's caller launches around the call (x.half(), ids.long(),
  * w.half(), out.to(x.dtype): sm120/serve/nq_vllm.py:522,560,573; fusing them is the open item of
@@ -112,7 +113,7 @@ typedef struct NqMoeArgs
                                  records (the format every artifact uses), 2 = the same planes read as rings of two records
                                  (the reference's test variant; not with sign-variant planes, not in prefill) */
     void* route_ws;           /* NQ_ROUTE_WS_BYTES of device memory, 64-byte aligned, contents irrelevant on entry: the call's first
-                                 launch (one workgroup) does the routing once -- picks -> runs of distinct experts with their table
+                                 launch does the routing once (every workgroup for itself, one of them writes the result) -- picks -> runs of distinct experts with their table
                                  rows (reference route(), sm120/nqmoe.cu:379-449, which every block of the reference repeats) -- and
                                  leaves it here for the two projection launches */
     int64_t route_ws_bytes;
@@ -120,11 +121,18 @@ typedef struct NqMoeArgs
                                  activations of every active pick, once (x * su_g and x * su_u -> Hadamard-128 -> fp16; reference
                                  sm120/nqmoe.cu:506-519, which every block repeats for its k-slice), for the gate|up launch */
     int64_t xrot_elems;
-    int64_t* mb_table;        /* optional mailbox: the effect of nq_mailbox(mb_table, mb_stage, mb_seq, mb_applied, mb_applied_host, E)
-                                 followed by the layer call, without a launch of its own (the reference's caller applies the mailbox
-                                 at the top of every layer step, sm120/serve/nq_vllm.py:546): the routing launch takes the staged row
-                                 of every picked expert whose update is pending, and one extra workgroup of the first projection
-                                 launch writes the table and publishes applied. NULL = no mailbox in this call; otherwise == table */
+    int64_t* mb_table;        /* optional mailbox of the call, without a launch of its own (the reference's caller launches nq_mailbox
+                                 at the top of every layer step, sm120/serve/nq_vllm.py:546). Two halves, one observer each:
+                                 (1) one extra workgroup of the call's LAST projection launch does table[e] <- stage[e] and
+                                 mb_applied[e] <- mb_seq[e] for every e whose seq differs -- after this call's routing has read the
+                                 table, so this call works from the rows as they were when it started and the next call from the
+                                 new ones; (2) the routing launch of the NEXT call with this mailbox (or the next nq_mailbox) copies
+                                 mb_applied to mb_applied_host. A row whose seq lands while call n runs is thus used and published
+                                 from call n + 1 on, as with nq_mailbox at the top of call n + 1; applied_host[e] == seq[e] still
+                                 means that no launch enqueued from then on reads the slot the replaced row named (reference
+                                 threads/13-moe-layer-kernel/INTEGRATION.md:226-227). The last published state lags the table by one
+                                 call: a caller that stops calling and wants it published launches nq_mailbox once.
+                                 NULL = no mailbox in this call; otherwise == table */
     const int64_t* mb_stage;
     const int32_t* mb_seq;
     int32_t* mb_applied;
@@ -147,8 +155,9 @@ int nq_moe_forward(const NqMoeArgs* args, void* stream);
 #define NQ_STATIC_SCRATCH_BYTES (16u << 20)
 int nq_moe_forward_static(const NqMoeArgs* args, void* stream);
 
-/* table[e] <- stage[e] for every e with seq[e] != applied[e]; then applied[e] <- seq[e], mirrored to applied_host
- * [host-mapped, optional]. Replaces mailbox (reference sm120/nqmoe.cu:908-929). */
+/* table[e] <- stage[e] for every e with seq[e] != applied[e]; then applied[e] <- seq[e]; applied_host [host-mapped, optional]
+ * receives every entry of applied (also those an earlier layer call's mailbox block applied without publishing them).
+ * Replaces mailbox (reference sm120/nqmoe.cu:908-929). */
 int nq_mailbox(int64_t* table, const int64_t* stage, const int32_t* seq, int32_t* applied, int32_t* applied_host, int E,
                void* stream);
 

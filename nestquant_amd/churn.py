@@ -4,8 +4,8 @@ The part of the reference's streaming runtime that touches the hot path (streami
 streaming/nqstream.cu:183-191 `issue_copies`, sm120/levelswitch_mbox.py:33-65): for an upgrade, copy the expert's
 refinement planes from pinned host memory into a free device slot with asynchronous copies (hipMemcpyAsync under
 torch's non_blocking copy_), then the new table row into `stage[e]`, then bump `seq[e]` -- all on ONE side stream, in
-that order; for a downgrade, post only the row. The compute stream never waits: `Mailbox.apply()` at the start of each
-layer call flips the rows whose `seq` changed. SSD / io_uring / LRU tiers of the reference engine are out of scope:
+that order; for a downgrade, post only the row. The compute stream never waits: the mailbox (`Mailbox.apply()` at the start of
+each layer call, or the layer call's own `mailbox=`) flips the rows whose `seq` changed. SSD / io_uring / LRU tiers of the reference engine are out of scope:
 the host store here is plain pinned RAM.
 
 Slot image of a nested expert (bytes, every part 256-byte aligned):
@@ -98,6 +98,9 @@ class ChurnExecutor:
         """table row of expert e at `level`; levels 3 / 4 point into `slot`"""
         r = s.base_row[e].clone()
         r[0] = level
+        sc = getattr(s.ex[e], "sc", None)                          # served experts carry one sign / scale vector per level
+        if sc is not None:
+            r[9] = sc[level].data_ptr()
         if level >= 3:
             b = s.slots[slot].data_ptr()
             p = s.lay.parts

@@ -106,7 +106,7 @@ static int moe_args(const char* who, const NqMoeArgs* p, bool own_ws, MoeArgs& a
     NQ_REQUIRE(p->E >= 1, "%s: E=%d", who, p->E);
     NQ_REQUIRE(shape_ok(p->H, p->I), "%s: H=%d I=%d must be positive multiples of 128", who, p->H, p->I);
     NQ_REQUIRE((p->which & ~15) == 0, "%s: which=%d", who, p->which);
-    NQ_REQUIRE(!(p->which & 4) || (own_ws && !p->mb_table), "%s: which bit 2 (routing of an earlier call) needs the caller's route_ws / xrot and no mailbox", who);
+    NQ_REQUIRE(!(p->which & 4) || own_ws, "%s: which bit 2 (routing of an earlier call) needs the caller's route_ws / xrot", who);
     NQ_REQUIRE(p->force_level == 0 || p->force_level == 2 || p->force_level == 3 || p->force_level == 4, "%s: force_level=%d", who, p->force_level);
     NQ_REQUIRE(p->x_dtype >= 0 && p->x_dtype <= 2 && p->rw_dtype >= 0 && p->rw_dtype <= 2 && p->sel_dtype >= 0 && p->sel_dtype <= 1 && p->out_dtype >= 0 && p->out_dtype <= 2,
                "%s: dtype codes x=%d sel=%d rw=%d out=%d", who, p->x_dtype, p->sel_dtype, p->rw_dtype, p->out_dtype);

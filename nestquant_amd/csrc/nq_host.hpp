@@ -36,12 +36,11 @@ struct MoeArgs
     int common_rows;                  // 1 = every row that can be picked has base window code 0 and no mask-mode flags; 0 = unknown
     int fuse;                         // both launches belong to this call: for runs whose row has neither a low-rank plane nor the
                                       // 512-wide rotation the down launch's staging does the gate|up finisher (set by launch_moe)
-    int ny_gu;                        // k-slices of the gate|up launch (the down launch's fused staging sums that many partials)
     RouteWs* route;                   // NQ_ROUTE_WS_BYTES of device memory: what the routing launch hands to the projection launches
     _Float16* xrot;                   // [B * topk][2][H] fp16: rotated activations of every active pick (gate, up), B-operand order
-    int mb_apply;                     // this projection launch carries the block that applies the mailbox (set by launch_moe)
+    int mb_apply;                     // this projection launch (the call's last) carries the block that applies the mailbox (set by launch_moe)
     int64_t* mb_table; const int64_t* mb_stage; const int32_t* mb_seq; int32_t* mb_applied; int32_t* mb_applied_host;
-                                      // mailbox of the call (mb_table == nullptr: none): pending rows are honoured by the routing launch, written by the first projection launch
+                                      // mailbox of the call (mb_table == nullptr: none): applied by the last projection launch, published by the next call's routing launch
 };
 
 // kernel launchers defined next to their kernels

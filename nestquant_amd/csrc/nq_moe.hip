@@ -1,14 +1,19 @@
 // Decode-path MoE layer for 1..8 tokens (reference sm120/nqmoe.cu:375-449 route, :493-771 do_item, :858-907 moe_forward,
-// :908-929 mailbox). Two launches on one stream, every routing / level / pointer decision read on the device:
+// :908-929 mailbox). Three launches on one stream, every routing / level / pointer decision read on the device:
 //
+//   nq_prep_k        routing once per call (picks -> runs of distinct experts, their table rows -> run headers in RouteWs) and
+//                 the rotation of the activations of every active pick (x * su -> Hadamard-128 -> fp16, B-operand order).
 //   nq_gemv_k<0, *>  gate|up: grid (strip-pair blocks, k-slices, runs). A run = one distinct routed expert + the tokens that
-//                 picked it. The block rotates those tokens' x (x * su -> Hadamard-128 -> fp16) into LDS, then every
-//                 wavefront decodes the records of two strips chunk by chunk straight into MFMA A operands
-//                 (v_mfma_f32_16x16x32_f16, tokens as the N dimension) and writes its k-slice partial sums. The block
-//                 that arrives last at a (run, 128-column group) counter sums the partials and finishes them:
-//                 Hadamard * sv, SwiGLU, * su_d, Hadamard -> h fp16.
-//   nq_gemv_k<1, *>  down: same kernel on h; the last block of a 128-row output group (counter over all runs) combines:
+//                 picked it. The block copies those tokens' rotated x into LDS, then every wavefront decodes the records of
+//                 two strips chunk by chunk straight into MFMA A operands (v_mfma_f32_16x16x32_f16, tokens as the N
+//                 dimension) and writes its k-slice partial sums. In a call of both launches that is all; in a gate|up-only
+//                 call (and for rows with a low-rank plane or the 512-wide rotation) the block that arrives last at a
+//                 (run, 128-column group) counter finishes the group: Hadamard * sv, SwiGLU, * su_d, Hadamard -> h fp16.
+//   nq_gemv_k<1, *>  down: staging forms h from the gate|up partial sums (or reads it), same decode loop; the last block of a
+//                 128-row output group (counter over all runs) combines:
 //                 out[b] = sum_k rw[b,k] * sv_o (.) Hadamard(sum of partials).
+//   A call with a mailbox: one workgroup of an extra plane of blocks of the call's LAST projection launch applies it
+//   (table <- stage, device applied <- seq); the NEXT routing launch publishes applied to the host. See mailbox_apply.
 //
 // Lane mapping of the GEMV (wave64): lane = 16 * t4 + 8 * ss + g decodes the record of lane (4 g + t4) of unit
 // (strip0 + ss, chunk); it holds 32 weights of row g and 32 of row g + 8, in columns 16 t + 2 t4 + {0,1,8,9}. An MFMA
@@ -138,7 +143,7 @@ struct PickInfo                   // per pick, for the down launch's combine
     const _Float16* signs[64];
     const _Float16* lr[64]; const _Float16* lr4[64]; unsigned char rg[64], rd[64], lv[64];
 };
-struct RouteWs { int nruns; int pad[15]; PickInfo picks; RunHdr run[2][64]; };
+struct RouteWs { int nruns; int ny_gu; int pad[14]; PickInfo picks; RunHdr run[2][64]; };   // ny_gu: k-slices of the gate|up launch that filled part_gu
 static_assert(sizeof(RunHdr) == 128, "RunHdr is read as 32 scalar words");
 static_assert(sizeof(RouteWs) <= NQ_ROUTE_WS_BYTES, "NQ_ROUTE_WS_BYTES in include/nq_moe_hip.h is too small");
 
@@ -153,12 +158,12 @@ __device__ __forceinline__ void ld_sys_row(const int64_t* p, int64_t* f)
 }
 
 // ---- routing dedup: picks -> runs (refined experts first, then by first occurrence); slots in pick order ----------------
-// One wavefront of nq_prep_k, once per call; lane s owns pick s (S <= 64). A run takes at most one pick per token: a token
+// One wavefront per workgroup of nq_prep_k; lane s owns pick s (S <= 64). A run takes at most one pick per token: a token
 // that names the same expert twice opens a second run of that expert, so a run never has more than B tokens. Every lane
-// requests all fields of its own pick's table row together, so the leader's fields cost no second round trip. With a mailbox
-// in the call the lane also reads the expert's seq / applied pair: when they differ, its row is the staged one (read after
-// seq, as the mailbox does), which is what the table holds once the mailbox part of this kernel has written it; nothing
-// writes the table before every routing read is done (see nq_prep_k), so the plain loads of the row cannot be torn.
+// requests all fields of its own pick's table row together, so the leader's fields cost no second round trip. The routing
+// reads the table and nothing else: no kernel writes the table while a routing launch runs (the mailbox of a call is applied
+// by its last projection launch, see mailbox_apply), so every workgroup of the launch sees the same rows and the rows cannot
+// be torn.
 struct PrepRows { int nq; unsigned char tok[64]; const _Float16* signs[64]; };    // LDS: the rows of xrot, one per active pick
 __device__ __forceinline__ void route(const MoeArgs& a, RouteWs* W, int lane, bool writer, PrepRows* Q)
 {
@@ -176,12 +181,6 @@ __device__ __forceinline__ void route(const MoeArgs& a, RouteWs* W, int lane, bo
             const int64_t* ent = a.table + (size_t)e * TBL_W;
 #pragma unroll
             for (int i = 0; i < TBL_W; ++i) f[i] = ent[i];
-            if (a.mb_table)
-            {
-                const int32_t ap = a.mb_applied[e];
-                const int32_t sq = __hip_atomic_load(a.mb_seq + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-                if (sq != ap) ld_sys_row(a.mb_stage + (size_t)e * TBL_W, f);
-            }
             lv = (int)f[0];
             ok = rw_at(a, lane) != 0.f && lv > 0;
         }
@@ -247,23 +246,38 @@ __device__ __forceinline__ void route(const MoeArgs& a, RouteWs* W, int lane, bo
     if (lane == 0) W->nruns = r;
 }
 
-// The mailbox's write half: table[e] <- stage[e] where seq[e] != applied[e], then applied[e] <- seq[e] (device copy and the
-// optional host-mapped mirror), by the threads of one workgroup.
-__device__ __forceinline__ void mailbox_apply(int64_t* table, const int64_t* stage, const int32_t* seq, int32_t* applied, int32_t* applied_host, int E)
+// The mailbox of a layer call (reference nq_mailbox, sm120/nqmoe.cu:908-923, a launch of its own there), in two halves that
+// keep the reference's rule "once applied_host[e] == seq[e] no later kernel can reference the old row's slot":
+//   apply   -- one workgroup of the call's LAST projection launch: for every e with seq[e] != applied[e], table[e] <- stage[e]
+//              and the device copy applied[e] <- seq[e]. This is the call's only reading of seq / stage (a single observer),
+//              it comes after the call's routing launch has ended (the routing of this call used the old rows, identically in
+//              all its workgroups), and neither projection launch reads the table, so a row cannot be torn and no two parts of
+//              the call can disagree about a row. Nothing is published to the host here: this call's launches may still be
+//              decoding from the slot that the old row names.
+//   publish -- the routing launch of the NEXT call (publish_applied): applied_host[e] <- applied[e] for every e. It runs after
+//              every launch of the earlier calls has ended (stream order), and from this routing launch on every launch works
+//              from rows read after the apply, so a slot released by a published row is no longer referenced by anything.
+// A row whose seq lands while call n runs is therefore used from call n + 1 on and published at the head of call n + 1, which is
+// when the reference's mailbox launch at the head of call n + 1 would have applied and published it.
+__device__ __forceinline__ void mailbox_apply(int64_t* table, const int64_t* stage, const int32_t* seq, int32_t* applied, int E)
 {
     for (int e = threadIdx.x; e < E; e += blockDim.x)
     {
         const int32_t ap = applied[e];
         const int32_t sq = __hip_atomic_load(seq + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-        if (sq == ap) continue;
-        int64_t row[TBL_W];
+        if (sq == ap) continue;                                  // the row is requested only after seq has been seen (the copy
+        int64_t row[TBL_W];                                      // stream wrote the row before seq)
         ld_sys_row(stage + (size_t)e * TBL_W, row);
 #pragma unroll
         for (int i = 0; i < TBL_W; ++i) table[(size_t)e * TBL_W + i] = row[i];
-        __threadfence();
-        applied[e] = sq;
-        if (applied_host) __hip_atomic_store(applied_host + e, sq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        applied[e] = sq;                                         // read again only by later launches on this stream
     }
+}
+// host mirror of the device's applied[]: plain re-publication of every entry (values only ever grow, equal values are harmless)
+__device__ __forceinline__ void publish_applied(const int32_t* applied, int32_t* applied_host, int E, int first, int step)
+{
+    for (int e = first; e < E; e += step)
+        __hip_atomic_store(applied_host + e, applied[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
 // First launch of every layer call. Every workgroup repeats the routing (its first wavefront; workgroup 0 writes the result:
@@ -272,13 +286,14 @@ __device__ __forceinline__ void mailbox_apply(int64_t* table, const int64_t* sta
 // wavefronts of the grid share the rotation of the activations: one task per (active pick q, gate or up, 128-column chunk):
 // xrot[q][gate|up][chunk] = fp16(Hadamard-128(x[token] * su)) in the MFMA B-operand column order, which the gate|up launch
 // copies into LDS (before, each of the 32 row blocks of a run repeated these rotations: 9 % of the launch's vector
-// instructions). With a mailbox in the call nothing here writes the table: a pick whose expert has an update pending takes
-// the staged row, and the first projection launch carries the workgroup that applies the mailbox (mailbox_apply).
+// instructions). With a mailbox in the call the other three wavefronts of workgroup 0 first publish what earlier calls applied
+// (publish_applied); nothing here reads seq or stage and nothing writes the table.
 __global__ void __launch_bounds__(256) nq_prep_k(MoeArgs a)
 {
     __shared__ PrepRows Q;
     const int lane = threadIdx.x & 63;
     if (threadIdx.x < 64) route(a, a.route, lane, blockIdx.x == 0, &Q);
+    else if (blockIdx.x == 0 && a.mb_table && a.mb_applied_host) publish_applied(a.mb_applied, a.mb_applied_host, a.E, threadIdx.x - 64, 192);
     __syncthreads();
     // workgroup 0 has the result to write (it ends ~1 us after the others' routing): with more than one workgroup in the grid the
     // rotation tasks go to the others, so that it is not also the last to finish
@@ -499,9 +514,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
     __shared__ int last;
     const int lane = threadIdx.x & 63, warp = threadIdx.x >> 6, SB = blockDim.x >> 6;
     if (a.mb_apply && blockIdx.z == gridDim.z - 1)
-    {   // the extra plane of blocks of a call with a mailbox: one of them applies it (the routing launch has already taken the
-        // staged rows of pending experts, and neither projection launch reads the table)
-        if (blockIdx.x == 0 && blockIdx.y == 0) mailbox_apply(a.mb_table, a.mb_stage, a.mb_seq, a.mb_applied, a.mb_applied_host, a.E);
+    {   // the extra plane of blocks of the last projection launch of a call with a mailbox: one of them applies it
+        if (blockIdx.x == 0 && blockIdx.y == 0) mailbox_apply(a.mb_table, a.mb_stage, a.mb_seq, a.mb_applied, a.E);
         return;
     }
     // the run's header, written by nq_prep_k: block-uniform, read through the scalar cache (constant address space)
@@ -514,6 +528,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
         for (int i = 0; i < (int)(sizeof(RunHdr) / 4); ++i) raw.w[i] = src[i];
     }
     const int nruns = W->nruns;
+    const int ny_gu = W->ny_gu;                                  // MODE 1: how many k-slices the gate|up launch that filled part_gu wrote
     const int N = MODE == 0 ? 2 * a.I : a.H, K = MODE == 0 ? a.H : a.I, C = K / 128;
     if (MODE == 1 && nruns == 0 && blockIdx.z == 0 && blockIdx.y == 0)
     {   // no active pick at all: nobody will arrive last, so the first plane of blocks writes the zero output
@@ -523,6 +538,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
     if ((int)blockIdx.z >= nruns) return;                        // block-uniform
     const RunHdr R = __builtin_bit_cast(RunHdr, raw);
     const int NY = C / NC;
+    if (MODE == 0 && threadIdx.x == 0 && blockIdx.x + blockIdx.y + blockIdx.z == 0) a.route->ny_gu = NY;   // for the down launch's fused staging
     const int ntok = R.ntok, chunk0 = blockIdx.y * NC, k0 = chunk0 * 128;
     const int rowstride = NC * 256 + 16;                         // bytes per staged token (+16: spread tokens over banks)
     char* zero = smem + ntok * rowstride;                        // 256 zero bytes after the token rows
@@ -572,7 +588,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
             const float* const rows2[2] = {p, p + a.I};
             const half2_t svg = *(const half2_t*)(sv_g + col), svu = *(const half2_t*)(sv_u + col), sud = *(const half2_t*)(su_d + col);
             float2 pq[2];
-            sum_partials<2>(rows2, (size_t)Sgu * 2 * a.I, a.ny_gu, pq);
+            sum_partials<2>(rows2, (size_t)Sgu * 2 * a.I, ny_gu, pq);
             float g0 = pq[0].x, g1 = pq[0].y, u0 = pq[1].x, u1 = pq[1].y;
             wht128(g0, g1, lane); wht128(u0, u1, lane);
             g0 *= (float)svg.x; g1 *= (float)svg.y; u0 *= (float)svu.x; u1 *= (float)svu.y;
@@ -649,19 +665,25 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
     if (threadIdx.x == 0) __hip_atomic_store(cnt, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// table[e] <- stage[e] where seq[e] != applied[e]; publish applied (device copy and optional host-mapped mirror)
+// The stand-alone mailbox (reference nq_mailbox, sm120/nqmoe.cu:914-923): table[e] <- stage[e] where seq[e] != applied[e], then
+// applied[e] <- seq[e]; the host mirror gets every entry of applied, changed or not, so that rows applied by the mailbox block
+// of an earlier layer call (which publishes nothing itself) are published here too. Safe to publish at once: this launch
+// follows every earlier launch on the stream, and every later one reads the table after it.
 __global__ void nq_mailbox_k(int64_t* table, const int64_t* stage, const int32_t* seq, int32_t* applied, int32_t* applied_host, int E)
 {
     const int e = blockIdx.x * blockDim.x + threadIdx.x;
     if (e >= E) return;
     const int32_t sq = __hip_atomic_load(seq + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-    if (sq == applied[e]) return;
+    int32_t ap = applied[e];
+    if (sq != ap)
+    {
 #pragma unroll
-    for (int i = 0; i < TBL_W; ++i)
-        table[(size_t)e * TBL_W + i] = __hip_atomic_load(stage + (size_t)e * TBL_W + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-    __threadfence();
-    applied[e] = sq;
-    if (applied_host) __hip_atomic_store(applied_host + e, sq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        for (int i = 0; i < TBL_W; ++i)
+            table[(size_t)e * TBL_W + i] = __hip_atomic_load(stage + (size_t)e * TBL_W + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        __threadfence();
+        applied[e] = ap = sq;
+    }
+    if (applied_host) __hip_atomic_store(applied_host + e, ap, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
 int launch_moe(const MoeArgs& a, const int* cfg_gu, const int* cfg_dn, int which, hipStream_t st)
@@ -676,8 +698,9 @@ int launch_moe(const MoeArgs& a, const int* cfg_gu, const int* cfg_dn, int which
         nq_prep_k<<<std::min((ntask + 3) / 4, 1023) + 1, 256, 0, st>>>(a);       // one workgroup per four rotation tasks, plus the writer
         NQ_LAUNCH_CHECK("moe_forward (routing)");
     }
-    if (a.mb_table && which == 0) return launch_mailbox(a.mb_table, a.mb_stage, a.mb_seq, a.mb_applied, a.mb_applied_host, a.E, st);
-    bool mb_todo = a.mb_table != nullptr;
+    // a call with a mailbox and no projection launch: the apply half as a launch of its own (nothing is published here either)
+    if (a.mb_table && which == 0) return launch_mailbox(a.mb_table, a.mb_stage, a.mb_seq, a.mb_applied, nullptr, a.E, st);
+    const int last_mode = (which & 2) ? 1 : 0;
     for (int mode = 0; mode < 2; ++mode)
     {
         if (!((which >> mode) & 1)) continue;
@@ -689,8 +712,7 @@ int launch_moe(const MoeArgs& a, const int* cfg_gu, const int* cfg_dn, int which
         const bool any = a.common_rows != 1;
         MoeArgs b = a;
         b.fuse = which == 3 || defer;                             // both launches belong to this call (or the caller says the other one follows)
-        b.ny_gu = (a.H / 128) / (cfg_gu[0] * cfg_gu[2]);
-        b.mb_apply = mb_todo; mb_todo = false;                    // the call's first projection launch carries the mailbox block
+        b.mb_apply = a.mb_table != nullptr && mode == last_mode;  // the call's last projection launch carries the mailbox block
         auto kern = mode == 0 ? (any ? nq_gemv_k<0, true> : nq_gemv_k<0, false>) : (any ? nq_gemv_k<1, true> : nq_gemv_k<1, false>);
         if (shm > 48 * 1024)
         {

@@ -227,8 +227,11 @@ class MoELayer:
         bf16, with the roundings of x.half(), rw.half() and out.to(dtype) (the casts the reference's caller launches as
         separate kernels, sm120/serve/nq_vllm.py:522,560).
         table: optional [E, TBL_W] override. Everything is enqueued on torch's current stream; nothing syncs.
-        mailbox: a Mailbox of this layer to apply at the head of the call (same effect as mailbox.apply() right before it,
-        one launch less: the call's routing launch does it before it reads the table).
+        mailbox: a Mailbox of this layer, served by the call without a launch of its own: the call's last projection launch
+        applies it (table rows and the device copy of `applied`) after the call's routing has read the table, and the routing
+        launch of the next call publishes `applied_host`. Rows that land while this call runs are used, and reported done, from
+        the next call on -- when `mailbox.apply()` at the head of the next call would have done both. After the last call of
+        a sequence one `mailbox.apply()` publishes what that call applied.
         static_ws: go through nq_moe_forward_static, which ignores this layer's workspaces and uses the library's built-in
         device scratch instead (for callers that must not allocate; calls on one GPU then share that scratch)."""
         assert x.dtype in _DT_IN and rw.dtype in _DT_IN and sel.dtype in _DT_SEL, (x.dtype, rw.dtype, sel.dtype)
@@ -462,7 +465,7 @@ def forward(layer, mailbox, x, topk_weights, topk_ids, pf_min=PF_MIN, sal=None):
     if 0 < T <= layer.Bmax:
         if sal is not None:
             sal(x, w, ids)
-        return layer(x, ids, w, out=torch.empty(T, layer.H, dtype=odt, device=x.device), mailbox=mailbox)   # applied by the call's first launch
+        return layer(x, ids, w, out=torch.empty(T, layer.H, dtype=odt, device=x.device), mailbox=mailbox)   # applied by the call's last launch, for the next step
     if mailbox is not None:
         mailbox.apply()
     if T == 0:

@@ -31,7 +31,7 @@ def test_every_declared_symbol_is_exported_and_bound():
         assert hasattr(L, n), n
         assert n in _lib.SIGNATURES, f"{n} has no ctypes signature"
     assert sorted(_lib.SIGNATURES) == names
-    assert L.nq_abi_version() == 2
+    assert L.nq_abi_version() == 3
 
 
 def _row(**kw):

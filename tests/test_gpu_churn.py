@@ -26,14 +26,26 @@ def test_slot_layout_and_rows():
     assert lay.spans(2, 4) == [(0, lay.bytes)] and lay.bytes >= 2 * (4718592 + 73728)
 
 
+@pytest.mark.parametrize("in_call", [False, True], ids=["mailbox_launch", "mailbox_in_call"])
 @pytest.mark.parametrize("native", [False, True], ids=["torch_copies", "engine_uploads"])
-def test_churn_racing_graph_replays(native):
+def test_churn_racing_graph_replays(native, in_call):
+    """in_call: the replayed step is L(..., mailbox=MB) instead of MB.apply(); L(...). Every expert has a sign vector of its own
+    per level (as served experts do: the level-2 and level-4 rows name different vectors), so a call whose parts disagreed
+    about a row's level would rotate with the wrong vector and miss the oracle of either state."""
     H, I, NE, NSLOT, B, K = 512, 256, 8, 3, 4, 4
     ex = {e: F.Expert(H, I, seed=70 + e, dev="cpu", nested=True, var=(e == 2)) for e in range(NE)}
     planes = {e: (oracle_plane(x.gu), oracle_plane(x.dn)) for e, x in ex.items()}
-    signs = {e: x.signs.numpy() for e, x in ex.items()}
+    gs = torch.Generator().manual_seed(700)
+    signs = {}
+    for e, x in ex.items():
+        x.sc = {2: x.signs}
+        for lv in (3, 4):
+            x.sc[lv] = (torch.randint(0, 2, x.signs.shape, generator=gs) * 2 - 1).half()
+        for lv in (2, 3, 4):
+            signs[e, lv] = x.sc[lv].numpy()
     for x in ex.values():
         x.gu.to(DEV); x.dn.to(DEV); x.signs = x.signs.to(DEV)
+        x.sc = {lv: (x.signs if lv == 2 else v.to(DEV)) for lv, v in x.sc.items()}
         x.gu.slot = x.gu.nested_plane(); x.dn.slot = x.dn.nested_plane()
     L = M.MoELayer(NE, H, I, Bmax=B, topk=K)
     MB = M.Mailbox(L)
@@ -48,7 +60,7 @@ def test_churn_racing_graph_replays(native):
     xn = x.cpu().numpy()
     dense = {(e, lv): (O.dense_W(planes[e][0], lv, nested=True).astype(np.float32), O.dense_W(planes[e][1], lv, nested=True).astype(np.float32))
              for e in range(NE) for lv in (2, 3, 4)}
-    yel = {k: O.expert_forward(xn, *w, signs[k[0]], dtype=np.float64) for k, w in dense.items()}
+    yel = {k: O.expert_forward(xn, *w, signs[k], dtype=np.float64) for k, w in dense.items()}
 
     def ref(level):
         y = np.zeros((B, H))
@@ -59,7 +71,7 @@ def test_churn_racing_graph_replays(native):
         return y
 
     s = torch.cuda.Stream()
-    step = lambda: (MB.apply(), L(x, sel, rw))
+    step = (lambda: L(x, sel, rw, mailbox=MB)) if in_call else (lambda: (MB.apply(), L(x, sel, rw)))
     with torch.cuda.stream(s):
         for _ in range(2):
             step()

@@ -227,12 +227,14 @@ def test_mailbox_kernel_matches_state_machine():
     assert MB.applied_host.numpy()[[1, 4]].tolist() == [1, 5]
 
 
-def test_mailbox_applied_by_the_layer_call_equals_apply_then_call():
-    """L(..., mailbox=MB) = MB.apply() followed by L(...): same table, same applied / applied_host, same output bits; rows posted
-    between calls (level changes of routed experts, 260 experts so that one thread handles two rows) take effect in that call"""
+def test_mailbox_in_the_layer_call_is_the_call_then_apply():
+    """L(..., mailbox=MB) = L(...) followed by MB.apply(), except that applied_host is published by the NEXT call's first launch:
+    same outputs bit for bit, same table and device `applied` after every call; a row posted before call n changes the result
+    of call n + 1 and is reported done after call n + 1 (260 experts so that one thread of the mailbox block handles two rows)"""
     H, I, NE = 256, 256, 260
     ex = to_dev(experts_on_gpu(H, I, 6, 11, nested_ids=range(6)))
     side = torch.cuda.Stream()
+    ops = [(257, 4), (3, 3), (259, 0), (0, 4), (257, 2), (2, 2)]         # the last op keeps level 2: one more call, nothing changes
     res = []
     for fused in (False, True):
         L = M.MoELayer(NE, H, I, Bmax=2, topk=4)
@@ -242,23 +244,71 @@ def test_mailbox_applied_by_the_layer_call_equals_apply_then_call():
         g = torch.Generator().manual_seed(3)
         x = (torch.randn(2, H, generator=g) * 0.05).half().to(DEV)
         sel = torch.tensor([[0, 257, 2, 3], [3, 4, 259, 0]], device=DEV); rw = torch.full((2, 4), 0.25, device=DEV).half()
-        outs = []
-        for step, (e, lv) in enumerate([(257, 4), (3, 3), (259, 0), (0, 4), (257, 2)]):
+        outs, tabs = [], []
+        for step, (e, lv) in enumerate(ops):
             MB.post(e, M.entry(ex[e % 6], lv), side)
             side.synchronize()
             if fused:
                 y = L(x, sel, rw, mailbox=MB)
             else:
-                MB.apply(); y = L(x, sel, rw)
+                y = L(x, sel, rw); MB.apply()
             torch.cuda.synchronize()
-            assert MB.done(e), (fused, step)
-            outs.append(y.clone())
-        res.append((outs, L.table.clone(), MB.applied.clone(), MB.applied_host.clone()))
-        assert len({o.cpu().numpy().tobytes() for o in outs}) == 5          # every posted row changed the result
+            assert int(MB.applied[e]) == MB.hseq[e] and int(L.table[e, 0]) == lv       # applied on the device by the end of the call
+            assert MB.done(e) == (not fused), (fused, step)                           # ... but published by the next call's head
+            if fused and step:
+                assert MB.done(ops[step - 1][0])
+            outs.append(y.clone()); tabs.append(L.table[:, 0].clone())
+        if fused:
+            MB.apply(); torch.cuda.synchronize()                                      # publishes what the last call applied
+        assert all(MB.done(e) for e in range(NE))
+        res.append((outs, tabs, MB.applied.clone(), MB.applied_host.clone()))
+        assert len({o.cpu().numpy().tobytes() for o in outs}) == len(ops)              # every posted row changed a result
     for a, b in zip(res[0][0], res[1][0]):
         assert torch.equal(a, b)
+    for a, b in zip(res[0][1], res[1][1]):
+        assert torch.equal(a, b)                                                      # levels (the other words are addresses of equal planes)
     assert torch.equal(res[0][2], res[1][2]) and torch.equal(res[0][3], res[1][3])
-    assert torch.equal(res[0][1][:, 0], res[1][1][:, 0])                     # levels (the other words are addresses of equal planes)
+
+
+def test_mailbox_in_call_never_publishes_a_row_the_call_did_not_use():
+    """A sequence number that lands between a call's routing launch and its projection launches (forced from the host with the
+    `which` bits: routing alone, then the demotion is posted and has landed, then both projections with the mailbox and the
+    earlier routing): the call decodes from the slot the old row names, so it may apply the new row but must not report it to
+    the host, which would release the slot under the running launches. The next call publishes it and uses the new row. The
+    expert's level-2 and level-4 rows name different sign vectors, as served experts do."""
+    H, I, NE = 256, 256, 4
+    ex = to_dev(experts_on_gpu(H, I, NE, 23, nested_ids=range(NE)))
+    g = torch.Generator().manual_seed(8)
+    alt = (torch.randint(0, 2, (3 * H + 3 * I,), generator=g) * 2 - 1).half().to(DEV)   # level 4 of expert 1 brings its own signs
+    def row(e, lv):
+        r = M.entry(ex[e], lv)
+        if e == 1 and lv == 4:
+            r[9] = alt.data_ptr()
+        return r
+    L = M.MoELayer(NE, H, I, Bmax=2, topk=2); MB = M.Mailbox(L)
+    ref = M.MoELayer(NE, H, I, Bmax=2, topk=2)
+    for e in range(NE):
+        lv = 4 if e == 1 else 2
+        L.table[e].copy_(row(e, lv)); ref.table[e].copy_(row(e, lv))
+    x = (torch.randn(2, H, generator=g) * 0.05).half().to(DEV)
+    sel = torch.tensor([[1, 2], [0, 1]], device=DEV); rw = torch.tensor([[0.5, 0.25], [0.75, 0.125]], device=DEV).half()
+    want4 = ref(x, sel, rw).clone()
+    ref.table[1].copy_(row(1, 2)); want2 = ref(x, sel, rw).clone()
+    torch.cuda.synchronize()
+    assert not torch.equal(want2, want4)
+    side = torch.cuda.Stream()
+    L(x, sel, rw, which=0)                                       # routing launch only: run headers name expert 1's level-4 row
+    torch.cuda.synchronize()
+    MB.post(1, row(1, 2), side); side.synchronize()              # the demotion lands now
+    y = L(x, sel, rw, which=3 | 4, mailbox=MB).clone()           # projections from the earlier routing, mailbox in this call
+    torch.cuda.synchronize()
+    assert torch.equal(y, want4)                                 # the call used the old row throughout, sign vector included
+    assert int(L.table[1, 0]) == 2 and int(MB.applied[1]) == 1   # applied on the device ...
+    assert int(MB.applied_host[1]) == 0 and not MB.done(1)       # ... and not published: the host must not free the slot yet
+    y = L(x, sel, rw, mailbox=MB).clone()                        # the next call: publishes first, then routes from the new row
+    torch.cuda.synchronize()
+    assert MB.done(1) and torch.equal(y, want2)
+    assert not L.cnt_gu.any() and not L.cnt_d.any()
 
 
 def test_caller_dtypes_and_forward_dispatch():

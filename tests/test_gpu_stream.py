@@ -302,8 +302,10 @@ class Sched:
     def cancelled(s, L, E): s.log.append(("cancelled", L, E))
 
 
-def test_executor_serves_a_layer_through_upgrades_and_downgrades(tmp_path):
-    """shards -> repack -> RankFile + resident planes -> RankExecutor: after every step the served layer equals, bitwise,
+@pytest.mark.parametrize("in_call", [False, True], ids=["mailbox_launch", "mailbox_in_call"])
+def test_executor_serves_a_layer_through_upgrades_and_downgrades(tmp_path, in_call):
+    """in_call: the step is served(..., mailbox=mb) instead of mb.apply(); served(...).
+    shards -> repack -> RankFile + resident planes -> RankExecutor: after every step the served layer equals, bitwise,
     the layer whose rows were set directly to the levels the mailbox has applied; slots are reused only after the
     downgrade was applied; with two slots for three wanted experts the third upgrade waits for a slot"""
     root, out = str(tmp_path / "fit"), str(tmp_path / "out")
@@ -337,8 +339,11 @@ def test_executor_serves_a_layer_through_upgrades_and_downgrades(tmp_path):
 
     def step():
         """one layer call as the serving loop makes it; returns the output and updates `levels` from the callbacks"""
-        mb.apply()
-        y = served(x, sel, rw).clone()
+        if in_call:
+            y = served(x, sel, rw, mailbox=mb).clone()
+        else:
+            mb.apply()
+            y = served(x, sel, rw).clone()
         torch.cuda.synchronize()
         n = len(sched.log)
         ex.poll(sched)
@@ -412,8 +417,10 @@ def test_executor_serves_a_layer_through_upgrades_and_downgrades(tmp_path):
         ex.close()
 
 
-def test_scheduler_executor_and_layer_in_one_serving_loop(tmp_path):
-    """the reference's serving step (sm120/serve/nq_vllm.py:546-574 with streaming/smoke_sched.py's loop): mailbox, layer
+@pytest.mark.parametrize("in_call", [False, True], ids=["mailbox_launch", "mailbox_in_call"])
+def test_scheduler_executor_and_layer_in_one_serving_loop(tmp_path, in_call):
+    """in_call: the step is served(..., mailbox=mb) instead of mb.apply(); served(...).
+    the reference's serving step (sm120/serve/nq_vllm.py:546-574 with streaming/smoke_sched.py's loop): mailbox, layer
     call with the hits export, counts -> Scheduler.step -> RankExecutor.apply, poll after the call. Routing favours two
     experts at a time and then moves on; whenever nothing is in flight the table's levels are the scheduler's, and the layer
     equals, bitwise, a layer set directly to those levels"""
@@ -443,9 +450,12 @@ def test_scheduler_executor_and_layer_in_one_serving_loop(tmp_path):
         for t in range(240):
             pair = [(0, 1), (3, 4), (6, 7), (4, 0)][(t // 60) % 4]
             sel = torch.tensor([pair], device=DEV)
-            mb.apply()
             prev = hits.clone()
-            y = served(x, sel, rw).clone()
+            if in_call:
+                y = served(x, sel, rw, mailbox=mb).clone()
+            else:
+                mb.apply()
+                y = served(x, sel, rw).clone()
             torch.cuda.synchronize()
             ex.poll(S)
             counts = (hits - prev).numpy().astype(np.float64)[None]
