@@ -8,7 +8,8 @@ of the last call. Steps are hipGraph replays (one captured graph per routing), t
 and all 4.85 GB of planes resident. Prints ONE JSON line:
   value     = code bytes of the distinct routed experts at their levels / time   (GB/s; the reference's nq_GBs)
   roofline  = the gate|up decode-GEMV kernel alone, timed live with events over K launches, against 8 TB/s HBM
-  cpu_baseline = the C oracle (dense decode + fp32 matvecs, OpenMP on all host cores) on whole layer steps, about 10 s of CPU work
+  cpu_baseline = the reference's torch-CPU path restated (dense decode + fp32 matmuls on all host cores) on whole layer steps,
+                 with the C oracle (OpenMP) timed beside it; about 10-20 s of CPU work together
 """
 import argparse
 import json

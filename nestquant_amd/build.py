@@ -12,7 +12,6 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libnq_moe_hip.so")
 NATIVE = os.path.join(HERE, "nq_bench_native")
-PROBE = os.path.join(HERE, "nq_issue_probe")
 OBJ = os.path.join(HERE, "build")
 ARCH = "gfx950"
 FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-ffp-contract=off",
@@ -47,12 +46,13 @@ def build(verbose=False, jobs=None):
     with ThreadPoolExecutor(max_workers=jobs or min(8, len(srcs))) as ex:
         list(ex.map(one, range(len(srcs))))
     _run([hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", LIB] + objs)
-    # torch-free driver of the C ABI (timing cross-check and the program rocprofv3 counter passes wrap)
-    _run([hipcc, "-O2", "-std=c++17", f"--offload-arch={ARCH}", "-x", "hip", os.path.join(CSRC, "nq_bench_native.cpp"),
-          "-o", NATIVE, "-L" + HERE, "-lnq_moe_hip", "-Wl,-rpath,$ORIGIN", "-Wno-unused-command-line-argument", "-Wno-unused-result"])
-    # stand-alone probe of the vector-instruction issue rates the decoder's design rests on (no library, no inputs)
-    _run([hipcc, "-O3", "-std=c++17", f"--offload-arch={ARCH}", "-x", "hip", os.path.join(CSRC, "nq_issue_probe.cpp"),
-          "-o", PROBE, "-Wno-unused-command-line-argument"])
+    # torch-free driver of the C ABI (timing cross-check and the program rocprofv3 counter passes wrap): a measurement aid,
+    # so a failure to build it is reported and does not fail the library's build
+    try:
+        _run([hipcc, "-O2", "-std=c++17", f"--offload-arch={ARCH}", "-x", "hip", os.path.join(CSRC, "nq_bench_native.cpp"),
+              "-o", NATIVE, "-L" + HERE, "-lnq_moe_hip", "-Wl,-rpath,$ORIGIN", "-Wno-unused-command-line-argument", "-Wno-unused-result"])
+    except RuntimeError as e:
+        print(f"warning: nq_bench_native was not built: {e}", file=sys.stderr)
     return LIB
 
 

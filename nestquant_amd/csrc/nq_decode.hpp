@@ -8,12 +8,12 @@
 //   level 2  w = fp16(A * (1024 + S_b) + B)                                      A = 0x1eee, B = 0xc931
 //   level 3/4 F = (Mb S_b + N S_r + 128) >> 8 ; w = fp16(A' * (1024 + F) + C)   block word Mb | N << 8 per unit
 //
-// gfx950 instruction choices:
-//   * the hash multiply is split into two full-rate 16-bit multiplies (v_mad_u32_u16 + v_pk_mad_u16 with op_sel), which
-//     read only a 16-bit half of their source, so a window needs no masking and every second window (offset + 16) is
-//     the high half of a register that was already produced for its partner: half a v_alignbit per weight;
+// gfx950 instruction choices (every opcode of the chain issues at the same measured rate, so their count is what matters):
+//   * one v_alignbit_b32 yields the register that holds two windows 16 bits apart; v_and / v_lshrrev (or one v_bfe_u32 where
+//     the window lies inside a word) cuts the 16-bit state; the hash is ONE v_mul_lo_u32 by 0x83DCD12D;
 //   * v_sad_u8 / v_sad_hi_u8 give the byte sums of two weights already packed as the fp16 pair (1024 + S);
-//   * v_dot4_u32_u8 folds Mb * S_b + N * S_r with the rounding constant in its accumulator; v_perm_b32 packs a pair.
+//   * v_dot4_u32_u8 folds Mb * S_b + N * S_r with the rounding constant in its accumulator; v_perm_b32 packs a pair;
+//   * v_pk_fma_f16 is the single-rounded fp16 FMA of the value map.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>

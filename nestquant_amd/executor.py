@@ -142,7 +142,7 @@ class RankExecutor:
         s.rows = Rows(layers, s.lay, s.pool.base or 256)
         s.by_key = {}                                             # (L, E) -> its one outstanding Op
         s.by_tag = {}                                             # engine tag -> Op, for ops in state ISSUED
-        s.queue = collections.deque()                             # keys of QUEUED upgrades, in arrival order
+        s.queue = []                             # keys of QUEUED upgrades, in arrival order
         s.count = collections.Counter()
         s.next_tag = 0
         s.lat = []                                                # end-to-end seconds of every landed upgrade
@@ -150,12 +150,13 @@ class RankExecutor:
         s.marks = {}                                              # io_stats(): caller name -> counters at its previous call
         s.tier_n = s.eng.tier_load([rf.rec(L, E) for L, E in tier]) if tier else 0
 
-    # ---- the reference's attribute surface, derived from the op objects
+    # ---- the reference's attribute surface, derived from the op objects: `ops`, `wait_apply` and `up_tag` are read-only views
+    # built on every access (changing the returned dict changes nothing); `pend` is the live queue
     slots = property(lambda s: s.pool.mem)
     slot0 = property(lambda s: s.pool.base)
     free = property(lambda s: s.pool.free)
     slot_of = property(lambda s: s.pool.owner)
-    pend = property(lambda s: list(s.queue))
+    pend = property(lambda s: s.queue)       # the live queue of upgrades waiting for a slot (callers may remove from it, as the reference's do)
     ops = property(lambda s: {t: (*o.key, o.level, o.seq) for t, o in s.by_tag.items()})
     wait_apply = property(lambda s: {o.key: (o.level, o.seq) for o in s.by_key.values() if o.state is State.WRITTEN})
     up_tag = property(lambda s: {o.key: t for t, o in s.by_tag.items() if o.level == 4})
@@ -231,7 +232,9 @@ class RankExecutor:
             if op.level == 2:
                 # the level-4 row is still live and points into the slot: keep slot and books, post the row again
                 if op.reposts >= REPOST_LIMIT:
-                    raise RuntimeError(f"the engine failed to post the level-2 row of layer {L} expert {E} {op.reposts + 1} times")
+                    # raised by poll() once the whole batch of reports has been handled, so that no other report of the batch is
+                    # lost; the op stays in by_key (the level-4 row is live and owns its slot: the expert takes no further op)
+                    return f"the engine failed to post the level-2 row of layer {L} expert {E} {op.reposts + 1} times"
                 op.reposts += 1
                 s.count["reposted"] += 1
                 s._to_engine(op)
@@ -262,15 +265,20 @@ class RankExecutor:
             s._tell(sched, "released", L, E)
 
     def poll(s, sched=None, issue=True):
+        fatal = []
         for tag, _hit, t_read, t_e2e in s.eng.poll():
-            s._engine_report(s.by_tag.pop(tag), t_read, t_e2e, sched)
+            why = s._engine_report(s.by_tag.pop(tag), t_read, t_e2e, sched)
+            if why:
+                fatal.append(why)
         for op in [o for o in s.by_key.values() if o.state is State.WRITTEN]:
             if s.port[op.key[0]].applied[op.key[1]] == op.seq:
                 s._mailbox_applied(op, sched)
         while issue and s.queue and s.pool.free:
-            op = s.by_key[s.queue.popleft()]
+            op = s.by_key[s.queue.pop(0)]
             s.pool.take(op.key)
             s._to_engine(op)
+        if fatal:
+            raise RuntimeError("; ".join(fatal))
 
     def cancel_up(s, L, E, sched=None):
         """drop an upgrade of (L, E) that has not started: still waiting for a slot here -> dropped now (True, and

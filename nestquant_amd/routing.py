@@ -9,29 +9,30 @@ import torch
 
 
 def make_sel(B, pool, mode="recency", p=0.4, rng=None, avoid=(), topk=8):
+    """B rows of topk distinct expert ids drawn from `pool` minus `avoid`. 'recency': a token keeps each id of the token before it
+    with probability p and fills up with fresh ones; 'distinct': no id serves two tokens; anything else: rows independent."""
     rng = rng or random.Random(0)
-    avoid = set(avoid)
-    pool = [e for e in pool if e not in avoid]
-    rows, used = [], set()
+    banned = set(avoid)
+    allowed = [e for e in pool if e not in banned]
+    rows, taken = [], set()
     for t in range(B):
-        row = []
-        if t and mode == "recency":
-            row = [e for e in rows[-1] if rng.random() < p]
-        cand = [e for e in pool if e not in row and (mode != "distinct" or e not in used)]
-        rng.shuffle(cand)
-        row += cand[: topk - len(row)]
+        kept = [e for e in rows[t - 1] if rng.random() < p] if (t > 0 and mode == "recency") else []
+        blocked = set(kept) | (taken if mode == "distinct" else set())
+        fresh = [e for e in allowed if e not in blocked]
+        rng.shuffle(fresh)
+        row = kept + fresh[: topk - len(kept)]
         rng.shuffle(row)
+        taken.update(row)
         rows.append(row)
-        used |= set(row)
     return rows
 
 
 def routing_tensors(rows, device="cuda", seed=0):
-    g = torch.Generator().manual_seed(seed)
-    sel = torch.tensor(rows, dtype=torch.long)
-    w = torch.rand(sel.shape, generator=g) + 0.1
-    w = w / w.sum(1, keepdim=True)
-    return sel.to(device), w.half().to(device)
+    """(sel int64 [B, topk], rw fp16 [B, topk]) for id rows: weights uniform in [0.1, 1.1), normalised per token"""
+    sel = torch.as_tensor(rows, dtype=torch.int64)
+    raw = 0.1 + torch.rand(sel.shape, generator=torch.Generator().manual_seed(seed))
+    rw = raw / raw.sum(dim=1, keepdim=True)
+    return sel.to(device), rw.to(torch.float16).to(device)
 
 
 def routings(B, NP, R, mode="recency", seed=0, device="cuda", topk=8):

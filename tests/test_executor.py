@@ -152,6 +152,28 @@ def test_a_failed_downgrade_keeps_its_slot_and_is_posted_again():
     assert ex.slot_of == {(L, 1): 0}
 
 
+def test_a_fatal_report_does_not_lose_the_rest_of_its_batch():
+    """the report that exhausts a downgrade's reposts and the completion of another expert's upgrade arrive in one poll(): the
+    error is raised after the whole batch has been handled, so the upgrade is in the books and lands"""
+    import pytest
+    from nestquant_amd import executor as EX
+    ex, eng, mb, exs, lay = make(nslot=2)
+    log = Log()
+    ex.apply([(L, 1)], [], log)
+    eng.finish(1); ex.poll(log); mb.applied_host[1] = 1; ex.poll(log)
+    ex.apply([], [(L, 1)], log)
+    tag = 2
+    for _ in range(EX.REPOST_LIMIT):                                     # every repost fails too
+        eng.finish(tag, trd=-5.0); ex.poll(log); tag += 1
+    ex.apply([(L, 5)], [], log)                                          # tag + 1: an upgrade of another expert
+    eng.finish(tag, trd=-5.0); eng.finish(tag + 1)                       # both reports in the next poll
+    with pytest.raises(RuntimeError, match="failed to post"):
+        ex.poll(log)
+    assert ex.wait_apply == {(L, 5): (4, 1)} and ex.n_landed == 1 + 1    # the upgrade's report was handled
+    mb.applied_host[5] = 1; ex.poll(log)
+    assert log.ev[-1] == ("landed", 5) and ex.slot_of[L, 1] == 0 and (L, 5) in ex.slot_of
+
+
 def test_shadow_posts_level_2_rows_and_io_stats_reports_intervals():
     ex, eng, mb, exs, lay = make(shadow=True)
     ex.apply([(L, 1)], [])

@@ -55,6 +55,29 @@ def test_static_scratch_entry_equals_caller_workspace_entry():
         gb = L(x, sel, rw, out=torch.empty(B, H, dtype=torch.bfloat16, device=DEV), static_ws=True)
         assert torch.equal(gb, wb)
     assert alloc == [0, 0, 0, 0]
+    # torch's counter sees only torch's allocator; the driver's own count of free device memory (hipMemGetInfo) would show a
+    # hipMalloc / hipFree inside the library, and a call recorded into a graph cannot allocate at all (it would fail the capture)
+    out = torch.empty(B, H, dtype=torch.float32, device=DEV)
+    want = L(x, sel, rw).clone()
+    torch.cuda.synchronize()
+    free0 = torch.cuda.mem_get_info()[0]
+    for _ in range(8):
+        L(x, sel, rw, out=out, static_ws=True)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0
+    st = torch.cuda.Stream()
+    gr = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(st):
+        L(x, sel, rw, out=out, static_ws=True)
+    torch.cuda.synchronize()
+    with torch.cuda.graph(gr, stream=st):
+        L(x, sel, rw, out=out, static_ws=True)
+    for _ in range(3):                                         # every replay against the eager result, eager work between them
+        out.fill_(float("nan"))
+        gr.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want)
+        assert torch.equal(L(x, sel, rw).clone(), want)
     del ex
     assert int(L.cnt_gu.abs().sum()) == 0 and int(L.cnt_d.abs().sum()) == 0
 
