@@ -433,11 +433,11 @@ def churn_leg(L, MB, ex, levels, routes, xs, dev, steps=64, ops_per_step=8, nati
     graphs = []
     for i in range(len(routes)):
         with torch.cuda.stream(s):
-            MB.apply(); L(xs[i], routes[i][0], routes[i][1])
+            L(xs[i], routes[i][0], routes[i][1], mailbox=MB)     # the step as the headline runs it: the mailbox inside the call
         torch.cuda.synchronize()
         gr = torch.cuda.CUDAGraph()
         with torch.cuda.graph(gr, stream=s):
-            MB.apply(); L(xs[i], routes[i][0], routes[i][1])
+            L(xs[i], routes[i][0], routes[i][1], mailbox=MB)
         graphs.append(gr)
 
     def run(churn):
@@ -779,18 +779,34 @@ def main():
     # graph replays must reproduce the eager results (outputs are bitwise repeatable)
     assert torch.equal(eager, outs), "graph replay differs from eager execution"
 
-    for _ in range(W // R):
-        g_full.replay()
-    if g_warm is not None:
-        g_warm.replay()
+    def run_steps(n, g_part):
+        for _ in range(n // R):
+            g_full.replay()
+        if g_part is not None:
+            g_part.replay()
+
+    # (1) wall clock: W untimed steps, synchronize, exactly K steps, synchronize. With few steps this also times the host's
+    # launch of one graph and the wake-up after the synchronize (~0.1 ms together), which are not part of a layer step.
+    with torch.cuda.stream(s):
+        run_steps(W, g_warm)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(K // R):
-        g_full.replay()
-    if g_rem is not None:
-        g_rem.replay()
+    with torch.cuda.stream(s):
+        run_steps(K, g_rem)
     torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
+    dt_wall = time.perf_counter() - t0
+    # (2) the same K steps between two HIP events recorded on the launch stream, with the W warm-up steps enqueued directly in
+    # front of them, so that the device is still busy when the timed graph arrives and the events bracket device time only.
+    # `value` is taken from this one; the wall-clock figure stays on the line beside it.
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(s):
+        run_steps(max(W, 1), g_warm if W else capture(1))
+        e0.record(s)
+        run_steps(K, g_rem)
+        e1.record(s)
+    torch.cuda.synchronize()
+    dt = e0.elapsed_time(e1) / 1e3
     nbytes = sum(code_bytes(ex, levels, routes[i % R][2]) for i in range(K))
     gbs = nbytes / dt / 1e9
     # spread of the same measurement with the reference's method (sm120/timing.py:2-29): the graphs under comparison are replayed
@@ -890,6 +906,10 @@ def main():
         "metric": "MoE layer us + HBM GB/s (decode bs1 top-8); prefill grouped-GEMM TFLOP/s",
         "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": round(dt / K * 1e3, 5), "us_per_layer": round(dt / K * 1e6, 2),
+        "timed": "exactly K layer steps (hipGraph replays) between two HIP events on the launch stream, W warm-up steps enqueued "
+                 "directly before them, torch.cuda.synchronize() on both sides; *_wall = the same K steps by the host's clock "
+                 "between two synchronizes (includes one graph launch and the wake-up after the synchronize)",
+        "ms_per_step_wall": round(dt_wall / K * 1e3, 5), "value_wall": round(nbytes / dt_wall / 1e9, 1),
         "us_per_layer_median": round(blocks[len(blocks) // 2], 2), "us_per_layer_min": round(blocks[0], 2),
         "us_layer_call_without_mailbox_median": round(call_blocks[len(call_blocks) // 2], 2), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",

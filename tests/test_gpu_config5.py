@@ -1,0 +1,122 @@
+"""Config 5 at its full size: the config-3 layer (H 6144, I 2048, 256 experts, top-8, one token) over 64 seeded steps, each
+step issuing 8 promotions (2 -> 4) / demotions (4 -> 2) through the upgrade engine's uploads from pinned host memory, racing
+graph replays of the layer step. The host synchronises only after every 8th step; there the step's output must equal the
+float64 oracle of the level state that step applied, the experts swapped since the last check must dequantise bit for bit to
+the C oracle's decode at their new level, and at the end the slot / table invariants (B)(T)(O)(K) must hold. Freed slots are
+reused by the next promotions while replays run, and every expert brings a sign vector of its own for level 4, so a call
+that mixed two states of a row, or a slot released too early, shows in the output. Stops at the first failure.
+(reference sm120/levelswitch_mbox.py:33-65, sm120/serve/nq_slotcheck.py:11-21)"""
+import random
+
+import numpy as np
+import pytest
+import torch
+
+from nestquant_amd import churn as CH, moe as M
+from oracle import nq_oracle as O
+from tests.util import rel_err, same_f16
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+STEPS, OPS_PER_STEP, SYNC_EVERY = 64, 8, 8
+
+
+@pytest.mark.parametrize("in_call", [True, False], ids=["mailbox_in_call", "mailbox_launch"])
+def test_config5_full_size_churn(in_call):
+    import bench as BN
+    H, I, E = BN.H, BN.I, BN.E
+    L, MB, ex, levels = BN.build_layer(DEV, Bmax=1)
+    g = torch.Generator().manual_seed(55)
+    for e in range(E):                                            # level 4 rotates and scales with a vector of its own
+        ex[e].sc = {2: ex[e].signs, 3: ex[e].signs, 4: (torch.randint(0, 2, ex[e].signs.shape, generator=g) * 2 - 1).half().to(DEV)}
+    hi = [e for e in range(E) if levels[e] >= 3]
+    X = CH.ChurnExecutor(L, MB, {e: ex[e] for e in range(E)}, nslots=len(hi) + 4 * OPS_PER_STEP, native=True)
+    try:
+        for e in range(E):
+            L.table[e].copy_(X.row(e, 2))
+
+        def settle():
+            for _ in range(4000):
+                MB.apply(); torch.cuda.synchronize()
+                X.poll()
+                if not X.pend:
+                    return
+                torch.cuda._sleep(100000)
+            raise AssertionError("ops did not land")
+
+        for e in hi:                                              # the config-3 pool: its level-3 and level-4 experts at level 4
+            assert X.promote(e, 4)
+        settle()
+        routes = BN.make_routings(1, STEPS, DEV)
+        xs = [(torch.randn(1, H, generator=g) * 0.05).half().to(DEV) for _ in range(STEPS)]
+        outs = torch.zeros(STEPS, 1, H, dtype=torch.float32, device=DEV)
+        s = torch.cuda.Stream()
+
+        def step(i):
+            if in_call:
+                L(xs[i], routes[i][0], routes[i][1], out=outs[i], mailbox=MB)
+            else:
+                MB.apply(); L(xs[i], routes[i][0], routes[i][1], out=outs[i])
+
+        graphs = []
+        for i in range(STEPS):
+            with torch.cuda.stream(s):
+                step(i)
+            torch.cuda.synchronize()
+            gr = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gr, stream=s):
+                step(i)
+            graphs.append(gr)
+        settle()
+
+        def oracle_out(i, level):
+            ids, w = routes[i][0].cpu().numpy(), routes[i][1].cpu().numpy()
+            dense = lambda e: tuple(M.dequant(X.row(e, level[e], X.slot_of.get(e)).to(DEV), p, H, I).float().cpu().numpy() for p in (0, 1))
+            return O.moe_forward(dense, [level[e] for e in range(E)], lambda e: ex[e].sc[level[e]].cpu().numpy(), xs[i].cpu().numpy(), ids, w,
+                                 dtype=np.float64)
+
+        rng = random.Random(5)
+        swapped, nops, nchecked_swaps, worst, moved = set(), 0, 0, 0.0, 0
+        for st in range(STEPS):
+            n = 0
+            cand = list(range(E)); rng.shuffle(cand)
+            for e in cand:                                        # the scheduler: 8 ops per step, no host synchronisation
+                if n == OPS_PER_STEP:
+                    break
+                if not X.idle(e):
+                    continue
+                if X.promote(e, 4) if X.level[e] == 2 else X.demote(e, 2):
+                    n += 1
+            nops += n
+            with torch.cuda.stream(s):
+                graphs[st].replay()
+            swapped |= set(X.poll())                              # reads applied_host as it is: may free slots under the replays
+            if st % SYNC_EVERY != SYNC_EVERY - 1:
+                continue
+            torch.cuda.synchronize()
+            swapped |= set(X.poll())
+            # the step that just ended applied exactly the published state: X.level after this poll. The rows of experts in
+            # transit may be ahead of it in the table (an applied, not yet published op), never what the step used.
+            y = outs[st, 0].cpu().numpy()
+            routed = set(routes[st][2])
+            moved += len(routed & swapped)
+            err = rel_err(y, oracle_out(st, X.level)[0])
+            worst = max(worst, err)
+            assert err < 1e-4, (st, err)                         # a stale or mixed state is off by percents; the reference holds ~1e-4 (sm120/results/check_I512.txt)
+            for e in sorted(swapped)[:6]:                         # bit-exact dequant after the swap, at the level the books say
+                if e in X.pend:
+                    continue
+                for proj in (0, 1):
+                    Wd = M.dequant(L.table[e].clone(), proj, H, I).cpu().numpy()
+                    assert same_f16(Wd, BN.c_oracle_dense(ex, e, X.level[e], proj)) == 0, (st, e, X.level[e], proj)
+                nchecked_swaps += 1
+            swapped.clear()
+        torch.cuda.synchronize()
+        settle()
+        X.check_invariants()
+        assert nops >= STEPS * OPS_PER_STEP // 2 and nchecked_swaps >= 16, (nops, nchecked_swaps)
+        print(f"config 5 full size ({'in-call' if in_call else 'launched'} mailbox): {nops} ops, {X.n_refused} refused, "
+              f"{nchecked_swaps} swapped experts dequantised bit-exactly, worst rel err of the synced steps {worst:.2e}, "
+              f"{moved} routed experts had changed level at a check")
+    finally:
+        X.close()

@@ -22,7 +22,7 @@ from tests.util import rel_err
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
-DECODE_LAYERS, PREFILL_LAYERS = 30, 12        # random layers per seed: 4 decode cases / 3 prefill cases on each
+DECODE_LAYERS, PREFILL_LAYERS = 400, 200        # random layers per seed: 4 decode cases / 3 prefill cases on each
 
 
 def _random_layer(rng, g, Bmax=8):
