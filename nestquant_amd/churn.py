@@ -107,7 +107,7 @@ class ChurnExecutor:
             r[2], r[6] = b + p["gu.p3"][0], b + p["dn.p3"][0]
             d = "d3" if level == 3 else "d4"
             r[3], r[7] = b + p["gu." + d][0], b + p["dn." + d][0]
-            r[10] = r[11] = CODE_L3 if level == 3 else CODE_L4N
+            r[10] = r[11] = CODE_L3 if level == 3 else int(getattr(s.ex[e], "l4code", CODE_L4N))
         return r
 
     def idle(s, e):

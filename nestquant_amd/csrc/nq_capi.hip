@@ -24,7 +24,7 @@ extern "C" const char* nq_last_error(void) { return error_buffer(); }
 extern "C" int nq_codes(uint32_t out[4])
 {
     NQ_REQUIRE(out, "nq_codes: null output");
-    out[0] = out[1] = (1u << NCODES) - 1u;   // residual codes 0..11 in both kernels
+    out[0] = out[1] = (1u << NCODES) - 1u;   // residual codes 0..12 in both kernels
     out[2] = out[3] = 3u;                     // base codes 0 (K = 2 ring base) and 1 (K = 1.75, sub-array layout)
     return 0;
 }

@@ -25,8 +25,9 @@ constexpr int TBL_W = 20;                       // int64 words per table row (re
 constexpr uint32_t HASH_MUL = 0x83DCD12Du;      // state -> 32-bit hash (reference sm120/moe.py:115, sm120/nqmoe.cu:79)
 constexpr uint32_t MUL1_A2 = 0x1eee1eeeu;       // fp16 A twice
 constexpr uint32_t MUL1_B2 = 0xc931c931u;       // fp16 B twice
-constexpr int CODE_L3 = 10, CODE_L4N = 11;      // nested planes of this build: K=1 plane; P3 record || P4 record
-constexpr int NCODES = 12;
+constexpr int CODE_L3 = 10, CODE_L4N = 11, CODE_L4B = 12;   // nested planes of this build: K=1 plane P3; P3 record || P4 record;
+                                                            // P3 and P4 records interleaved bit by bit
+constexpr int NCODES = 13;
 
 // plane pointers come out of int64 table words; naming the global address space keeps their loads off the flat path
 // (flat loads also tick the LDS counter, so a prefetch in flight would stall every LDS read behind it)
@@ -59,6 +60,8 @@ template <> struct Pat<8>  { static constexpr int KA = 1, M = 0xFEFE; static con
 template <> struct Pat<9>  { static constexpr int KA = 2, M = 0xD5AA; static constexpr bool SPLIT = false; };
 template <> struct Pat<10> { static constexpr int KA = 1, M = 0x0000; static constexpr bool SPLIT = false; };
 template <> struct Pat<11> { static constexpr int KA = 2, M = 0x0000; static constexpr bool SPLIT = true; };
+template <> struct Pat<12> { static constexpr int KA = 2, M = 0x0000; static constexpr bool SPLIT = true; };
+template <int CODE> constexpr bool interleaved_planes = CODE == CODE_L4B;
 
 __host__ __device__ constexpr int popc16(int m) { int c = 0; for (int i = 0; i < 16; ++i) c += (m >> i) & 1; return c; }
 __host__ __device__ constexpr int step_off(int j, int KA, int M)
@@ -76,8 +79,8 @@ template <int CODE> struct Rec
 };
 __host__ inline int rec_bits(int code)
 {
-    constexpr int ka[NCODES] = {2, 1, 2, 2, 3, 1, 1, 2, 1, 2, 1, 2};
-    constexpr int mk[NCODES] = {0, 0xEEEE, 0xAAAA, 0x8888, 0, 0xAAAA, 0xFFFE, 0x9248, 0xFEFE, 0xD5AA, 0, 0};
+    constexpr int ka[NCODES] = {2, 1, 2, 2, 3, 1, 1, 2, 1, 2, 1, 2, 2};
+    constexpr int mk[NCODES] = {0, 0xEEEE, 0xAAAA, 0x8888, 0, 0xAAAA, 0xFFFE, 0x9248, 0xFEFE, 0xD5AA, 0, 0, 0};
     return 4 * (16 * ka[code] + popc16(mk[code]));
 }
 
@@ -106,15 +109,45 @@ constexpr SubArrays sub_arrays(int bits)
 template <int... Is, class F> __device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, Is...>) { (f(CodeTag<Is>{}), ...); }
 template <int N, class F> __device__ __forceinline__ void static_for(F&& f) { static_for_impl(f, std::make_integer_sequence<int, N>{}); }
 
-// the record `rec` of a plane at p, as 32-bit words w[0 .. NW). Code 11 stores its 128-bit record as the 64-bit records of
-// plane P3 followed by those of plane P4.
+// 32 bits of the interleaved stream: bit 2 i = bit i of the 16-bit piece of plane P3, bit 2 i + 1 = bit i of the piece of P4.
+// z holds, from its low byte up, (P3 byte, P4 byte, next P3 byte, next P4 byte); each 16-bit half is shuffled by swapping its
+// middle nibbles, then the middle bit pairs of every byte, then the middle bits of every nibble (a perfect shuffle in three
+// stages of five instructions: shift, and, the same again the other way, or).
+__device__ __forceinline__ uint32_t shuffle_halves(uint32_t z)
+{
+    z = (z & 0xF00FF00Fu) | ((z & 0x00F000F0u) << 4) | ((z >> 4) & 0x00F000F0u);
+    z = (z & 0xC3C3C3C3u) | ((z & 0x0C0C0C0Cu) << 2) | ((z >> 2) & 0x0C0C0C0Cu);
+    z = (z & 0x99999999u) | ((z & 0x22222222u) << 1) | ((z >> 1) & 0x22222222u);
+    return z;
+}
+
+// What is left to do on a loaded record before its windows are cut, kept apart from load_record so that a record requested one
+// chunk ahead is not waited for at the point of the request. Code 12: w = (P3 lo, P3 hi, P4 lo, P4 hi) -> the interleaved
+// 128 bits. Every other code: nothing.
+template <int CODE>
+__device__ __forceinline__ void prepare_record(uint32_t* w)
+{
+    if constexpr (interleaved_planes<CODE>)
+    {
+        const uint32_t a0 = w[0], a1 = w[1], b0 = w[2], b1 = w[3];
+        w[0] = shuffle_halves(__builtin_amdgcn_perm(b0, a0, 0x05010400u));
+        w[1] = shuffle_halves(__builtin_amdgcn_perm(b0, a0, 0x07030602u));
+        w[2] = shuffle_halves(__builtin_amdgcn_perm(b1, a1, 0x05010400u));
+        w[3] = shuffle_halves(__builtin_amdgcn_perm(b1, a1, 0x07030602u));
+    }
+}
+
+// the record `rec` of a plane at p, as 32-bit words w[0 .. NW). Codes 11 and 12 take the 64-bit record of plane P3 and, nrec
+// records further on, the 64-bit record of plane P4: code 11's 128-bit record is the first followed by the second, code 12's
+// is the two interleaved bit by bit (stream bit 2 i = bit i of P3's record, bit 2 i + 1 = bit i of P4's), so that every
+// 16-bit window holds eight bits of each plane.
 template <int CODE>
 __device__ __forceinline__ void load_record(uint32_t* w, gp_u8 p, size_t rec, size_t nrec)
 {
     if constexpr (Pat<CODE>::SPLIT)
     {
         const u32x2 lo = ((gp_u2)p)[rec], hi = ((gp_u2)(p + nrec * 8))[rec];
-        w[0] = lo.x; w[1] = lo.y; w[2] = hi.x; w[3] = hi.y;
+        w[0] = lo.x; w[1] = lo.y; w[2] = hi.x; w[3] = hi.y;   // code 12: interleaved by prepare_record() where the record is used
     }
     else
     {
@@ -336,7 +369,8 @@ __device__ __forceinline__ void dispatch_code(int code, F&& f)
         case 1: f(CodeTag<1>{}); break;   case 2: f(CodeTag<2>{}); break;   case 3: f(CodeTag<3>{}); break;
         case 4: f(CodeTag<4>{}); break;   case 5: f(CodeTag<5>{}); break;   case 6: f(CodeTag<6>{}); break;
         case 7: f(CodeTag<7>{}); break;   case 8: f(CodeTag<8>{}); break;   case 9: f(CodeTag<9>{}); break;
-        case 10: f(CodeTag<10>{}); break; case 11: f(CodeTag<11>{}); break; default: f(CodeTag<0>{}); break;
+        case 10: f(CodeTag<10>{}); break; case 11: f(CodeTag<11>{}); break; case 12: f(CodeTag<12>{}); break;
+        default: f(CodeTag<0>{}); break;
     }
 }
 

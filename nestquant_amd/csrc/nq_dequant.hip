@@ -74,6 +74,7 @@ __device__ __forceinline__ void decode_unit_bk(const Planes& P, int lv, size_t u
         constexpr int CODE = decltype(tag)::value;
         uint32_t wr[Rec<CODE>::NW + 2];
         load_record<CODE>(wr, P.res, runit * 32 + lane32, rnrec);
+        prepare_record<CODE>(wr);
         ext_words<Rec<CODE>::BITS, Rec<CODE>::NW>(wr, __shfl(wr[0], src));
         decode_to_tile<true, CODE, BK>(wb, wr, k, tile, lane32);
     });

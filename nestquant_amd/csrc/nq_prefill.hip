@@ -440,7 +440,7 @@ __device__ __forceinline__ void wdecode_chunks(const Planes& P, const LaneCtx& L
         ext_base<0>(wb, __shfl(wb[0], L.src));
         const uint32_t sgm = ((var >> L.g) & 1u) * 0x80008000u;
         FoldK k;
-        if constexpr (RES) { ext_words<Rec<CODE>::BITS, Rec<CODE>::NW>(wr, __shfl(wr[0], L.src)); k = consts_fold(dw, sgm); }
+        if constexpr (RES) { prepare_record<CODE>(wr); ext_words<Rec<CODE>::BITS, Rec<CODE>::NW>(wr, __shfl(wr[0], L.src)); k = consts_fold(dw, sgm); }
         else k = consts_l2(sgm);
         u32x4* d = dst + (size_t)c * 8 * 64 + lane;
         static_for<4>([&](auto mm) {
@@ -634,6 +634,7 @@ __device__ __forceinline__ void pf_chunks(const Planes& P, const LaneCtx& L, int
         {
             if constexpr (RES)
             {
+                prepare_record<CODE>(wr);
                 ext_words<Rec<CODE>::BITS, Rec<CODE>::NW>(wr, __shfl(wr[0], L.src));
                 const FoldK k = consts_fold(dw, sgm);
                 static_for<4>([&](auto mm) {

@@ -134,6 +134,7 @@ __device__ __forceinline__ void gemv_chunks_masked(const Planes& P, const LaneCt
         const char* xp = L.xs + c * L.xstep;
         if (on)
         {
+            prepare_record<CODE>(wr);
             ext_words<Rec<CODE>::BITS, Rec<CODE>::NW>(wr, __shfl(wr[0], L.src));
             const FoldK k = consts_fold(dw, sgm);
             static_for<4>([&](auto mm) {
@@ -185,6 +186,7 @@ __device__ __forceinline__ void gemv_chunks(const Planes& P, const LaneCtx& L, i
         FoldK k;
         if constexpr (RES)
         {
+            prepare_record<CODE>(wr);
             ext_words<Rec<CODE>::BITS, Rec<CODE>::NW>(wr, __shfl(wr[0], L.src));
             k = consts_fold(dw, sgm);
         }

@@ -7,17 +7,19 @@ loaders and tests written against the reference read the same here. Base codes 0
 
 Nested levels of this build (the reference serves levels 0/2/4 only): an expert built with nested=True also carries
 P3 (64 bits / record, K=1 windows, code 10) with block words d3, and P4 (64 bits / record) with block words d4n. Level 3
-decodes base + P3; nested level 4 decodes base + the 128-bit record P3 || P4 read with K=2 windows (code 11). In device
-memory P4's uint2 sub-array follows P3's, so promotion 3 -> 4 uploads only P4 and d4n.
+decodes base + P3; nested level 4 decodes base + a 128-bit record made of P3's and P4's records and read with K=2 windows:
+either the two concatenated, P3 || P4 (code 11), or the two interleaved bit by bit, stream bit 2 i = P3 bit i and bit 2 i + 1 =
+P4 bit i (code 12, for experts built with interleave=True), so that every 16-bit window holds eight bits of each plane. In
+device memory P4's uint2 sub-array follows P3's either way, so promotion 3 -> 4 uploads only P4 and d4n.
 """
 import torch
 
 TBL_W = 20
 # window-pattern code -> (KA, MASK): step p carries KA + ((MASK >> (p % 16)) & 1) bits
 RKP = {0: (2, 0), 1: (1, 0xEEEE), 2: (2, 0xAAAA), 3: (2, 0x8888), 4: (3, 0), 5: (1, 0xAAAA), 6: (1, 0xFFFE),
-       7: (2, 0x9248), 8: (1, 0xFEFE), 9: (2, 0xD5AA), 10: (1, 0), 11: (2, 0)}
+       7: (2, 0x9248), 8: (1, 0xFEFE), 9: (2, 0xD5AA), 10: (1, 0), 11: (2, 0), 12: (2, 0)}
 RK_OF = {2: 0, 1.75: 1, 2.5: 2, 2.25: 3, 3: 4, 1.5: 5, 1.9375: 6, 2.3125: 7, 1.875: 8, 2.5625: 9}
-CODE_L3, CODE_L4N = 10, 11
+CODE_L3, CODE_L4N, CODE_L4B = 10, 11, 12
 
 
 def popc(m):
@@ -148,6 +150,15 @@ def rings_from_lane_words(w, bits, G=4):
 _MBN = None
 
 
+def interleave_words(p3w, p4w):
+    """record words of planes P3 and P4 (int64 [nrec, 2] holding uint32 values) -> the words [nrec, 4] of the 128-bit records of
+    window code 12: stream bit 2 i = bit i of P3's record, bit 2 i + 1 = bit i of P4's"""
+    sh = torch.arange(32, device=p3w.device)
+    bits = lambda w: ((w[..., None] >> sh) & 1).reshape(w.shape[0], 64)
+    both = torch.stack([bits(p3w), bits(p4w)], -1).reshape(p3w.shape[0], 4, 32)
+    return (both << sh).sum(-1)
+
+
 def all_MbN():
     """every valid block word (Mb, N): 1 <= Mb <= 255, 0 <= N <= 255, Mb + N <= 257"""
     global _MBN
@@ -243,7 +254,7 @@ class Expert:
     [H su_g | I sv_g | I sv_u | I su_d | H sv_o | H su_u] (reference sm120/moe.py:177-183)."""
 
     def __init__(s, H, I, seed, nm_gu=None, nm_dn=None, dev="cuda", rk_gu=0, rk_dn=0, mbn="rand", var=False,
-                 bk_gu=0, bk_dn=0, nested=False, gen_dev="cpu"):
+                 bk_gu=0, bk_dn=0, nested=False, gen_dev="cpu", interleave=False):
         gen = torch.Generator(device=gen_dev).manual_seed(seed)
         mbn_dn = mbn if mbn == "rand" else ("exh", mbn[1] + (2 * I // 16) * (H // 128))
         s.gu = Proj(2 * I, H, gen, nm_gu, rk_gu, mbn, var, bk_gu, nested).to(dev)
@@ -251,6 +262,7 @@ class Expert:
         signs = lambda n: torch.randint(0, 2, (n,), generator=gen, device=gen_dev) * 2 - 1
         s.signs = torch.cat([signs(2 * H + 3 * I), signs(H)]).half().to(dev)     # five vectors in one draw, then su_u
         s.H, s.I, s.nested = H, I, nested
+        s.l4code = CODE_L4B if interleave else CODE_L4N           # how nested level 4 reads P3 and P4: interleaved or concatenated
         s.lr, s.lr4, s.rg, s.rd = None, None, 0, 0
         if nested:                                       # slot image: [P3 | P4] per projection, contiguous
             s.gu.slot = s.gu.nested_plane(); s.dn.slot = s.dn.nested_plane()

@@ -9,7 +9,7 @@ import ctypes as C
 import torch
 
 from . import _lib
-from .format import (CODE_L3, CODE_L4N, RK_OF, RKP, TBL_W, Expert, Proj, all_MbN, make_flags, pack_words, popc, proj_sizes,  # noqa: F401
+from .format import (CODE_L3, CODE_L4B, CODE_L4N, RK_OF, RKP, TBL_W, Expert, Proj, all_MbN, make_flags, pack_words, popc, proj_sizes,  # noqa: F401
                      rbits, split_bits, step_off, unpack_words)
 
 
@@ -36,8 +36,8 @@ def H128(dev="cuda", n=128):
 
 def entry(ex, level):
     """table row int64[TBL_W] of expert `ex` at `level` (0, 2, 3, 4). Level 3 points at the one-bit plane p3 (code 10); level 4
-    points, for experts built with nested=True, at the record P3 || P4 (code 11), otherwise at the wide residual plane p4
-    (code rk)."""
+    points, for experts built with nested=True, at the planes P3 and P4 read as one record (code 11: concatenated, or code 12
+    for experts built with interleave=True: interleaved bit by bit), otherwise at the wide residual plane p4 (code rk)."""
     e = torch.zeros(TBL_W, dtype=torch.int64)
     e[0] = level
     nested = bool(getattr(ex, "nested", False))
@@ -60,7 +60,7 @@ def entry(ex, level):
             e[off + 3] = p.flags.data_ptr()
     e[9] = ex.signs.data_ptr()
     if nested or l3:
-        e[10] = e[11] = CODE_L3 if l3 else CODE_L4N
+        e[10] = e[11] = CODE_L3 if l3 else int(getattr(ex, "l4code", CODE_L4N))
     else:
         e[10], e[11] = ex.gu.rk, ex.dn.rk
     for i, p in ((12, ex.gu), (13, ex.dn)):

@@ -15,8 +15,8 @@
 #include <string.h>
 #include <stdlib.h>
 
-static const int PAT_KA[12]   = {2, 1, 2, 2, 3, 1, 1, 2, 1, 2, 1, 2};
-static const int PAT_MASK[12] = {0x0000, 0xEEEE, 0xAAAA, 0x8888, 0x0000, 0xAAAA, 0xFFFE, 0x9248, 0xFEFE, 0xD5AA, 0x0000, 0x0000};
+static const int PAT_KA[13]   = {2, 1, 2, 2, 3, 1, 1, 2, 1, 2, 1, 2, 2};
+static const int PAT_MASK[13] = {0x0000, 0xEEEE, 0xAAAA, 0x8888, 0x0000, 0xAAAA, 0xFFFE, 0x9248, 0xFEFE, 0xD5AA, 0x0000, 0x0000, 0x0000};
 
 static int popc(int m) { int c = 0; while (m) { c += m & 1; m >>= 1; } return c; }
 int nqo_rbits(int code) { return 4 * (16 * PAT_KA[code] + popc(PAT_MASK[code])); }
@@ -98,7 +98,8 @@ void nqo_fold_consts(int Mb, int N, uint16_t* Ah, uint16_t* Ch)
 }
 
 /* unpack the sub-array layout (uint4 x n4 | uint2 | uint | ushort | bit-packed tail) into words[nrec][NW];
- * split != 0: 128-bit records stored as uint2 | uint2 */
+ * split == 1: 128-bit records stored as uint2 | uint2 (plane P3's records, then plane P4's); split == 2: the same storage, the
+ * record being the two 64-bit records interleaved bit by bit (bit 2 i from P3, bit 2 i + 1 from P4) */
 void nqo_unpack(const uint8_t* buf, long nrec, int code, int split, uint32_t* words)
 {
     const int bits = nqo_rbits(code), nw = (bits + 31) / 32;
@@ -106,7 +107,16 @@ void nqo_unpack(const uint8_t* buf, long nrec, int code, int split, uint32_t* wo
     if (split)
     {
         const uint32_t* a = (const uint32_t*)buf; const uint32_t* b = a + nrec * 2;
-        for (long r = 0; r < nrec; ++r) { words[r * 4] = a[2 * r]; words[r * 4 + 1] = a[2 * r + 1]; words[r * 4 + 2] = b[2 * r]; words[r * 4 + 3] = b[2 * r + 1]; }
+        for (long r = 0; r < nrec; ++r)
+        {
+            if (split == 1) { words[r * 4] = a[2 * r]; words[r * 4 + 1] = a[2 * r + 1]; words[r * 4 + 2] = b[2 * r]; words[r * 4 + 3] = b[2 * r + 1]; continue; }
+            const uint64_t p3 = (uint64_t)a[2 * r] | ((uint64_t)a[2 * r + 1] << 32), p4 = (uint64_t)b[2 * r] | ((uint64_t)b[2 * r + 1] << 32);
+            for (int i = 0; i < 64; ++i)
+            {
+                words[r * 4 + (2 * i) / 32] |= (uint32_t)((p3 >> i) & 1u) << ((2 * i) & 31);
+                words[r * 4 + (2 * i + 1) / 32] |= (uint32_t)((p4 >> i) & 1u) << ((2 * i + 1) & 31);
+            }
+        }
         return;
     }
     const int n4 = bits / 128, r1 = bits % 128, n2 = r1 / 64, r2 = r1 % 64, n1 = r2 / 32, nh = (r2 % 32) / 16, T = bits % 16;

@@ -43,8 +43,20 @@ K0 = 1024.0 * A_ + B_                       # -3.453125 exactly
 RKP = {0: (2, 0x0000), 1: (1, 0xEEEE), 2: (2, 0xAAAA), 3: (2, 0x8888), 4: (3, 0x0000), 5: (1, 0xAAAA),
        6: (1, 0xFFFE), 7: (2, 0x9248), 8: (1, 0xFEFE), 9: (2, 0xD5AA),
        10: (1, 0x0000),                       # nested level 3: one refinement plane, 1 bit per step
-       11: (2, 0x0000)}                       # nested level 4: P3 record || P4 record, 2 bits per step
-NESTED_L3, NESTED_L4 = 10, 11
+       11: (2, 0x0000),                       # nested level 4: P3 record || P4 record, 2 bits per step
+       12: (2, 0x0000)}                       # nested level 4: P3 and P4 records interleaved bit by bit, 2 bits per step
+NESTED_L3, NESTED_L4, NESTED_L4B = 10, 11, 12
+
+
+def interleave_words(p3, p4):
+    """lane records of planes P3 and P4 (uint32 [nrec, 2] each: 64 bits per record) -> the 128-bit records [nrec, 4] whose
+    stream bit 2 i is bit i of P3's record and bit 2 i + 1 is bit i of P4's, so that every 16-bit window of the 2-bits-per-step
+    stream holds eight bits of each plane (the state of the reference's research decoder T2R2, threads/04-decode-kernel/
+    nqk.cu:109, in LSB-first stream order). Lane and ring boundaries stay where they are: the ring stream of the result is
+    the bitwise interleave of the two planes' ring streams."""
+    bits = lambda w: ((np.asarray(w, np.uint64)[..., None] >> np.arange(32, dtype=np.uint64)) & np.uint64(1)).reshape(len(w), -1)
+    b = np.stack([bits(p3), bits(p4)], -1).reshape(len(p3), 128)
+    return (b.reshape(len(p3), 4, 32) << np.arange(32, dtype=np.uint64)).sum(-1).astype(np.uint32)
 
 
 def popc(m):
@@ -271,6 +283,8 @@ class Plane:
         """-> (code, words, block words) used at `level`"""
         if level == 3:
             return NESTED_L3, self.p3, self.d3
+        if nested == "interleave":
+            return NESTED_L4B, interleave_words(self.p3, self.p4n), self.d4n
         if nested:
             return NESTED_L4, np.concatenate([self.p3, self.p4n], 1), self.d4n
         return self.rk, self.res, self.d4

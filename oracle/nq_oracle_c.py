@@ -42,6 +42,8 @@ def _p(a):
 
 
 def unpack(buf, nrec, code, split=False):
+    """split: False / 0 = the sub-array layout of `code`; True / 1 = P3's 64-bit records followed by P4's, concatenated per record
+    (code 11); 2 = the same storage, interleaved bit by bit per record (code 12)"""
     buf = np.ascontiguousarray(np.frombuffer(np.ascontiguousarray(buf).tobytes(), np.uint8))
     nw = (lib().nqo_rbits(code) + 31) // 32
     out = np.zeros((nrec, nw), np.uint32)

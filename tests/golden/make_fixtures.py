@@ -77,6 +77,40 @@ def shard_loader():
         np.savez_compressed(os.path.join(OUT, f"shards_{name}.npz"), **out)
 
 
+def nested_interleaved():
+    """10. two-plane level 4 with the planes interleaved bit by bit (stream bit 2 i = bit i of P3's lane record, bit 2 i + 1 =
+    bit i of P4's): the reference's generic decode_unit with Kr = 2 over the interleaved lane records, and level 3 (Kr = (1, 0))
+    over P3 alone from the same planes. The interleave is done here on Python integers, one record at a time. Needs only the
+    reference's numpy spec."""
+    sys.path.insert(0, REF)
+    import ref15_spec as SP
+    rng = np.random.default_rng(12)
+    units = []
+    for u in range(4):
+        base = rng.integers(0, 2**32, (32, 4), dtype=np.uint64).astype(np.uint32)
+        p3 = rng.integers(0, 2**32, (32, 2), dtype=np.uint64).astype(np.uint32)
+        p4 = rng.integers(0, 2**32, (32, 2), dtype=np.uint64).astype(np.uint32)
+        Mb3 = int(rng.integers(1, 256)); N3 = int(rng.integers(0, min(255, 257 - Mb3) + 1))
+        Mb4 = int(rng.integers(120, 256)); N4 = int(rng.integers(0, 257 - Mb4 + 1))
+        mixed = np.zeros((32, 4), np.uint32)
+        for lane in range(32):
+            a = int(p3[lane, 0]) | int(p3[lane, 1]) << 32
+            b = int(p4[lane, 0]) | int(p4[lane, 1]) << 32
+            v = 0
+            for i in range(64):
+                v |= ((a >> i) & 1) << (2 * i) | ((b >> i) & 1) << (2 * i + 1)
+            mixed[lane] = [(v >> (32 * k)) & 0xFFFFFFFF for k in range(4)]
+        bs = SP.rings_from_lane_words(base, 128)
+        Q2, Q3 = SP.decode_unit(bs, SP.rings_from_lane_words(p3, 64), Mb3, N3, Kb=2, Kr=(1, 0))
+        _, Q4 = SP.decode_unit(bs, SP.rings_from_lane_words(mixed, 128), Mb4, N4, Kb=2, Kr=2)
+        units.append(dict(base=base, p3=p3, p4=p4, d3=Mb3 | N3 << 8, d4=Mb4 | N4 << 8,
+                          U2=SP.to_unit(Q2).T.astype(np.float16).view(np.uint16),      # [16 rows, 128 cols]
+                          U3=SP.to_unit(Q3).T.astype(np.float16).view(np.uint16),
+                          U4=SP.to_unit(Q4).T.astype(np.float16).view(np.uint16)))
+    np.savez_compressed(os.path.join(OUT, "nested_interleaved_units.npz"),
+                        **{k: np.stack([np.asarray(u[k]) for u in units]) for k in units[0]})
+
+
 def main():
     R, SP = load_reference()
 
@@ -185,6 +219,7 @@ def main():
     base_code(R)
     rings_of_two(R)
     shard_loader()
+    nested_interleaved()
     print("fixtures written to", OUT)
 
 
@@ -195,5 +230,7 @@ if __name__ == "__main__":
         rings_of_two(load_reference()[0])
     elif sys.argv[1:] == ["shard_loader"]:       # only the fixtures of section 9
         load_reference(); shard_loader()
+    elif sys.argv[1:] == ["nested_interleaved"]:  # only the fixture of section 10
+        nested_interleaved()
     else:
         main()

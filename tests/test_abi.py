@@ -52,13 +52,14 @@ def test_validate_row_accepts_supported_rows():
     assert _validate(_row(f0=4, f2=8, f3=8, f6=8, f7=8, f10=7, f11=3)) == 0
     assert _validate(_row(f0=3, f2=8, f3=8, f6=8, f7=8, f10=10, f11=10)) == 0
     assert _validate(_row(f0=4, f2=8, f3=8, f6=8, f7=8, f10=11, f11=11, f12=8, f18=128)) == 0
+    assert _validate(_row(f0=4, f2=8, f3=8, f6=8, f7=8, f10=12, f11=12)) == 0            # P3 and P4 interleaved
     assert _validate(_row(f19=1)) == 0 and _validate(_row(f19=0x101)) == 0 and _validate(_row(f19=0x100)) == 0   # K = 1.75 base
 
 
 @pytest.mark.parametrize("bad,word", [
     (dict(f0=1), "level"), (dict(f0=5), "level"), (dict(f0=3, f2=8, f3=8, f6=8, f7=8, f10=10, f11=10, f4=8), "mask mode"), (dict(f0=4, f2=8, f3=8, f6=8, f7=8, f10=11, f11=11, f8=8), "mask mode"),
     (dict(f14=8), "low-rank"), (dict(f16=2), "low-rank"), (dict(f18=512), "in_had_down"), (dict(f19=2), "base code"), (dict(f19=0x10001), "base code"),
-    (dict(f0=4), "residual planes"), (dict(f0=4, f2=8, f3=8, f6=8, f7=8, f10=12), "out of range"),
+    (dict(f0=4), "residual planes"), (dict(f0=4, f2=8, f3=8, f6=8, f7=8, f10=13), "out of range"),
     (dict(f0=3, f2=8, f3=8, f6=8, f7=8, f10=0, f11=10), "level 3"), (dict(f0=4, f2=8, f3=8, f6=8, f7=8, f10=10), "level 4"),
     (dict(f1=0), "null base"),
 ])
@@ -72,7 +73,7 @@ def test_shape_errors_and_code_masks():
     assert _validate(_row(), H=200) != 0 and "multiples of 128" in _lib.lib().nq_last_error().decode()
     out = (C.c_uint32 * 4)()
     assert _lib.lib().nq_codes(out) == 0
-    assert out[0] == out[1] == 0xFFF and out[2] == out[3] == 3
+    assert out[0] == out[1] == 0x1FFF and out[2] == out[3] == 3
     with pytest.raises(RuntimeError, match="multiples of 128"):
         _lib.check(_validate(_row(), I=100))
 

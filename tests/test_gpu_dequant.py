@@ -27,10 +27,13 @@ class _Ex:
         s.lr = None
 
 
-def gpu_dense(p, level, N, K, mode=0):
-    """decode projection p (already on the device) as gate|up (mode 0: N = 2I, K = H) or down (mode 1)"""
+def gpu_dense(p, level, N, K, mode=0, l4code=None):
+    """decode projection p (already on the device) as gate|up (mode 0: N = 2I, K = H) or down (mode 1); l4code: the window code
+    nested level 4 reads P3 and P4 with (default: concatenated)"""
     H, I = (K, N // 2) if mode == 0 else (N, K)
     ex = _Ex(p, mode, H, I)
+    if l4code is not None:
+        ex.l4code = l4code
     if p.nested:
         p.slot = p.nested_plane()
     row = M.entry(ex, level)
@@ -64,6 +67,36 @@ def test_golden_nested_units():
         W = gpu_dense(p, lv, 16, 128 * n, mode=1)
         for u in range(n):
             assert same_f16(W[:, 128 * u:128 * (u + 1)], z[key][u].view(np.float16)) == 0, (lv, u)
+
+
+def test_golden_interleaved_nested_units():
+    """window code 12 (P3 and P4 interleaved bit by bit) on the fixture the reference's generic decode_unit wrote; both dense
+    decoders (stand-alone and the multi-expert prefill decode)"""
+    z = np.load(os.path.join(GOLD, "nested_interleaved_units.npz"))
+    n = z["base"].shape[0]
+    gen = torch.Generator().manual_seed(0)
+    p = F.Proj(16, 128 * n, gen, nested=True)
+    p.base = torch.from_numpy(z["base"].reshape(-1).view(np.int32).copy())
+    p.p3 = F.pack_words(torch.from_numpy(z["p3"].reshape(-1, 2).astype(np.int64)), 64)
+    p.p4n = F.pack_words(torch.from_numpy(z["p4"].reshape(-1, 2).astype(np.int64)), 64)
+    p.d3 = torch.from_numpy(z["d3"].astype(np.int32)); p.d4n = torch.from_numpy(z["d4"].astype(np.int32))
+    p.to(DEV)
+    for lv, key in ((2, "U2"), (3, "U3"), (4, "U4")):
+        W = gpu_dense(p, lv, 16, 128 * n, mode=1, l4code=F.CODE_L4B)
+        for u in range(n):
+            assert same_f16(W[:, 128 * u:128 * (u + 1)], z[key][u].view(np.float16)) == 0, (lv, u)
+
+
+@pytest.mark.parametrize("var", [False, True])
+def test_interleaved_nested_projection_vs_oracle(var):
+    """a projection of several strips and chunks at levels 3 and interleaved 4, sign plane on and off, against the numpy oracle"""
+    gen = torch.Generator().manual_seed(31)
+    p = F.Proj(64, 512, gen, None, 0, "rand", var=var, nested=True)
+    op = oracle_plane(p)
+    p.to(DEV)
+    for mode in (0, 1):
+        assert same_f16(gpu_dense(p, 4, 64, 512, mode=mode, l4code=F.CODE_L4B), O.dense_W(op, 4, nested="interleave")) == 0
+        assert same_f16(gpu_dense(p, 3, 64, 512, mode=mode, l4code=F.CODE_L4B), O.dense_W(op, 3, nested=True)) == 0
 
 
 @pytest.mark.parametrize("rk", range(10))

@@ -78,6 +78,47 @@ def test_small_layer_all_levels_and_codes_vs_full_oracle():
         assert rel_err(y.cpu().numpy(), pure) < 1e-3
 
 
+def test_interleaved_two_plane_level4_in_decode_and_prefill():
+    """experts whose nested level 4 reads P3 and P4 interleaved bit by bit (window code 12) beside concatenated ones (code 11) in
+    one layer: the decode path at 1-8 tokens and prefill() against the oracle's decode and layer math; the same experts at level
+    3 read P3 alone"""
+    H, I, NE = 512, 256, 6
+    ex = []
+    for i in range(NE):
+        ex.append(F.Expert(H, I, seed=500 + i, dev="cpu", nested=True, interleave=i % 2 == 0, var=i == 2))
+    kind = ["interleave" if e.l4code == F.CODE_L4B else True for e in ex]
+    planes = [(oracle_plane(e.gu), oracle_plane(e.dn), k) for e, k in zip(ex, kind)]
+    signs = [e.signs.numpy() for e in ex]
+    levels = [4, 4, 4, 3, 3, 2]
+    to_dev(ex)
+    L = M.MoELayer(NE, H, I, Bmax=8, topk=3)
+    for e in range(NE):
+        L.set(e, ex[e], levels[e])
+    assert [int(L.table[e, 10]) for e in range(NE)] == [12, 11, 12, 10, 10, 11]
+    rng = random.Random(4)
+    g = torch.Generator().manual_seed(6)
+    for B in (1, 4, 8):
+        sel, rw = RT.routing_tensors(RT.make_sel(B, range(NE), "recency", p=0.5, rng=rng, topk=3), seed=B)
+        x = (torch.randn(B, H, generator=g) * 0.05).half().to(DEV)
+        want = oracle_layer(planes, levels, signs, x, sel, rw)
+        y = L(x, sel, rw).clone()
+        torch.cuda.synchronize()
+        assert rel_err(y.cpu().numpy(), want) < 5e-5, B
+    T = 40
+    sel = torch.stack([torch.randperm(NE, generator=g)[:3] for _ in range(T)]).to(DEV)
+    rw = torch.rand(T, 3, generator=g).half().to(DEV)
+    x = (torch.randn(T, H, generator=g) * 0.05).half().to(DEV)
+    want = oracle_layer(planes, levels, signs, x, sel, rw)
+    y = L.prefill(x, sel, rw)
+    torch.cuda.synchronize()
+    assert rel_err(y.cpu().numpy(), want) < 5e-5
+    # the two readings of the same planes differ: an expert flipped from interleaved to concatenated changes the result
+    ex[0].l4code = F.CODE_L4N
+    L.set(0, ex[0], 4)
+    sel1 = torch.tensor([[0, 1, 2]], device=DEV); rw1 = torch.tensor([[0.5, 0.25, 0.25]], device=DEV).half()
+    assert rel_err(L(x[:1], sel1, rw1).cpu().numpy(), oracle_layer(planes, levels, signs, x[:1], sel1, rw1)) > 1e-2
+
+
 def test_golden_layer_fixture(golden_dir):
     """the reference's own moe_ref output on the small golden layer (levels 2/4/4/0, codes 3/7, a sign plane, rw == 0)"""
     z = np.load(f"{golden_dir}/layer_small.npz")

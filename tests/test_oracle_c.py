@@ -15,8 +15,8 @@ GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 
 def test_scalar_pieces():
     L = OC.lib()
-    assert [L.nqo_rbits(c) for c in range(12)] == [O.rbits(c) for c in range(12)]
-    for c in range(12):
+    assert [L.nqo_rbits(c) for c in range(13)] == [O.rbits(c) for c in range(13)]
+    for c in range(13):
         assert [L.nqo_step_off(p, c) for p in range(0, 257, 3)] == O.step_off(np.arange(0, 257, 3), *O.RKP[c]).tolist()
     st = np.arange(0, 65536, 13)
     assert [L.nqo_hash_sum(int(s)) for s in st] == O.hash_sum(st).tolist()
@@ -74,5 +74,9 @@ def test_nested_levels_and_random_projection_vs_numpy():
     assert same_f16(OC.decode_proj(op.base, 64, 384, 3, 10, op.p3, op.d3, op.var), O.dense_W(op, 3, nested=True)) == 0
     both = np.concatenate([op.p3, op.p4n], 1)
     assert same_f16(OC.decode_proj(op.base, 64, 384, 4, 11, both, op.d4n, op.var), O.dense_W(op, 4, nested=True)) == 0
+    stored = np.concatenate([op.p3.reshape(-1), op.p4n.reshape(-1)])                  # the device layout: P3's records, then P4's
+    mixed = OC.unpack(stored, op.p3.shape[0], 12, split=2)
+    assert np.array_equal(mixed, O.interleave_words(op.p3, op.p4n))
+    assert same_f16(OC.decode_proj(op.base, 64, 384, 4, 12, mixed, op.d4n, op.var), O.dense_W(op, 4, nested="interleave")) == 0
     W = O.dense_W(op, 4); x = np.random.default_rng(0).standard_normal(384).astype(np.float32)
     assert np.allclose(OC.matvec_f16(W, x), W.astype(np.float32) @ x, rtol=1e-4, atol=1e-3)

@@ -18,7 +18,7 @@ PROJ_FILES = sorted(glob.glob(os.path.join(GOLD, "proj_rk*_var*.npz")))
 
 def test_fixture_inventory():
     assert len(PROJ_FILES) == 8 and len(glob.glob(os.path.join(GOLD, "proj_bk1_rk*.npz"))) == 2
-    for f in ("nested_units.npz", "layer_small.npz", "pack_words.npz"):
+    for f in ("nested_units.npz", "nested_interleaved_units.npz", "layer_small.npz", "pack_words.npz"):
         assert os.path.exists(os.path.join(GOLD, f))
 
 
@@ -76,6 +76,31 @@ def test_nested_levels_match_reference_generic_decoder():
         for u in range(n):
             assert same_f16(W[:, 128 * u:128 * (u + 1)], z[key][u].view(np.float16)) == 0, (lv, u)
     assert same_f16(O.dense_W(p, 3, nested=True), O.dense_W(p, 4, nested=True)) > 1000
+
+
+def test_interleaved_two_plane_level4_matches_reference_generic_decoder():
+    """window code 12: level 4 over P3 and P4 interleaved bit by bit = the reference's decode_unit(Kr=2) over lane records that the
+    fixture script interleaved on Python integers; level 3 over the same P3 as before; the interleave itself by its definition"""
+    z = np.load(os.path.join(GOLD, "nested_interleaved_units.npz"))
+    n = z["base"].shape[0]
+    base = z["base"].reshape(n * 32, 4); p3 = z["p3"].reshape(n * 32, 2); p4 = z["p4"].reshape(n * 32, 2)
+    p = O.Plane(16, 128 * n, base, p3=p3, d3=z["d3"].astype(np.uint32), p4n=p4, d4n=z["d4"].astype(np.uint32))
+    for lv, key in ((2, "U2"), (3, "U3"), (4, "U4")):
+        W = O.dense_W(p, lv, nested="interleave")
+        for u in range(n):
+            assert same_f16(W[:, 128 * u:128 * (u + 1)], z[key][u].view(np.float16)) == 0, (lv, u)
+    assert same_f16(O.dense_W(p, 4, nested="interleave"), O.dense_W(p, 4, nested=True)) > 1000       # not the concatenated record
+    il = O.interleave_words(p3, p4)
+    as_int = lambda w: [sum(int(v) << (32 * i) for i, v in enumerate(r)) for r in w]
+    for a, b, v in zip(as_int(p3[:9]), as_int(p4[:9]), as_int(il[:9])):
+        assert all((v >> (2 * i)) & 1 == (a >> i) & 1 and (v >> (2 * i + 1)) & 1 == (b >> i) & 1 for i in range(64))
+    t = F.interleave_words(torch.from_numpy(p3.astype(np.int64)), torch.from_numpy(p4.astype(np.int64)))
+    assert np.array_equal(t.numpy().astype(np.uint32), il)
+    # every 16-bit window of the 2-bits-per-step stream holds eight bits of each plane: state(j) of lane 0, read off the planes
+    a, b = as_int(p3[:1])[0], as_int(p4[:1])[0]
+    for j in (0, 5, 31, 40, 56):
+        st = (as_int(il[:1])[0] >> (2 * j)) & 0xFFFF
+        assert all((st >> (2 * m)) & 1 == (a >> (j + m)) & 1 and (st >> (2 * m + 1)) & 1 == (b >> (j + m)) & 1 for m in range(8))
 
 
 def _small_layer():
