@@ -513,12 +513,15 @@ def config2_leg(L, ex, levels, dev, R=64, reps=4):
     s = torch.cuda.Stream()
     picks = [(37 * i) % E for i in range(R)]
     out = {}
-    for lv in (2, 3, 4):
+    for tag in ("2", "3", "4", "4i"):                           # 4 = P3 || P4 (window code 11); 4i = P3 and P4 interleaved (code 12)
+        lv = int(tag[0])
         for e in picks:
+            ex[e].l4code = F.CODE_L4B if tag == "4i" else F.CODE_L4N
             L.set(e, ex[e], lv)
+            ex[e].l4code = F.CODE_L4N
         nbytes = sum(code_bytes(ex, [lv] * E, [e], which="gu") for e in picks) / R
         for B in (1, 4, 8):
-            if B > L.out.shape[0]:
+            if B > L.out.shape[0] or (tag == "4i" and B != 1):
                 continue
             x = (torch.randn(B, H, generator=g) * 0.05).half().to(dev)
             rw = torch.ones(B, 1, dtype=torch.float16, device=dev)
@@ -579,13 +582,14 @@ def config2_leg(L, ex, levels, dev, R=64, reps=4):
             fin = alone(1 | 4, best[1])
             part = min((alone(1 | 4 | 8, nst), nst) for nst in (6, 3, 2))      # as the layer runs it: ends with the k-slice partial sums
             L.route, L.xrot = keep
-            out[f"L{lv}_B{B}"] = dict(us=round(best[0], 2), GBps=round(nbytes / best[0] / 1e3, 1), k_slice_chunks=best[1],
+            out[f"L{tag}_B{B}"] = dict(us=round(best[0], 2), GBps=round(nbytes / best[0] / 1e3, 1), k_slice_chunks=best[1],
                                       us_projection_launch=round(fin, 2), GBps_projection_launch=round(nbytes / fin / 1e3, 1),
                                       us_to_partial_sums=round(part[0], 2), GBps_to_partial_sums=round(nbytes / part[0] / 1e3, 1),
                                       k_slice_chunks_to_partial_sums=part[1])
     L.table.copy_(saved)
     out["workload"] = ("one expert's gate|up projection per launch (N=4096, K=6144), 64 experts in turn, best k-slice of 12 / 6 / 3 / 2 chunks; "
-                       "code bytes per launch: " + ", ".join(f"L{lv} {int(sum(code_bytes(ex, [lv] * E, [e], which='gu') for e in picks) / R)}" for lv in (2, 3, 4)))
+                       "code bytes per launch: " + ", ".join(f"L{lv} {int(sum(code_bytes(ex, [lv] * E, [e], which='gu') for e in picks) / R)}" for lv in (2, 3, 4))
+                       + "; L4 reads planes P3 and P4 as one record P3 || P4, L4i reads them interleaved bit by bit (same bytes, ~1 more vector instruction per weight)")
     return out
 
 

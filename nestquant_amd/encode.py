@@ -87,6 +87,62 @@ def viterbi_ring(w, lut, K=2, state_bits=16):
     return idx
 
 
+def spread8(a):
+    """8-bit values -> their bits at the even positions of a 16-bit value (bit i -> bit 2 i)"""
+    a = (a | (a << 4)) & 0x0F0F
+    a = (a | (a << 2)) & 0x3333
+    return (a | (a << 1)) & 0x5555
+
+
+def viterbi_ring_given_p3(w, a, lut):
+    """The second refinement plane of the interleaved two-plane code, with the first one frozen. Stream bit 2 p is P3's bit p
+    (given), bit 2 p + 1 is P4's bit p (sought); the state at position p interleaves the 8-bit windows a(p) = P3 bits [p, p + 8)
+    and b(p) = P4 bits [p, p + 8): state = spread(a) | spread(b) << 1. What is left to choose is one bit per step with eight steps
+    of memory, over a codebook that changes from step to step with a: value(b) = lut[spread(a) | spread(b) << 1].
+    w [T, L] targets and a [T, L] P3 windows, both in Viterbi order (b_t = ((b_{t-1} << 1) | new bit) mod 256) -> b int64 [T, L],
+    the tail-biting path of least squared error, found as viterbi_ring finds its own (two passes)."""
+    T, L = w.shape
+    dev = w.device
+    E = 128                                                      # low seven bits of b ("edge"); its top bit is the choice
+    e = torch.arange(E, device=dev)
+    q = torch.arange(2, device=dev)
+    states = (q[:, None] << 7) | e[None, :]
+    prev = states >> 1
+    sb = spread8(states) << 1                                    # P4's share of the 16-bit state
+    sa = spread8(a)
+    back = torch.empty((L, T, E), dtype=torch.uint8, device=dev)
+
+    def forward(roll, pre):
+        cost = None
+        for i in range(L):
+            ri = (i + roll) % L
+            d = (lut[sa[:, ri, None, None] | sb[None]] - w[:, ri, None, None]).square()     # [T, 2, E]
+            if cost is None:
+                c = d if pre is None else torch.where(prev[None] == pre[:, None, None], d, torch.full_like(d, float("inf")))
+            else:
+                c = d + cost[:, prev]
+            cost, arg = c.min(1)
+            back[ri] = arg.to(torch.uint8)
+        return cost
+
+    def trace(roll, edge, stop_at_zero):
+        out = torch.empty((T, L), dtype=torch.int64, device=dev)
+        tt = torch.arange(T, device=dev)
+        for i in range(L - 1, -1, -1):
+            ri = (i + roll) % L
+            st = (back[ri][tt, edge].long() << 7) | edge
+            out[:, ri] = st
+            edge = st >> 1
+            if stop_at_zero and ri == 0:
+                break
+        return out, edge
+
+    c = forward(L // 2, None)
+    _, start = trace(L // 2, c.argmin(1), True)
+    forward(0, start)
+    return trace(0, start, False)[0]
+
+
 def ring_index(dev="cpu"):
     """[8, 256]: ring g, position p -> index (column * 16 + row) inside a 16 x 128 unit (reference ref15_spec.py:118-125)"""
     g = torch.arange(8, device=dev)[:, None, None]; t4 = torch.arange(4, device=dev)[None, :, None]
@@ -137,6 +193,25 @@ def viterbi_rings(rings, K=2, chunk=64):
     for a in range(0, rings.shape[0], chunk):
         st[a:a + chunk] = viterbi_ring(rings[a:a + chunk][:, ip].contiguous(), lut, K)[:, ip]
     return st
+
+
+def viterbi_rings_given_p3(rings, st3, chunk=256):
+    """rings [T, 256] targets and st3 [T, 256] the 16-bit states of the one-bit plane P3, both in ring position order ->
+    (b [T, 256]: 8-bit windows of plane P4, st4 [T, 256]: the 16-bit states of the interleaved stream), position order"""
+    dev = rings.device
+    ip = (-torch.arange(256, device=dev)) % 256
+    lut = codebook(dev)
+    a = st3 & 0xFF                                               # P3 bits [p, p + 8)
+    b = torch.empty(rings.shape, dtype=torch.int64, device=dev)
+    for i in range(0, rings.shape[0], chunk):
+        b[i:i + chunk] = viterbi_ring_given_p3(rings[i:i + chunk][:, ip].contiguous(), a[i:i + chunk][:, ip].contiguous(), lut)[:, ip]
+    return b, spread8(a) | (spread8(b) << 1)
+
+
+def one_bit_states(bits):
+    """ring bits [T, 256] (bit p of a one-bit-per-step stream) -> the 16-bit states [T, 256]: state(p) = bits [p, p + 16), wrapping"""
+    idx = (torch.arange(256, device=bits.device)[:, None] + torch.arange(16, device=bits.device)[None]) % 256
+    return (bits[:, idx] << torch.arange(16, device=bits.device)).sum(-1)
 
 
 def lane_records(st, K):
@@ -193,6 +268,7 @@ def encode_level2(W, seed=0, chunk=64):
 A_ = float(torch.tensor([0x1EEE], dtype=torch.int16).view(torch.float16))
 K0 = 1024.0 * A_ + float(torch.tensor([0xC931 - 65536], dtype=torch.int16).view(torch.float16))
 RES_SCALE = {1: 1.1, 2: 1.0}     # best input scale of the refinement stage on Gaussian data (reference exp3_mul1L.log:3-4)
+RES_SCALE_GIVEN_P3 = 1.2         # the same for the interleaved second plane (one free bit per step, eight steps of memory); found here
 
 
 def hash_sum(st):
@@ -275,11 +351,14 @@ def base_rings(rings, chunk=64, var=False):
     return st, sign
 
 
-def encode_residual(target, st_base, K, chunk=64, scale=None, cost=None, sign=None):
+def encode_residual(target, st_base, K, chunk=64, scale=None, cost=None, sign=None, p3_states=None, states=None):
     """One refinement stage on the frozen base plane. target fp32 [U, 8, 256] and st_base int64 [U, 8, 256] in ring position
     order, K = 1 or 2 bits per weight -> dict(states [U, 8, 256], Mb [U], N [U], Q fp32 [U, 8, 256], delta [U]).
     cost: error fp64 [U, 8, 256] -> [U], what the block-word search minimises (default: the squared error).
-    sign [U, 8, 1] (+-1): rings whose decoded values are negated, base and refinement alike."""
+    sign [U, 8, 1] (+-1): rings whose decoded values are negated, base and refinement alike.
+    p3_states [U, 8, 256] (with K = 2): the 16-bit states of an already fitted one-bit plane P3, which stays as it is; the stage
+    then fits plane P4 of the interleaved two-plane code (window code 12) and also returns its ring bits as `p4_bits`.
+    states [U, 8, 256]: the refinement plane's states are these (no search); only the block word is fitted."""
     U = target.shape[0]
     dev = target.device
     lut = codebook(dev)
@@ -288,8 +367,17 @@ def encode_residual(target, st_base, K, chunk=64, scale=None, cost=None, sign=No
     Sb = hash_sum(st_base)
     r = (target * sign).double() - lut[st_base].double()         # in the ring's own orientation
     rms = r.square().mean((1, 2)).sqrt().clamp_min(1e-12)
-    s0 = rms / (RES_SCALE[K] if scale is None else scale)
-    st = viterbi_rings((r / s0[:, None, None]).float().reshape(U * 8, 256), K, chunk).reshape(U, 8, 256)
+    p4_bits = None
+    if states is not None:
+        st = states
+    elif p3_states is None:
+        s0 = rms / (RES_SCALE[K] if scale is None else scale)
+        st = viterbi_rings((r / s0[:, None, None]).float().reshape(U * 8, 256), K, chunk).reshape(U, 8, 256)
+    else:
+        assert K == 2
+        s0 = rms / (RES_SCALE_GIVEN_P3 if scale is None else scale)
+        b, st = viterbi_rings_given_p3((r / s0[:, None, None]).float().reshape(U * 8, 256), p3_states.reshape(U * 8, 256))
+        st, p4_bits = st.reshape(U, 8, 256), (b & 1).reshape(U, 8, 256)
     Sr = hash_sum(st)
     a = A_ * Sr.double() + K0                                    # unrounded value of the refinement code
     delta = ((a * r).sum((1, 2)) / a.square().sum((1, 2)).clamp_min(1e-30)).clamp_min(0)
@@ -304,7 +392,7 @@ def encode_residual(target, st_base, K, chunk=64, scale=None, cost=None, sign=No
             w = c < best["c"]
             best["c"] = torch.where(w, c, best["c"]); best["Q"][w] = q[w]
             best["Mb"][w] = Mbs[w, ci]; best["N"][w] = Ns[w, ci]
-    return dict(states=st, Mb=best["Mb"], N=best["N"], Q=best["Q"], delta=delta)
+    return dict(states=st, Mb=best["Mb"], N=best["N"], Q=best["Q"], delta=delta, p4_bits=p4_bits)
 
 
 def pack_planes(r, N, K, st2, fits, sign=None):
@@ -321,6 +409,12 @@ def pack_planes(r, N, K, st2, fits, sign=None):
         r["var"] = ((sign.reshape(-1, 8) < 0).long() << torch.arange(8, device=dev)).sum(1).to(torch.uint8)
     r["Q"] = from_rings(q2.reshape(-1, 256), N, K)
     for lvl, e in fits.items():
+        if lvl == "4n":                                          # plane P4 of the interleaved two-plane level 4: 64-bit records of its own
+            r["p4n"] = pack_words(lane_records(one_bit_states(e["p4_bits"].reshape(-1, 256)), 1), 64)
+            r["d4n"] = signed32(e["Mb"] | (e["N"] << 8))
+            r["Q4n"] = from_rings(e["Q"].reshape(-1, 256), N, K)
+            r["states4n"] = e["states"]
+            continue
         bpw = lvl - 2
         r["p%d" % lvl] = pack_words(lane_records(e["states"].reshape(-1, 256), bpw), 64 * bpw)
         r["d%d" % lvl] = signed32(e["Mb"] | (e["N"] << 8))
@@ -329,18 +423,39 @@ def pack_planes(r, N, K, st2, fits, sign=None):
     return r
 
 
-def encode_nested(W, seed=0, chunk=64, var=False):
+def encode_nested(W, seed=0, chunk=64, var=False, interleave=False, share4=0.0):
     """encode_level2 plus the two refinement planes, each fitted to the residual of the same frozen base plane:
     p3 / d3 (one bit per weight, 64-bit records; level 3 = base + P3) and p4 / d4 (two bits per weight, 128-bit records of
     window code 0; level 4 = base + the wide plane). Adds p3, d3, Q3, p4, d4, Q4 (Q3 / Q4 fp32 [N, K]: the matrices the
     decoder reproduces bit for bit at levels 3 / 4) to encode_level2's dict. var: also fit every ring negated and keep the
-    better orientation (adds the sign plane `var`)."""
+    better orientation (adds the sign plane `var`).
+    interleave: also the strictly nested two-plane level 4 of window code 12 -- P3 stays as level 3 fitted it and a second
+    one-bit plane P4 is fitted so that base + the bitwise interleave of P3 and P4 is as close as one more bit per weight gets
+    it: adds p4n, d4n, Q4n (a promotion 2 -> 3 -> 4 then uploads P3 + d3, then P4 + d4n). Both levels read one hashed window
+    per weight, so the bits that level 3 chose carry nothing for level 4's code: with P3 frozen everywhere, level 4 is a fresh
+    one-bit fit with half the memory, no better than level 3 (N(0,1): 0.0209 against 0.0186). share4 in [0, 1] trades the levels
+    against each other unit by unit: that share of the units (largest base residual first) gets both planes from one two-bit fit
+    -- P3 = the low bit, P4 = the high bit of every step, so level 4 is the wide plane's fit there -- while level 3 in those
+    units falls back to about the base plane (its block word is fitted to bits not chosen for it and comes out near N = 0)."""
     N, K = W.shape
     su, sv, target = prepare(W, seed)
     tr = to_rings(target).reshape(-1, 8, 256)
     st2, sign = base_rings(tr.reshape(-1, 256), chunk, var)
     st2, sign = st2.reshape(-1, 8, 256), sign.reshape(-1, 8, 1)
     fits = {lvl: encode_residual(tr, st2, lvl - 2, chunk, sign=sign) for lvl in (3, 4)}
+    if interleave:
+        fits["4n"] = encode_residual(tr, st2, 2, chunk, sign=sign, p3_states=fits[3]["states"])
+        nj = int(round(share4 * tr.shape[0]))
+        if nj:
+            resid = (tr * sign - codebook(tr.device)[st2]).square().sum((1, 2))
+            ju = torch.argsort(resid, descending=True)[:nj]
+            wide = fits[4]["states"][ju]                         # two bits per step: bit 0 of each state is P3's, bit 1 is P4's
+            st3 = one_bit_states((wide & 1).reshape(-1, 256)).reshape(nj, 8, 256)
+            e3 = encode_residual(tr[ju], st2[ju], 1, chunk, sign=sign[ju], states=st3)
+            for k in ("states", "Mb", "N", "Q"):
+                fits[3][k][ju] = e3[k]
+                fits["4n"][k][ju] = fits[4][k][ju]
+            fits["4n"]["p4_bits"][ju] = (wide >> 1) & 1
     return pack_planes(dict(su=su, sv=sv, target=target), N, K, st2, fits, sign if var else None)
 
 
@@ -428,9 +543,11 @@ class EncodedProj(Proj):
     """a Proj (nestquant_amd.format) holding encoded planes: the level-2 base plane and, when given, the refinement planes
     p3 / d3 (level 3, the one-bit nested plane), p4 / d4 (level 4, wide plane of window code 0) and the sign plane var"""
 
-    def __init__(s, N, K, base, p3=None, d3=None, p4=None, d4=None, var=None):
+    def __init__(s, N, K, base, p3=None, d3=None, p4=None, d4=None, var=None, p4n=None, d4n=None):
+        """p4n / d4n: plane P4 and the block words of the nested two-plane level 4; with them the projection is `nested` (its
+        level-4 row then points at P3 followed by P4 in one buffer, `slot`, read with the expert's l4code)"""
         s.z = proj_sizes(N, K)
-        s.N, s.K, s.rk, s.bk, s.nested = N, K, 0, 0, False
+        s.N, s.K, s.rk, s.bk, s.nested = N, K, 0, 0, p4n is not None
         s.base = base
         zero = lambda: torch.zeros(1, dtype=torch.int32, device=base.device)
         s.p4 = zero() if p4 is None else p4
@@ -438,4 +555,7 @@ class EncodedProj(Proj):
         s.p4w = s.Mb = s.Nn = s.flags = s.fl = None
         s.var = var
         s.p3, s.d3 = p3, d3
-        s.p4n = s.d4n = s.p3w = s.p4nw = None
+        s.p4n, s.d4n = p4n, d4n
+        s.p3w = s.p4nw = None
+        if s.nested:
+            s.slot = torch.cat([p3, p4n])

@@ -113,6 +113,63 @@ def test_refinement_distortion_matches_reference_report():
             assert float(mine) <= float(c.min()) * 1.01
 
 
+def test_second_plane_search_with_the_first_plane_frozen():
+    """viterbi_ring_given_p3 on rings of 16 steps against brute force over all 2^16 P4 rings: a valid tail-biting ring (every
+    8-bit window extends its predecessor, also across the wrap); exactly the best of all rings that close on the same seven
+    bits (the second pass is an exact search under that constraint); never better than the best ring of all. How close it
+    comes to that one is the two-pass heuristic's business (the reference's, harness.py:297-364), and a ring of 16 steps is
+    only twice this code's memory, where the real rings are 32 times."""
+    g = torch.Generator().manual_seed(3)
+    L = 16
+    lut = EN.codebook()
+    seqs = torch.arange(1 << L)
+    bits = (seqs[:, None] >> torch.arange(L)) & 1                 # bits[s, i] = the bit that enters at Viterbi step i
+    win = torch.zeros(1 << L, L, dtype=torch.int64)
+    for i in range(L):
+        for back in range(8):
+            win[:, i] |= bits[:, (i - back) % L] << back
+    for trial in range(4):
+        w = torch.randn(3, L, generator=g) * 1.2
+        a = torch.randint(0, 256, (3, L), generator=g)
+        b = EN.viterbi_ring_given_p3(w, a, lut)
+        for t in range(3):
+            for i in range(L):
+                assert int(b[t, i]) >> 1 == int(b[t, (i - 1) % L]) & 0x7F
+            err = (lut[EN.spread8(a[t])[None] | EN.spread8(win) << 1] - w[t][None]).square().sum(1)
+            got = float((lut[EN.spread8(a[t]) | EN.spread8(b[t]) << 1] - w[t]).square().sum())
+            same_close = (win[:, L - 1] & 0x7F) == (int(b[t, L - 1]) & 0x7F)
+            assert abs(got - float(err[same_close].min())) < 1e-4, (trial, t)
+            assert got >= float(err.min()) - 1e-5
+
+
+def test_interleaved_two_plane_level4_fit_and_what_it_costs():
+    """encode_nested(interleave=True): level 3 = base + P3 as before; level 4 = base + P3 and P4 interleaved (window code 12),
+    decoded bit for bit by the oracle from the packed planes. With P3 frozen everywhere the second plane is a fresh one-bit fit
+    with eight steps of memory, no better than level 3 -- the two levels read unrelated hashed windows, so a strictly nested
+    hash code cannot be good at both (the reference's three-plane code that reaches 0.00516 / 0.00493 ADDS two refinement
+    terms, threads/03-nested-trellis-code/REPORT.md:27-28, which this single-window format cannot express). share4 moves
+    units from one end to the other: both planes of a unit from one two-bit fit (level 4 = the wide plane's 0.0047 there, level
+    3 ~ the base plane's 0.068)."""
+    g = torch.Generator().manual_seed(2)
+    N, K = 64, 256
+    W = torch.randn(N, K, generator=g)
+    nrec = (N // 16) * (K // 128) * 32
+    got = {}
+    for share in (0.0, 0.5, 1.0):
+        r = EN.encode_nested(W, seed=3, interleave=True, share4=share)
+        p = O.Plane(N, K, u32(r["base"]).reshape(-1, 4), p3=O.unpack_words(r["p3"].numpy(), nrec, 64), d3=u32(r["d3"]),
+                    p4n=O.unpack_words(r["p4n"].numpy(), nrec, 64), d4n=u32(r["d4n"]))
+        assert same_f16(O.dense_W(p, 3, nested=True), r["Q3"].half().numpy()) == 0
+        assert same_f16(O.dense_W(p, 4, nested="interleave"), r["Q4n"].half().numpy()) == 0
+        got[share] = tuple(float((r[k] - r["target"]).square().mean()) for k in ("Q", "Q3", "Q4n", "Q4"))
+    d2, d3, d4n, d4w = got[0.0]
+    assert abs(d3 / 0.018747 - 1) < 0.08 and abs(d4w / 0.004729 - 1) < 0.08
+    assert 0.019 < d4n < 0.023                                    # a one-bit fit with eight steps of memory: not better than level 3
+    assert got[1.0][2] == got[1.0][3] and abs(got[1.0][1] / d2 - 1) < 0.03          # all units joint: level 4 = wide plane, level 3 ~ base
+    assert got[0.5][1] > d3 and got[0.5][2] < d4n and got[0.5][2] < got[0.5][1]     # half and half: monotone 2 -> 3 -> 4 again
+    print("N(0,1) distortion at levels 2 / 3 / nested 4 / wide 4 by share4:", {k: tuple(round(x, 5) for x in v) for k, v in got.items()})
+
+
 def test_encode_decode_round_trip_through_the_oracle():
     g = torch.Generator().manual_seed(2)
     N, K = 128, 128

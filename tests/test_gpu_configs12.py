@@ -66,6 +66,39 @@ def test_config1_encode_decode_gemv():
         print("config 1 level %d: dequant bit-exact, GEMV rel err %.1e, vs unquantised W x %.3f" % (level, rel_err(y, want), rel_err(y, exact)))
 
 
+def test_interleaved_two_plane_fit_decodes_bit_for_bit():
+    """encode_nested(interleave=True) run on the GPU: base + P3 at level 3 and base + P3, P4 interleaved (window code 12) at
+    level 4, from ONE slot buffer that holds P3's records followed by P4's (what a 2 -> 3 -> 4 promotion fills in two uploads):
+    the HIP decoder reproduces the encoder's matrices bit for bit and the fused GEMV agrees with the oracle's product"""
+    N, K = 256, 256
+    g = torch.Generator().manual_seed(4)
+    W = torch.randn(N, K, generator=g)
+    r = EN.encode_nested(W.to(DEV), seed=2, interleave=True, share4=0.5)
+    H, I = K, N // 2
+    ex = _Ex()
+    ex.H, ex.I, ex.nested, ex.lr, ex.l4code = H, I, True, None, F.CODE_L4B
+    ex.gu = EN.EncodedProj(N, K, r["base"], r["p3"], r["d3"], p4n=r["p4n"], d4n=r["d4n"])
+    zd = F.proj_sizes(H, I)
+    zeros = lambda n: torch.zeros(n, dtype=torch.int32, device=DEV)
+    unit_words = torch.ones(zd["S"] * zd["C"], dtype=torch.int32, device=DEV)
+    ex.dn = EN.EncodedProj(H, I, zeros(zd["base"] // 4), zeros(zd["nrec_r"] * 2), unit_words, p4n=zeros(zd["nrec_r"] * 2), d4n=unit_words)
+    ex.signs = torch.ones(2 * H + 3 * I + H, dtype=torch.float16, device=DEV)
+    L = M.MoELayer(1, H, I, Bmax=4, topk=1)
+    x = (torch.randn(4, K, generator=g) * 0.3).half().to(DEV)
+    xr = O.wht(x.float().cpu().numpy()).astype(np.float16).astype(np.float64)
+    errs = {}
+    for level, key in ((2, "Q"), (3, "Q3"), (4, "Q4n")):
+        L.set(0, ex, level)
+        assert int(L.table[0, 10]) == (10 if level == 3 else 12)
+        Wq = M.dense_W(ex, 0, level).cpu().numpy()
+        assert same_f16(Wq, r[key].half().cpu().numpy()) == 0
+        raw = M.proj_gemv(L, x).cpu().numpy()
+        assert rel_err(raw, xr @ Wq.astype(np.float64).T) < 1e-4
+        errs[level] = float((r[key] - r["target"]).square().mean())
+    assert errs[4] < errs[3] < errs[2]                            # with half the units fitted jointly the levels refine in order
+    print("interleaved two-plane fit (share4 = 0.5): distortion at levels 2 / 3 / 4 = %.4f / %.4f / %.4f" % (errs[2], errs[3], errs[4]))
+
+
 def test_hessian_aware_fit_on_the_gpu_decodes_bit_for_bit():
     """encode_ldlq run on the GPU (256 x 256 weight, activations with shared strong directions): its three matrices are what
     the HIP decoder reproduces from its planes, and the expected output error is below the H-agnostic fit's at every level"""
