@@ -55,7 +55,8 @@ int nq_pf_decode(const int64_t* table, const int32_t* experts, int G, void* Wgu_
 
 /* One decode-path MoE layer call, B <= 8 tokens, B * topk <= 64 picks (reference moe_forward, sm120/nqmoe.cu:858-907).
  * cfg = {cpw, sb, nst, 0}: k-slice = cpw * nst chunks of 128 columns per block; sb = 1, 2 or 4 wavefronts per block (each
- * wavefront decodes two 16-row strips, so sb = 4 covers the reference's largest block of 128 rows); the 4th entry
+ * wavefront decodes two 16-row strips, so sb = 4 covers the reference's largest block of 128 rows); sb must divide N / 32 (and I / 32
+ * for gate|up); the 4th entry
  * (persistent mode) must be 0. Workspaces: acc_gu / acc_d hold k-slice partial sums (plain stores, no float atomics):
  * acc_gu >= (H/128/(cpw*nst)) * B*topk * 2I floats, acc_d >= (I/128/(cpw*nst)) * B*topk * H floats, h >= B*topk * I
  * halfs; cnt_gu >= B*topk * I/128 and cnt_d >= H/128 int32 arrival counters, zero on entry and zero again on exit (the
@@ -137,6 +138,14 @@ typedef struct NqMoeArgs
     const int32_t* mb_seq;
     int32_t* mb_applied;
     int32_t* mb_applied_host; /* [host-mapped], may be NULL */
+    int32_t hoist_value_map;  /* 0 (the default): every decoded weight is rounded to fp16 before it is multiplied, as the reference's kernel
+                                 and its dense decoder do; results are within 5e-5 of the float64 layer over the exact fp16 weights.
+                                 1: runs at level 2 whose row has no sign plane and is of the common kind (common_rows = 1) multiply the
+                                 integers 1024 + S and apply the value map A (.) + B once to each sum (the reference's "RM_P RAW" affine
+                                 hoisting, threads/15-level4-decode/REPORT.md:40,42,66): one vector instruction fewer per weight pair,
+                                 the weights are NOT rounded to fp16, and the results move ~2e-4 (relative l2) from the exact form's --
+                                 inside the layer's 1e-3 tolerance. nq_dequant is never affected. */
+    int32_t reserved_;
 } NqMoeArgs;
 #define NQ_ROUTE_WS_BYTES 32768
 int nq_moe_forward(const NqMoeArgs* args, void* stream);

@@ -25,7 +25,7 @@ class NqMoeArgs(C.Structure):
                 ("common_rows", C.c_int32), ("G", C.c_int32),
                 ("route_ws", C.c_void_p), ("route_ws_bytes", C.c_int64), ("xrot", C.c_void_p), ("xrot_elems", C.c_int64),
                 ("mb_table", C.c_void_p), ("mb_stage", C.c_void_p), ("mb_seq", C.c_void_p), ("mb_applied", C.c_void_p),
-                ("mb_applied_host", C.c_void_p)]
+                ("mb_applied_host", C.c_void_p), ("hoist_value_map", C.c_int32), ("reserved_", C.c_int32)]
 
 
 ROUTE_WS_BYTES = 32768          # NQ_ROUTE_WS_BYTES

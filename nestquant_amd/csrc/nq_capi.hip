@@ -119,8 +119,8 @@ static int moe_args(const char* who, const NqMoeArgs* p, bool own_ws, MoeArgs& a
         const int N = mode == 0 ? 2 * p->I : p->H, K = mode == 0 ? p->H : p->I, C = K / 128;
         NQ_REQUIRE(cf[0] >= 1 && cf[1] >= 1 && cf[2] >= 1 && cf[3] == 0, "bad cfg: {%d,%d,%d,%d} (cpw, sb, nst >= 1; persistent mode is not implemented)", cf[0], cf[1], cf[2], cf[3]);
         const int NC = cf[0] * cf[2], SB = cf[1];
-        NQ_REQUIRE(C % NC == 0 && (SB == 1 || SB == 2 || SB == 4) && NC <= 48,
-                   "bad cfg: k-slice %d chunks of %d, %d wavefronts per block for N=%d (sb must be 1, 2 or 4)", NC, C, SB, N);
+        NQ_REQUIRE(C % NC == 0 && (SB == 1 || SB == 2 || SB == 4) && NC <= 48 && (N / 32) % SB == 0 && (mode == 1 || (p->I / 32) % SB == 0),
+                   "bad cfg: k-slice %d chunks of %d, %d wavefronts per block for N=%d (sb must be 1, 2 or 4 and divide N / 32, for gate|up also I / 32)", NC, C, SB, N);
         const int64_t need = (int64_t)(C / NC) * S * N, have = mode == 0 ? p->acc_gu_elems : p->acc_d_elems;
         NQ_REQUIRE(!own_ws || have >= need, "workspace too small: %s holds %lld floats, needs %lld", mode == 0 ? "acc_gu" : "acc_d", (long long)have, (long long)need);
     }
@@ -150,6 +150,8 @@ static int moe_args(const char* who, const NqMoeArgs* p, bool own_ws, MoeArgs& a
         NQ_REQUIRE((const int64_t*)p->mb_table == p->table, "%s: the mailbox must be the one of the table the call reads", who);
         a.mb_table = p->mb_table; a.mb_stage = p->mb_stage; a.mb_seq = p->mb_seq; a.mb_applied = p->mb_applied; a.mb_applied_host = p->mb_applied_host;
     }
+    NQ_REQUIRE(p->hoist_value_map == 0 || p->hoist_value_map == 1, "%s: hoist_value_map=%d (0 or 1)", who, p->hoist_value_map);
+    a.hoist = p->hoist_value_map;
     NQ_REQUIRE(p->common_rows == 0 || p->common_rows == 1, "%s: common_rows=%d (0 or 1)", who, p->common_rows);
     a.common_rows = p->common_rows;
     NQ_REQUIRE(p->G == 0 || p->G == 4 || p->G == 2, "%s: G=%d (rings of 4 lanes, or 2)", who, p->G);

@@ -281,7 +281,9 @@ __device__ __forceinline__ uint32_t weight_pair(const uint32_t* wb, const uint32
 // from the one that needs its result. The hash multiplies are volatile asm: the compiler keeps them in this order and fits
 // the rest around them (measured at two wavefronts per SIMD: 2.39 -> 2.02 ns per instruction; at four 2.03 -> 1.85). Values
 // and roundings are those of weight_pair.
-template <bool RES, int CODE, int JA, int JB, int BK = 0>
+// RAW: stop before the value map and hand out the fp16 pairs (1024 + S) or (1024 + F) themselves -- exact integers -- for a
+// caller that applies the affine map to its accumulated products instead of to every weight (gemv_chunks<..., RAW>).
+template <bool RES, int CODE, int JA, int JB, int BK = 0, bool RAW = false>
 __device__ __forceinline__ void weight_pairs2(const uint32_t* wb, const uint32_t* wr, const FoldK& k, uint32_t& ua, uint32_t& ub)
 {
     constexpr int B0 = Rec<BK>::off(JA), B1 = Rec<BK>::off(JA + 8), B2 = Rec<BK>::off(JB), B3 = Rec<BK>::off(JB + 8);
@@ -292,7 +294,8 @@ __device__ __forceinline__ void weight_pairs2(const uint32_t* wb, const uint32_t
         const uint32_t x0 = times_hash(y0), x1 = times_hash(y1), x2 = times_hash(y2), x3 = times_hash(y3);
         const uint32_t ta = __builtin_amdgcn_sad_u8(x0, 0u, 0x64006400u), tb = __builtin_amdgcn_sad_u8(x2, 0u, 0x64006400u);
         const uint32_t ca = __builtin_amdgcn_sad_hi_u8(x1, 0u, ta), cb = __builtin_amdgcn_sad_hi_u8(x3, 0u, tb);
-        ua = pk_fma(ca, k.A2, k.C2); ub = pk_fma(cb, k.A2, k.C2);
+        if constexpr (RAW) { ua = ca; ub = cb; }
+        else { ua = pk_fma(ca, k.A2, k.C2); ub = pk_fma(cb, k.A2, k.C2); }
     }
     else
     {
@@ -306,7 +309,8 @@ __device__ __forceinline__ void weight_pairs2(const uint32_t* wb, const uint32_t
         t0 = __builtin_amdgcn_udot4(v0, k.Nrep, t0, false); t1 = __builtin_amdgcn_udot4(v1, k.Nrep, t1, false);
         t2 = __builtin_amdgcn_udot4(v2, k.Nrep, t2, false); t3 = __builtin_amdgcn_udot4(v3, k.Nrep, t3, false);
         const uint32_t ca = __builtin_amdgcn_perm(t1, t0, 0x06050201u), cb = __builtin_amdgcn_perm(t3, t2, 0x06050201u);
-        ua = pk_fma(ca, k.A2, k.C2); ub = pk_fma(cb, k.A2, k.C2);
+        if constexpr (RAW) { ua = ca; ub = cb; }
+        else { ua = pk_fma(ca, k.A2, k.C2); ub = pk_fma(cb, k.A2, k.C2); }
     }
 }
 

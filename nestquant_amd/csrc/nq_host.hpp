@@ -38,6 +38,7 @@ struct MoeArgs
                                       // 512-wide rotation the down launch's staging does the gate|up finisher (set by launch_moe)
     RouteWs* route;                   // NQ_ROUTE_WS_BYTES of device memory: what the routing launch hands to the projection launches
     _Float16* xrot;                   // [B * topk][2][H] fp16: rotated activations of every active pick (gate, up), B-operand order
+    int hoist;                        // NqMoeArgs::hoist_value_map: level-2 runs without a sign plane apply the value map to the sums
     int mb_apply;                     // this projection launch (the call's last) carries the block that applies the mailbox (set by launch_moe)
     int64_t* mb_table; const int64_t* mb_stage; const int32_t* mb_seq; int32_t* mb_applied; int32_t* mb_applied_host;
                                       // mailbox of the call (mb_table == nullptr: none): applied by the last projection launch, published by the next call's routing launch

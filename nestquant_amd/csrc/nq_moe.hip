@@ -631,7 +631,11 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
         const float nan = __builtin_nanf("");
         acc[0] = float4_t{nan, nan, nan, nan}; acc[1] = acc[0];
     }
-    else if (R.level == 2) gemv_chunks<false, 0, 0, false>(P, L, NC, acc, nb0);
+    else if (R.level == 2)
+    {
+        if (a.hoist && P.var == nullptr) gemv_chunks<false, 0, 0, false, true>(P, L, NC, acc, nb0);   // block-uniform: the caller's option
+        else gemv_chunks<false, 0, 0, false>(P, L, NC, acc, nb0);
+    }
     else dispatch_code(P.code, [&](auto tag) { gemv_chunks<true, decltype(tag)::value, 0, false>(P, L, NC, acc, nb0); });
 
     __builtin_amdgcn_s_setprio(3);                               // the tail is a chain of latencies: nothing should wait behind decoders

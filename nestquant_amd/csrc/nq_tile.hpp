@@ -66,13 +66,13 @@ __device__ __forceinline__ int bop_index(int c)
 }
 
 // A operand of MFMA (MM, RHO): rows g + 8 RHO, columns of t = 2 MM and 2 MM + 1
-template <bool RES, int CODE, int MM, int RHO, int BK = 0>
+template <bool RES, int CODE, int MM, int RHO, int BK = 0, bool RAW = false>
 __device__ __forceinline__ half8_t a_operand(const uint32_t* wb, const uint32_t* wr, const FoldK& k)
 {
     constexpr int J = 16 * MM + 2 * RHO;
     uint32_t u[4];
-    weight_pairs2<RES, CODE, J + 0, J + 1, BK>(wb, wr, k, u[0], u[1]);
-    weight_pairs2<RES, CODE, J + 4, J + 5, BK>(wb, wr, k, u[2], u[3]);
+    weight_pairs2<RES, CODE, J + 0, J + 1, BK, RAW>(wb, wr, k, u[0], u[1]);
+    weight_pairs2<RES, CODE, J + 4, J + 5, BK, RAW>(wb, wr, k, u[2], u[3]);
     return __builtin_bit_cast(half8_t, *(u32x4*)u);
 }
 
@@ -158,9 +158,18 @@ __device__ __forceinline__ void gemv_chunks_masked(const Planes& P, const LaneCt
 }
 
 // MASKOK = false leaves the mask-mode loop out (the caller has made sure that P.flags is null)
-template <bool RES, int CODE, int BK = 0, bool MASKOK = true>
+// RAW (level 2 without a sign plane only: one affine map for the whole plane): the MFMAs multiply the integers 1024 + S, exact in
+// fp16, and the value map w = A (1024 + S) + B is applied once to the sums: sum_k w_k x_k = A sum_k (1024 + S_k) x_k + B sum_k x_k,
+// with sum_k x_k from one more MFMA per operand against a row of ones. That removes the packed FMA of every weight pair (32 of the
+// loop's ~276 vector instructions per chunk) and, with it, the rounding of each weight to fp16: the result is that of the
+// UNROUNDED weights, ~2e-4 (relative, l2) from the product with the exact fp16 weights that the other form and the reference
+// compute -- inside the layer's 1e-3, outside the 5e-5 that the exact form holds, hence an option the caller has to ask for.
+template <bool RES, int CODE, int BK = 0, bool MASKOK = true, bool RAW = false>
 __device__ __forceinline__ void gemv_chunks(const Planes& P, const LaneCtx& L, int NC, float4_t* acc, u32x4 nb)
 {
+    static_assert(!RAW || (!RES && BK == 0), "the hoisted value map is built for the level-2 loop");
+    float4_t accx = {0.f, 0.f, 0.f, 0.f};
+    const half8_t ones = {(_Float16)1, (_Float16)1, (_Float16)1, (_Float16)1, (_Float16)1, (_Float16)1, (_Float16)1, (_Float16)1};
     if constexpr (RES && MASKOK)
         if (P.flags) { gemv_chunks_masked<CODE, BK>(P, L, NC, acc, nb); return; }     // block-uniform
     constexpr int NW = RES ? Rec<CODE>::NW : 1;
@@ -195,9 +204,20 @@ __device__ __forceinline__ void gemv_chunks(const Planes& P, const LaneCtx& L, i
         static_for<4>([&](auto mm) {
             constexpr int MM = decltype(mm)::value;
             const half8_t b = *(const half8_t*)(xp + MM * 64);
-            acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_operand<RES, CODE, MM, 0, BK>(wb, wr, k), b, acc[0], 0, 0, 0);
-            acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_operand<RES, CODE, MM, 1, BK>(wb, wr, k), b, acc[1], 0, 0, 0);
+            acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_operand<RES, CODE, MM, 0, BK, RAW>(wb, wr, k), b, acc[0], 0, 0, 0);
+            acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_operand<RES, CODE, MM, 1, BK, RAW>(wb, wr, k), b, acc[1], 0, 0, 0);
+            if constexpr (RAW) accx = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, b, accx, 0, 0, 0);
         });
+    }
+    if constexpr (RAW)
+    {   // every row of accx holds the token's sum of x over the k-slice; A and B as the fp32 values of the fp16 constants
+        const float A = 0.00676727294921875f /* fp16 0x1eee = 1774 / 2^18 */, B = -10.3828125f /* fp16 0xc931 */;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+        {
+            acc[0][i] = __builtin_fmaf(A, acc[0][i], B * accx[i]);
+            acc[1][i] = __builtin_fmaf(A, acc[1][i], B * accx[i]);
+        }
     }
 }
 

@@ -111,6 +111,9 @@ def test_argument_checks_run_before_any_device_work():
     a.mb_table = None; a.G = 3
     a.G = 0; a.common_rows = 2
     assert L.nq_moe_forward(C.byref(a), None) != 0 and "common_rows" in err()
+    a.common_rows = 0; a.hoist_value_map = 2
+    assert L.nq_moe_forward(C.byref(a), None) != 0 and "hoist_value_map" in err()
+    a.hoist_value_map = 0
     assert L.nq_pf_plan(base, 256, 0, 1024, base, 256, None, 0, 0, None) != 0 and "cap" in err()
     assert L.nq_pf_plan(base, 256, 0, 1024, base + 4, 512, None, 0, 0, None) != 0 and "aligned" in err()
     assert L.nq_pf_gemm(base, base, 1, 48, 0, base, base, base, 4, 256, 256, None, None) != 0 and "tile height" in err()

@@ -119,6 +119,43 @@ def test_interleaved_two_plane_level4_in_decode_and_prefill():
     assert rel_err(L(x[:1], sel1, rw1).cpu().numpy(), oracle_layer(planes, levels, signs, x[:1], sel1, rw1)) > 1e-2
 
 
+def test_hoisted_value_map_is_an_option_with_its_own_tolerance():
+    """hoist=True: level-2 runs without a sign plane multiply the integers 1024 + S and apply A (.) + B to the sums, so their
+    weights are not rounded to fp16: within 6e-4 of the float64 oracle over the exact fp16 weights (the default holds 5e-5) and
+    within 1e-3 of the fp32 pipeline; runs at other levels or with a sign plane are not touched (same bits as the default)"""
+    H, I, NE = 1024, 512, 6
+    ex = experts_on_gpu(H, I, NE, 810, nested_ids=(3, 4), var_ids=(2,))
+    planes = [(oracle_plane(e.gu), oracle_plane(e.dn), e.nested) for e in ex]
+    signs = [e.signs.numpy() for e in ex]
+    levels = [2, 2, 2, 3, 4, 4]
+    to_dev(ex)
+    L = M.MoELayer(NE, H, I, Bmax=8, topk=3)
+    for e in range(NE):
+        L.set(e, ex[e], levels[e])
+    g = torch.Generator().manual_seed(12)
+    rng = random.Random(2)
+    worst = 0.0
+    for B in (1, 3, 8):
+        sel, rw = RT.routing_tensors(RT.make_sel(B, range(NE), "recency", p=0.5, rng=rng, topk=3), seed=B)
+        x = (torch.randn(B, H, generator=g) * 0.05).half().to(DEV)
+        y0 = L(x, sel, rw).clone()
+        y1 = L(x, sel, rw, hoist=True).clone()
+        y1b = L(x, sel, rw, hoist=True, out=torch.empty_like(y1), static_ws=True)
+        torch.cuda.synchronize()
+        want = oracle_layer(planes, levels, signs, x, sel, rw)
+        pure = oracle_layer(planes, levels, signs, x, sel, rw, round_acts=False, dtype=np.float32)
+        assert rel_err(y0.cpu().numpy(), want) < 5e-5
+        err = rel_err(y1.cpu().numpy(), want)
+        worst = max(worst, err)
+        assert 1e-6 < err < 6e-4 and rel_err(y1.cpu().numpy(), pure) < 1e-3, (B, err)
+        assert not torch.equal(y0, y1) and torch.equal(y1, y1b)
+    sel = torch.tensor([[2, 3, 4], [5, 4, 2]], device=DEV)        # a sign plane, level 3, level 4: nothing to hoist
+    rw = torch.tensor([[0.5, 0.25, 0.25], [0.3, 0.3, 0.4]], device=DEV).half()
+    x = (torch.randn(2, H, generator=g) * 0.05).half().to(DEV)
+    assert torch.equal(L(x, sel, rw).clone(), L(x, sel, rw, hoist=True))
+    print(f"hoisted value map: worst distance from the float64 oracle {worst:.2e}")
+
+
 def test_golden_layer_fixture(golden_dir):
     """the reference's own moe_ref output on the small golden layer (levels 2/4/4/0, codes 3/7, a sign plane, rw == 0)"""
     z = np.load(f"{golden_dir}/layer_small.npz")
