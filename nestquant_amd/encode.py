@@ -19,6 +19,12 @@ it is not the reference's production encoder. What it restates, in plain torch t
     searched over the reference's twelve block-word candidates (nq_encode.py:186-198, nq_decode.py:158-163) with the
     integer fold itself (sm120/ref15_spec.py:79-90) as the cost, so the chosen word is the best of them for the values
     the decoder really produces.
+  * the input scale of a fit found by the reference's grid search (g_scale_search: coarse grid, fine grid, parabola vertex;
+    threads/05-exl3-harness/harness.py:371-387), for the base plane (folded into su) and the refinement stages;
+  * the two-sided schedule (encode_ldlq2, nq_encode.py:206-339): an output metric beside the input Hessian, both block LDL
+    factored, units fitted along anti-diagonals from the far corner with the errors of the fitted units carried over by both
+    factors, and the reference's inner iterations (accept-if-better tries with the errors fed back inside a chunk);
+  * the second plane of the interleaved two-plane level 4 (window code 12) with the first plane frozen (viterbi_ring_given_p3).
 The reference's encoder depends on exllamav3 1.5.1, which is not available here, so bit parity with it is not claimed;
 the tests pin this encoder by brute force on a small trellis, by decode(encode) self-consistency and by the Gaussian
 distortion the reference reports for this code (MSE 0.068 at 2 bits, threads/03-nested-trellis-code/REPORT.md:21; base +
@@ -251,12 +257,14 @@ def signed32(w):
     return torch.where(w >= 2**31, w - 2**32, w).to(torch.int32)
 
 
-def encode_level2(W, seed=0, chunk=64):
+def encode_level2(W, seed=0, chunk=64, g_scale=False):
     """W [N, K] float (N % 16 == 0, K % 128 == 0; N % 128 == 0 for the output rotation) ->
     dict(base int32 [nrec*4], su fp16 [K], sv fp16 [N], states int64 [units, 8, 256] (ring position order), Q fp32 [N, K])
     with  W ~= D(sv) B_N Q B_K D(su)  and Q the matrix the decoder reproduces bit for bit from `base`."""
     N, K = W.shape
     su, sv, target = prepare(W, seed)
+    if g_scale:                                                  # the fit's input scale from the grid search instead of 1
+        su, target, _ = apply_g_scale(su, target)
     st = viterbi_rings(to_rings(target), 2, chunk)
     base = signed32(lane_records(st, 2).reshape(-1))             # record = (unit, lane 4 g + t4): 4 words
     Q = from_rings(codebook(W.device)[st], N, K)                 # decoded values
@@ -537,6 +545,187 @@ def encode_ldlq(W, H, seed=0, chunk=64, lam=0.3, sigma=0.01, var=False):
                     sign.reshape(-1, 8, 1) if var else None)
     r["proxy"] = {2: proxy_loss(r["Q"], target, Hr), 3: proxy_loss(r["Q3"], target, Hr), 4: proxy_loss(r["Q4"], target, Hr)}
     return r
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# input scale of a trellis fit: grid search
+CB_RMS = 1.24371088              # rms of the codebook's 65536 values (reference nq_encode.py:32)
+
+
+def g_scale_search(rings, K, quantize=None):
+    """The scale s by which rings [T, 256] (Viterbi order does not matter here) are multiplied before the fit so that
+    mean((q(s x) / s - x)^2) is least: a coarse grid 0.1, 0.3 .. 1.9 on every third ring, five points 0.075 apart around the best
+    of them on all rings, then the vertex of the parabola through the best point and its neighbours, at most half a step away
+    (reference threads/05-exl3-harness/harness.py:371-387, after exllamav3's g_scale_search_batch). quantize(x, K) -> values of
+    the fitted code (default: the tail-biting Viterbi over the mul1 codebook). -> (scale >= 0.01, mse at the best grid point)"""
+    if quantize is None:
+        lut = codebook(rings.device)
+        quantize = lambda x, k: lut[viterbi_ring(x, lut, k)]
+
+    def mse(x, s):
+        return float((quantize(x * s, K) / s - x).square().mean())
+    coarse = [0.1 + 0.2 * i for i in range(10)]
+    third = rings[::3]
+    c = min(coarse, key=lambda v: mse(third, v))
+    step = 0.075
+    fine = [c + step * (i - 2) for i in range(5)]
+    m = [mse(rings, v) if v > 0 else float("inf") for v in fine]
+    best = min(range(5), key=lambda i: m[i])
+    shift = 0.0
+    if 0 < best < 4 and m[best - 1] < float("inf"):
+        bend = m[best - 1] - 2 * m[best] + m[best + 1]
+        if bend > 0:
+            shift = max(-0.5, min(0.5, 0.5 * (m[best - 1] - m[best + 1]) / bend))
+    return max(fine[best] + shift * step, 0.01), m[best]
+
+
+def sample_rings(rings, limit=384):
+    """an evenly spaced sample of at most `limit` rings (the reference samples tiles with exllamav3's sample_scale_tiles, which is
+    not available here)"""
+    T = rings.shape[0]
+    return rings if T <= limit else rings[torch.linspace(0, T - 1, limit, device=rings.device).round().long()]
+
+
+def apply_g_scale(su, target, K=2):
+    """the searched scale folded into the fit: the code is fitted to gs * target and the input scale vector carries 1 / gs, so
+    that W ~= D(sv) B Q B D(su) still holds (reference nq_encode.py:175-177: weight *= gs; su /= gs). The target is rebuilt from
+    the fp16-rounded su so that it is exactly what the decoder's scales imply. -> (su fp16, target fp32, gs)"""
+    gs, _ = g_scale_search(sample_rings(to_rings(target)), K)
+    su2 = (su.double() / gs).half()
+    ratio = (su.double() / su2.double()).float()                  # = gs up to the fp16 rounding of every channel's scale
+    return su2, blocked_had(blocked_had(target, 1) * ratio[None, :], 1), gs
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# two-sided LDLQ: an output metric beside the input Hessian, units fitted along anti-diagonals, inner iterations
+def rotated_out_metric(G, sv, sigma=0.03):
+    """second moment of what the layer's output error is weighed with, in the rotated output basis: the output is
+    y = D(sv) B (Q xr), so an error E of Q costs e^T G e with e = D(sv) B E xr, i.e. the metric on the rotated rows is
+    B D(sv) G D(sv) B; then sigma * mean(diag) on the diagonal (the reference builds this with exllamav3's prepare_H_out from
+    G and sv, nq_encode.py:178-183; that function is not available here and this is the form the layer math gives)"""
+    Gs = G.double() * sv.double()[:, None] * sv.double()[None, :]
+    Gr = blocked_had(blocked_had(Gs, 0), 1)
+    return Gr + sigma * Gr.diagonal().mean() * torch.eye(G.shape[0], dtype=torch.float64, device=G.device)
+
+
+def encode_ldlq2(W, H, G, seed=0, chunk=64, lam=0.3, sigma=0.01, sigma_out=0.03, var=False, inner=0, beta=1.0, g_scale=False):
+    """encode_ldlq with a metric on both sides (reference nq_encode.py:206-339, its two-sided schedule): the expected cost of an
+    error E = T - Q of the rotated weight is tr(Go E H' E^T), Go [N, N] the rotated output metric (rotated_out_metric) and H'
+    [K, K] the rotated input Hessian. With H' = Lk Din Lk^T (unit block lower, blocks of 128 columns = a chunk) and
+    Go = Ln Dout Ln^T (blocks of 16 rows = a strip) the cost is the sum over the units (strip c, chunk a) of
+    tr(Dout_c eta Din_a eta^T), eta_ca = block (c, a) of Ln^T E Lk = E_ca + the errors of the units with c' >= c and a' >= a
+    carried over by both factors. So the units are fitted along anti-diagonals from the far corner (largest c + a first), each
+    to its weight plus what the already fitted units pass on, T_ca = W_ca + (Ln^T E Lk)_ca over the fitted units only, and its
+    own fitting error is eta_ca. One error state per level, as in encode_ldlq.
+    inner > 0 (reference :249-258,:271-302): that many further tries per stage inside a unit's chunk. Din_a itself factors
+    with blocks of 16 columns, Din_a = L16 D16 L16^T; a try refits the stage to its target plus beta * (target - the previous
+    try's values) (L16 - I), the errors of the later 16-column groups fed to the earlier ones, and is kept for the units whose
+    local cost tr(Dout eta Din eta^T) it lowers, so the cost never rises.
+    g_scale: search the input scale of the base fit (apply_g_scale) and of the refinement stages (on the first anti-diagonal's
+    residuals) instead of the constants 1 and RES_SCALE.
+    Adds Hr, Go, Din, Dout, eta = {2, 3, 4: fp64 [N, K]}, proxy = {2, 3, 4} and, with inner, n_inner_kept to encode_nested's dict."""
+    N, K = W.shape
+    S, C = N // 16, K // 128
+    dev = W.device
+    su, sv, target = prepare(W, seed)
+    gs = 1.0
+    if g_scale:
+        su, target, gs = apply_g_scale(su, target)
+    Hr = rotated_hessian(H.to(dev), su, sigma)
+    Go = rotated_out_metric(G.to(dev), sv, sigma_out)
+    Lk, Din = block_ldl(Hr, 128)
+    Ln, Dout = block_ldl(Go, 16)
+    U16 = None
+    if inner:
+        U16 = torch.stack([block_ldl(Din[a], 16)[0] for a in range(C)]) - torch.eye(128, dtype=torch.float64, device=dev)
+    Tg = target.double()
+    levels = (2, 3, 4)
+    err = {l: torch.zeros(N, K, dtype=torch.float64, device=dev) for l in levels}     # W - Q of the fitted units
+    eta = {l: torch.zeros(N, K, dtype=torch.float64, device=dev) for l in levels}
+    st2 = torch.empty(S, C, 8, 256, dtype=torch.int64, device=dev)
+    sign = torch.ones(S, C, 8, 1, device=dev)
+    fit = {l: dict(states=torch.empty(S, C, 8, 256, dtype=torch.int64, device=dev), Q=torch.empty(S, C, 8, 256, device=dev),
+                   Mb=torch.empty(S, C, dtype=torch.int64, device=dev), N=torch.empty(S, C, dtype=torch.int64, device=dev)) for l in (3, 4)}
+    Q2u = torch.empty(S, C, 16, 128, device=dev)
+    lut = codebook(dev)
+    kept = 0
+    res_scale = dict(RES_SCALE)
+
+    def units_of(M, cs, as_):                                   # [N, K] -> [T, 16, 128]
+        return M.reshape(S, 16, C, 128).permute(0, 2, 1, 3)[cs, as_]
+
+    def rings_of(U):                                            # [T, 16, 128] -> [T, 8, 256] ring position order
+        flat = U.permute(0, 2, 1).reshape(U.shape[0], 2048)     # [unit, column * 16 + row]
+        return flat[:, ring_index(dev).reshape(-1)].reshape(-1, 8, 256)
+
+    def unit_of_rings(R):                                       # inverse of rings_of
+        flat = torch.empty(R.shape[0], 2048, dtype=R.dtype, device=dev)
+        flat[:, ring_index(dev).reshape(-1)] = R.reshape(R.shape[0], 2048)
+        return flat.reshape(-1, 128, 16).permute(0, 2, 1)
+
+    for s in range(S + C - 2, -1, -1):
+        as_ = torch.arange(max(0, s - (S - 1)), min(C - 1, s) + 1, device=dev)
+        cs = s - as_
+        Tn = len(as_)
+        Da, Do = Din[as_], Dout[cs]
+        lcost = lambda E: ((Do @ E.double() @ Da) * E.double()).sum((1, 2))            # tr(Dout eta Din eta^T) per unit
+        Tl = {l: units_of(Tg + Ln.T @ err[l] @ Lk, cs, as_) for l in levels}           # unfitted units contribute nothing: their err is 0
+
+        def fit_base(tb):
+            sa, sg = base_rings(rings_of(tb.float()).reshape(-1, 256), chunk, var)
+            sa, sg = sa.reshape(Tn, 8, 256), sg.reshape(Tn, 8, 1)
+            return sa, sg, unit_of_rings(lut[sa] * sg)
+        tb = (1 - lam) * Tl[2] + lam * Tl[4]
+        sa, sg, q2 = fit_base(tb)
+        if inner:
+            c_best, cur = lcost(tb - q2), q2
+            for _ in range(inner):
+                na, ng, nq = fit_base(tb + beta * (tb - cur.double()) @ U16[as_])
+                c = lcost(tb - nq); w = c < c_best
+                sa[w], sg[w], q2[w] = na[w], ng[w], nq[w]
+                c_best = torch.where(w, c, c_best); cur = nq; kept += int(w.sum())
+        st2[cs, as_], sign[cs, as_], Q2u[cs, as_] = sa, sg, q2
+        Wu = units_of(Tg, cs, as_)
+
+        def put(M, U):                                          # write units back into [N, K]
+            M.reshape(S, 16, C, 128).permute(0, 2, 1, 3)[cs, as_] = U
+        put(err[2], Wu - q2.double()); put(eta[2], Tl[2] - q2.double())
+        cost = lambda E: lcost(unit_of_rings(E))                  # encode_residual hands over errors in ring order
+        for l in (3, 4):
+            Kb = l - 2
+            if g_scale and s == S + C - 2:                        # first units: search the refinement stage's input scale once
+                rr = (rings_of(Tl[l].float()) * sg - lut[sa]).reshape(-1, 256)
+                rr = rr / rr.square().mean(1, keepdim=True).sqrt().clamp_min(1e-12)
+                res_scale[Kb] = g_scale_search(sample_rings(rr), Kb)[0]
+            tr_l = rings_of(Tl[l].float())
+            e = encode_residual(tr_l, sa, Kb, chunk, cost=cost, sign=sg, scale=res_scale[Kb])
+            if inner:
+                c_best = cost((tr_l - e["Q"]).double()); cur = unit_of_rings(e["Q"])
+                for _ in range(inner):
+                    t_try = Tl[l] + beta * (Tl[l] - cur.double()) @ U16[as_]
+                    n = encode_residual(rings_of(t_try.float()), sa, Kb, chunk, cost=cost, sign=sg, scale=res_scale[Kb])
+                    # the try's block word was fitted to the shifted target: cost it, and refit the word, against the real one
+                    n = encode_residual(tr_l, sa, Kb, chunk, cost=cost, sign=sg, states=n["states"])
+                    c = cost((tr_l - n["Q"]).double()); w = c < c_best
+                    for k in ("states", "Q", "Mb", "N"):
+                        e[k][w] = n[k][w]
+                    c_best = torch.where(w, c, c_best); cur = unit_of_rings(n["Q"]); kept += int(w.sum())
+            for k in ("states", "Q", "Mb", "N"):
+                fit[l][k][cs, as_] = e[k]
+            q = unit_of_rings(e["Q"]).double()
+            put(err[l], Wu - q); put(eta[l], Tl[l] - q)
+    flat = {l: dict(states=f["states"].reshape(-1, 8, 256), Q=f["Q"].reshape(-1, 8, 256), Mb=f["Mb"].reshape(-1), N=f["N"].reshape(-1))
+            for l, f in fit.items()}
+    r = pack_planes(dict(su=su, sv=sv, target=target, Hr=Hr, Go=Go, Din=Din, Dout=Dout, eta=eta, gs=gs, res_scale=res_scale, n_inner_kept=kept),
+                    N, K, st2.reshape(-1, 8, 256), flat, sign.reshape(-1, 8, 1) if var else None)
+    r["proxy"] = {2: proxy_loss2(r["Q"], target, Hr, Go), 3: proxy_loss2(r["Q3"], target, Hr, Go), 4: proxy_loss2(r["Q4"], target, Hr, Go)}
+    return r
+
+
+def proxy_loss2(Q, target, Hr, Go):
+    """tr(Go E H' E^T) / tr(Go T H' T^T) with E = Q - T: the expected weighted output error relative to the output's"""
+    E, T = Q.double() - target.double(), target.double()
+    return float(((Go @ E @ Hr) * E).sum() / ((Go @ T @ Hr) * T).sum())
 
 
 class EncodedProj(Proj):

@@ -248,3 +248,59 @@ def test_ldlq_fit_feeds_errors_forward_and_lowers_the_output_error():
                 p3=O.unpack_words(r["p3"].numpy(), nrec, 64), d3=u32(r["d3"]))
     for level, key in ((2, "Q"), (3, "Q3"), (4, "Q4")):
         assert same_f16(O.dense_W(p, level), r[key].half().numpy()) == 0
+
+
+def test_g_scale_search_grid_and_vertex():
+    """the reference's scale search (threads/05-exl3-harness/harness.py:371-387). With rings of ones the stand-in quantiser sees
+    y = s and returns y (1 + (y - s*)), so mean((q / s - x)^2) = (s - s*)^2 exactly: the coarse grid must pick the right
+    neighbourhood, the fine grid the nearest point, and the parabola's vertex must land on s* itself; a wrong sign of the
+    vertex shift, a swapped neighbour or a wrong step would miss it. Then the real trellis fit on Gaussian rings: the found
+    scale is at least as good as every point of the fine grid around it and as no scaling at all."""
+    ones = torch.ones(9, 256)
+    for target in (0.42, 0.97, 1.33, 1.84):
+        q = lambda y, K, t=target: y * (1 + (y - t))
+        s, m = EN.g_scale_search(ones, 2, q)
+        assert abs(s - target) < 1e-6 and m <= 0.0375 ** 2 + 1e-9, (target, s, m)
+    s, _ = EN.g_scale_search(ones, 2, lambda y, K: y * (1 + (y - 0.004)))          # below the grid: its lowest positive point region
+    assert 0.01 <= s <= 0.1
+    g = torch.Generator().manual_seed(4)
+    w = torch.randn(24, 256, generator=g) * 0.8                   # not unit variance: the search must undo it
+    lut = EN.codebook()
+    mse = lambda v: float((lut[EN.viterbi_ring(w * v, lut, 2)] / v - w).square().mean())
+    s, _ = EN.g_scale_search(w, 2)
+    here = mse(s)
+    assert 1.0 < s < 1.6 and here <= mse(1.0)
+    assert all(here <= mse(s + d) * 1.01 for d in (-0.15, -0.075, 0.075, 0.15))
+    # in units of the data's own rms the found scale is the same whatever the data's size
+    s2, _ = EN.g_scale_search(w * 1.25, 2)
+    assert abs(s2 * 1.25 / s - 1) < 0.06
+
+
+def test_two_sided_ldlq_identity_and_gain():
+    """encode_ldlq2 on one chunk of 128 columns and eight strips, activations and output weights with a few strong directions.
+    Pinned: tr(Go E H' E^T) = sum over the units of tr(Dout eta Din eta^T) with eta each unit's own fitting error against the
+    target it was given -- exact for any quantiser, broken by a wrong sign, a transposed factor or a wrong order of the units;
+    the unit in the far corner gets no feedback, so it is fitted as the plain encoder fits it. The packed planes decode bit for
+    bit through the oracle. (The gain over the one-sided and the plain fit is measured on the GPU, tests/test_gpu_configs12.py.)"""
+    g = torch.Generator().manual_seed(5)
+    N, K = 128, 128
+    W = torch.randn(N, K, generator=g)
+    X = torch.randn(4096, 4, generator=g) @ torch.randn(4, K, generator=g) * 1.5 + torch.randn(4096, K, generator=g)
+    Y = torch.randn(4096, 3, generator=g) @ torch.randn(3, N, generator=g) * 1.5 + torch.randn(4096, N, generator=g)
+    H, G = (X.T @ X / 4096).double(), (Y.T @ Y / 4096).double()
+    r = EN.encode_ldlq2(W, H, G, seed=3)
+    T = r["target"].double()
+    S = N // 16
+    for lvl, key in ((2, "Q"), (3, "Q3"), (4, "Q4")):
+        E = T - r[key].double()
+        lhs = float(((r["Go"] @ E @ r["Hr"]) * E).sum())
+        eta = r["eta"][lvl].reshape(S, 16, 128)
+        rhs = float(sum(((r["Dout"][c] @ eta[c] @ r["Din"][0]) * eta[c]).sum() for c in range(S)))
+        assert abs(lhs / rhs - 1) < 1e-9, (lvl, lhs, rhs)
+    last = EN.to_rings(r["target"][N - 16:].contiguous())         # strip 7: nothing was fitted before it
+    assert torch.equal(EN.viterbi_rings(last, 2), r["states"][S - 1].reshape(8, 256))
+    nrec = (N // 16) * (K // 128) * 32
+    p = O.Plane(N, K, u32(r["base"]).reshape(-1, 4), rk=0, res=O.unpack_words(r["p4"].numpy(), nrec, 128), d4=u32(r["d4"]),
+                p3=O.unpack_words(r["p3"].numpy(), nrec, 64), d3=u32(r["d3"]))
+    for level, key in ((2, "Q"), (3, "Q3"), (4, "Q4")):
+        assert same_f16(O.dense_W(p, level), r[key].half().numpy()) == 0
