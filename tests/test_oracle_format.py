@@ -10,7 +10,7 @@ from oracle import nq_oracle as O
 
 def test_record_bits_table():
     # reference threads/13-moe-layer-kernel/INTEGRATION.md:43-44 and sm120/NQ_RES_V2.md:24
-    want = {0: 128, 1: 112, 2: 160, 3: 144, 4: 192, 5: 96, 6: 124, 7: 148, 8: 120, 9: 164, 10: 64, 11: 128}
+    want = {0: 128, 1: 112, 2: 160, 3: 144, 4: 192, 5: 96, 6: 124, 7: 148, 8: 120, 9: 164, 10: 64, 11: 128, 12: 128}
     assert {c: O.rbits(c) for c in O.RKP} == want
 
 
