@@ -813,7 +813,7 @@ def main():
         e1.record(s)
     torch.cuda.synchronize()
     dt = e0.elapsed_time(e1) / 1e3
-    # (3) the same steps with the opt-in hoisted value map (level-2 experts multiply unrounded weights): its own figure and its
+    # (3) the same steps with the opt-in hoisted value map (unrounded weights): its own figure and its
     # distance from the default's outputs, never the headline
     hoisted[0] = True
     h_full, h_rem = capture(R), (capture(K % R) if K % R else None)
@@ -939,8 +939,8 @@ def main():
         "ms_per_step_wall": round(dt_wall / K * 1e3, 5), "value_wall": round(nbytes / dt_wall / 1e9, 1),
         "hoisted_value_map": {"us_per_layer": round(dt_h / K * 1e6, 2), "GBps": round(nbytes / dt_h / 1e9, 1),
                               "rel_l2_from_default_max": float(f"{rel_h.max().item():.2e}"), "rel_l2_from_default_mean": float(f"{rel_h.mean().item():.2e}"),
-                              "note": "opt-in (NqMoeArgs.hoist_value_map): level-2 experts multiply the integers 1024 + S and apply the value map "
-                                      "to the sums, so their weights are not rounded to fp16; same steps, same timing method; not the headline"},
+                              "note": "opt-in (NqMoeArgs.hoist_value_map): the MFMAs multiply the integers 1024 + S / 1024 + F and the value map is "
+                                      "applied to the sums, so no weight is rounded to fp16; same steps, same timing method; not the headline"},
         "us_per_layer_median": round(blocks[len(blocks) // 2], 2), "us_per_layer_min": round(blocks[0], 2),
         "us_layer_call_without_mailbox_median": round(call_blocks[len(call_blocks) // 2], 2), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",

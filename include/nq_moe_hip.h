@@ -140,11 +140,13 @@ typedef struct NqMoeArgs
     int32_t* mb_applied_host; /* [host-mapped], may be NULL */
     int32_t hoist_value_map;  /* 0 (the default): every decoded weight is rounded to fp16 before it is multiplied, as the reference's kernel
                                  and its dense decoder do; results are within 5e-5 of the float64 layer over the exact fp16 weights.
-                                 1: runs at level 2 whose row has no sign plane and is of the common kind (common_rows = 1) multiply the
-                                 integers 1024 + S and apply the value map A (.) + B once to each sum (the reference's "RM_P RAW" affine
+                                 1: runs whose row has no sign plane and is of the common kind (common_rows = 1) multiply the integers
+                                 1024 + S (level 2) or 1024 + F (levels 3, 4) and apply the value map to the sums -- once per k-slice
+                                 at level 2, where A and B are global, per unit at levels 3 / 4 (the reference's "RM_P RAW" affine
                                  hoisting, threads/15-level4-decode/REPORT.md:40,42,66): one vector instruction fewer per weight pair,
-                                 the weights are NOT rounded to fp16, and the results move ~2e-4 (relative l2) from the exact form's --
-                                 inside the layer's 1e-3 tolerance. nq_dequant is never affected. */
+                                 the weights are NOT rounded to fp16, and the layer output moves 4.6e-4 (relative l2, mean; 6.3e-4 at
+                                 most over 64 routings of the full shape) from the exact form's -- inside the layer's 1e-3 tolerance,
+                                 with little room to spare. nq_dequant is never affected. */
     int32_t reserved_;
 } NqMoeArgs;
 #define NQ_ROUTE_WS_BYTES 32768

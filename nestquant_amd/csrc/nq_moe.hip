@@ -636,6 +636,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
         if (a.hoist && P.var == nullptr) gemv_chunks<false, 0, 0, false, true>(P, L, NC, acc, nb0);   // block-uniform: the caller's option
         else gemv_chunks<false, 0, 0, false>(P, L, NC, acc, nb0);
     }
+    else if (a.hoist && P.var == nullptr) dispatch_code(P.code, [&](auto tag) { gemv_chunks<true, decltype(tag)::value, 0, false, true>(P, L, NC, acc, nb0); });
     else dispatch_code(P.code, [&](auto tag) { gemv_chunks<true, decltype(tag)::value, 0, false>(P, L, NC, acc, nb0); });
 
     __builtin_amdgcn_s_setprio(3);                               // the tail is a chain of latencies: nothing should wait behind decoders

@@ -167,8 +167,14 @@ __device__ __forceinline__ void gemv_chunks_masked(const Planes& P, const LaneCt
 template <bool RES, int CODE, int BK = 0, bool MASKOK = true, bool RAW = false>
 __device__ __forceinline__ void gemv_chunks(const Planes& P, const LaneCtx& L, int NC, float4_t* acc, u32x4 nb)
 {
-    static_assert(!RAW || (!RES && BK == 0), "the hoisted value map is built for the level-2 loop");
+    static_assert(!RAW || BK == 0, "the hoisted value map is built for base window code 0");
     float4_t accx = {0.f, 0.f, 0.f, 0.f};
+    // RAW at levels 3 / 4: the value map differs from unit to unit, w = A'_u (1024 + F) + C_u, so it is applied chunk by chunk: the
+    // chunk's integer products go to accumulators of their own (zero at the chunk's start) and enter the running sums times A'_u;
+    // C_u sum_k x_k comes from two more MFMAs per operand whose A operand is C_u in every place (the rows a lane decodes and the
+    // rows it supplies to the MFMA are the same, so its own unit's C_u is the right one). The accumulator rows a lane HOLDS belong
+    // to the strip (lane >> 5), whose A' it fetches from a lane that decodes that strip.
+    const int lane_of_out_strip = (int)((threadIdx.x & 0x37u) | ((threadIdx.x >> 2) & 8u));
     const half8_t ones = {(_Float16)1, (_Float16)1, (_Float16)1, (_Float16)1, (_Float16)1, (_Float16)1, (_Float16)1, (_Float16)1};
     if constexpr (RES && MASKOK)
         if (P.flags) { gemv_chunks_masked<CODE, BK>(P, L, NC, acc, nb); return; }     // block-uniform
@@ -201,15 +207,38 @@ __device__ __forceinline__ void gemv_chunks(const Planes& P, const LaneCtx& L, i
         }
         else k = consts_l2(sgm);
         const char* xp = L.xs + c * L.xstep;
-        static_for<4>([&](auto mm) {
-            constexpr int MM = decltype(mm)::value;
-            const half8_t b = *(const half8_t*)(xp + MM * 64);
-            acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_operand<RES, CODE, MM, 0, BK, RAW>(wb, wr, k), b, acc[0], 0, 0, 0);
-            acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_operand<RES, CODE, MM, 1, BK, RAW>(wb, wr, k), b, acc[1], 0, 0, 0);
-            if constexpr (RAW) accx = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, b, accx, 0, 0, 0);
-        });
+        if constexpr (RAW && RES)
+        {
+            float4_t c0 = {0.f, 0.f, 0.f, 0.f}, c1 = {0.f, 0.f, 0.f, 0.f};
+            const u32x4 cu = {k.C2, k.C2, k.C2, k.C2};
+            const half8_t cop = __builtin_bit_cast(half8_t, cu);
+            static_for<4>([&](auto mm) {
+                constexpr int MM = decltype(mm)::value;
+                const half8_t b = *(const half8_t*)(xp + MM * 64);
+                c0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_operand<RES, CODE, MM, 0, BK, true>(wb, wr, k), b, c0, 0, 0, 0);
+                c1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_operand<RES, CODE, MM, 1, BK, true>(wb, wr, k), b, c1, 0, 0, 0);
+                acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(cop, b, acc[0], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(cop, b, acc[1], 0, 0, 0);
+            });
+            const float Amine = (float)__builtin_bit_cast(_Float16, (uint16_t)(k.A2 & 0xFFFFu));
+            const float Aout = __shfl(Amine, lane_of_out_strip);
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+            {
+                acc[0][i] = __builtin_fmaf(Aout, c0[i], acc[0][i]);
+                acc[1][i] = __builtin_fmaf(Aout, c1[i], acc[1][i]);
+            }
+        }
+        else
+            static_for<4>([&](auto mm) {
+                constexpr int MM = decltype(mm)::value;
+                const half8_t b = *(const half8_t*)(xp + MM * 64);
+                acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_operand<RES, CODE, MM, 0, BK, RAW>(wb, wr, k), b, acc[0], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_operand<RES, CODE, MM, 1, BK, RAW>(wb, wr, k), b, acc[1], 0, 0, 0);
+                if constexpr (RAW) accx = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, b, accx, 0, 0, 0);
+            });
     }
-    if constexpr (RAW)
+    if constexpr (RAW && !RES)
     {   // every row of accx holds the token's sum of x over the k-slice; A and B as the fp32 values of the fp16 constants
         const float A = 0.00676727294921875f /* fp16 0x1eee = 1774 / 2^18 */, B = -10.3828125f /* fp16 0xc931 */;
 #pragma unroll

@@ -232,8 +232,9 @@ class MoELayer:
         launch of the next call publishes `applied_host`. Rows that land while this call runs are used, and reported done, from
         the next call on -- when `mailbox.apply()` at the head of the next call would have done both. After the last call of
         a sequence one `mailbox.apply()` publishes what that call applied.
-        hoist: level-2 experts (without a sign plane, rows of the common kind) multiply the unrounded integers 1024 + S and apply the
-        value map to the sums: a few percent faster, ~2e-4 from the default's result (NqMoeArgs.hoist_value_map; off by default).
+        hoist: experts without a sign plane (rows of the common kind) multiply the integers 1024 + S / 1024 + F and apply the value
+        map to the sums, so no weight is rounded to fp16: ~4 % faster, ~5e-4 from the default's result (NqMoeArgs.hoist_value_map;
+        off by default).
         static_ws: go through nq_moe_forward_static, which ignores this layer's workspaces and uses the library's built-in
         device scratch instead (for callers that must not allocate; calls on one GPU then share that scratch)."""
         assert x.dtype in _DT_IN and rw.dtype in _DT_IN and sel.dtype in _DT_SEL, (x.dtype, rw.dtype, sel.dtype)

@@ -120,9 +120,9 @@ def test_interleaved_two_plane_level4_in_decode_and_prefill():
 
 
 def test_hoisted_value_map_is_an_option_with_its_own_tolerance():
-    """hoist=True: level-2 runs without a sign plane multiply the integers 1024 + S and apply A (.) + B to the sums, so their
-    weights are not rounded to fp16: within 6e-4 of the float64 oracle over the exact fp16 weights (the default holds 5e-5) and
-    within 1e-3 of the fp32 pipeline; runs at other levels or with a sign plane are not touched (same bits as the default)"""
+    """hoist=True: runs without a sign plane multiply the integers 1024 + S (level 2) or 1024 + F (levels 3, 4) and apply the value
+    map to the sums, so their weights are not rounded to fp16: within 9e-4 of the float64 oracle over the exact fp16 weights (the
+    default holds 5e-5) and within 1e-3 of the fp32 pipeline; runs with a sign plane are not touched (same bits as the default)"""
     H, I, NE = 1024, 512, 6
     ex = experts_on_gpu(H, I, NE, 810, nested_ids=(3, 4), var_ids=(2,))
     planes = [(oracle_plane(e.gu), oracle_plane(e.dn), e.nested) for e in ex]
@@ -147,9 +147,9 @@ def test_hoisted_value_map_is_an_option_with_its_own_tolerance():
         assert rel_err(y0.cpu().numpy(), want) < 5e-5
         err = rel_err(y1.cpu().numpy(), want)
         worst = max(worst, err)
-        assert 1e-6 < err < 6e-4 and rel_err(y1.cpu().numpy(), pure) < 1e-3, (B, err)
+        assert 1e-6 < err < 9e-4 and rel_err(y1.cpu().numpy(), pure) < 1e-3, (B, err)
         assert not torch.equal(y0, y1) and torch.equal(y1, y1b)
-    sel = torch.tensor([[2, 3, 4], [5, 4, 2]], device=DEV)        # a sign plane, level 3, level 4: nothing to hoist
+    sel = torch.tensor([[2, 2, 2], [2, 2, 2]], device=DEV)        # only the expert with a sign plane: nothing to hoist
     rw = torch.tensor([[0.5, 0.25, 0.25], [0.3, 0.3, 0.4]], device=DEV).half()
     x = (torch.randn(2, H, generator=g) * 0.05).half().to(DEV)
     assert torch.equal(L(x, sel, rw).clone(), L(x, sel, rw, hoist=True))
