@@ -4,7 +4,7 @@
 // (--pmc FETCH_SIZE / WRITE_SIZE) can wrap; `--calib` adds one 256 MiB device copy as the known-size kernel that scales
 // those counters.
 //
-//   nq_bench_native [--experts 64] [--batch 1] [--steps 32] [--calib] [--level L] [--prefill ROWS]
+//   nq_bench_native [--experts 64] [--batch 1] [--steps 32] [--calib] [--level L] [--prefill ROWS] [--hoist]
 //
 // --prefill ROWS times the decode-fused grouped GEMMs of the prefill path instead (nq_pf_gemm, gate|up then down): every
 // expert gets ROWS pair rows (<= 256, one tile each); --level L puts every expert at level L.
@@ -43,16 +43,17 @@ __global__ void copy_words(const uint4* __restrict__ a, uint4* __restrict__ b, s
 
 int main(int argc, char** argv)
 {
-    int E = 64, B = 1, steps = 32, calib = 0, level = 0, pf_rows = 0;
+    int E = 64, B = 1, steps = 32, calib = 0, level = 0, pf_rows = 0, hoist = 0;
     for (int i = 1; i < argc; ++i)
     {
         if (!strcmp(argv[i], "--experts") && i + 1 < argc) E = atoi(argv[++i]);
         else if (!strcmp(argv[i], "--batch") && i + 1 < argc) B = atoi(argv[++i]);
         else if (!strcmp(argv[i], "--steps") && i + 1 < argc) steps = atoi(argv[++i]);
         else if (!strcmp(argv[i], "--calib")) calib = 1;
+        else if (!strcmp(argv[i], "--hoist")) hoist = 1;
         else if (!strcmp(argv[i], "--level") && i + 1 < argc) level = atoi(argv[++i]);
         else if (!strcmp(argv[i], "--prefill") && i + 1 < argc) pf_rows = atoi(argv[++i]);
-        else { fprintf(stderr, "usage: %s [--experts E>=16] [--batch B<=8] [--steps K] [--calib] [--level 2|3|4] [--prefill ROWS<=256]\n", argv[0]); return 2; }
+        else { fprintf(stderr, "usage: %s [--experts E>=16] [--batch B<=8] [--steps K] [--calib] [--level 2|3|4] [--prefill ROWS<=256] [--hoist]\n", argv[0]); return 2; }
     }
     if ((level && level != 2 && level != 3 && level != 4) || pf_rows < 0 || pf_rows > 256) { fprintf(stderr, "need level in {2,3,4} and 0 <= ROWS <= 256\n"); return 2; }
     if (E < 16 || B < 1 || B > 8) { fprintf(stderr, "need E >= 16 and 1 <= B <= 8\n"); return 2; }
@@ -150,7 +151,7 @@ int main(int argc, char** argv)
     a.x = x; a.rw = rw; a.table = d_table; a.out = out; a.acc_gu = acc_gu; a.h = h; a.acc_d = acc_d; a.cnt_gu = cnt_gu; a.cnt_d = cnt_d;
     a.acc_gu_elems = (int64_t)ny_gu * S * 2 * I; a.acc_d_elems = (int64_t)ny_dn * S * H; a.h_elems = (int64_t)S * I; a.out_elems = (int64_t)B * H;
     a.cnt_gu_elems = (int64_t)S * (I / 128); a.cnt_d_elems = H / 128; a.cnt_h = cnt_h; a.cnt_h_elems = (int64_t)S * (I / 128); a.zd = zd; a.zd_elems = (int64_t)S * (I / 128) * 4; a.route_ws = route_ws; a.route_ws_bytes = NQ_ROUTE_WS_BYTES; a.xrot = xrot; a.xrot_elems = (int64_t)S * 2 * H; a.common_rows = 1;   /* every row here has the K=2 base and a dense residual plane */
-    a.B = B; a.topk = topk; a.E = E; a.H = H; a.I = I; a.which = 3;
+    a.B = B; a.topk = topk; a.E = E; a.H = H; a.I = I; a.which = 3; a.hoist_value_map = hoist;
     memcpy(a.cfg_gu, cfg_gu, sizeof cfg_gu); memcpy(a.cfg_dn, cfg_dn, sizeof cfg_dn);
     hipEvent_t e0, e1; HIPCHK(hipEventCreate(&e0)); HIPCHK(hipEventCreate(&e1));
     a.sel = sel; NQCHK(nq_moe_forward(&a, nullptr)); HIPCHK(hipDeviceSynchronize());            // warm-up
