@@ -198,6 +198,34 @@ def cpu_baseline(ex, levels, routes, xs, budget_s=10.0):
     return rec, y0, yt0
 
 
+def sclk_under_load(fn, settle_s=0.7):
+    """engine clock in MHz that the GPU holds while fn() is enqueued in a loop (rocm-smi read from a child process once the load
+    has run for settle_s); None where the tool is missing. The published peaks are quoted at 2400 MHz: a kernel that draws enough
+    power to be clocked down cannot reach them, whatever its code does."""
+    import re
+    import subprocess
+    import threading
+    got = []
+
+    def read():
+        time.sleep(settle_s)
+        try:
+            r = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=30)
+            m = re.search(r"sclk clock level:\s*\d+:\s*\((\d+)Mhz\)", r.stdout)
+            if m:
+                got.append(int(m.group(1)))
+        except Exception:
+            pass
+    th = threading.Thread(target=read)
+    th.start()
+    t0 = time.time()
+    while th.is_alive() and time.time() - t0 < 40:
+        fn()
+        torch.cuda.synchronize()
+    th.join()
+    return got[0] if got else None
+
+
 def zipf_routing(T, dev, seed=11, skew=1.1):
     """prefill routing: expert popularity ~ rank^-skew over a seeded permutation, 8 distinct experts per token (Gumbel top-k)"""
     g = torch.Generator().manual_seed(seed)
@@ -253,13 +281,16 @@ def prefill_leg(L, ex, dev, T=4096, reps=3):
         hot_parts = prefill_parts(L, x, sel, dev)
     finally:
         M.PF_HOT_SLOTS = 0
+    sclk = sclk_under_load(lambda: L.prefill(x, sel, rw))
     L.table.copy_(saved)
     flops = T * TOPK * 6 * H * I
     cnt = torch.bincount(sel.flatten().cpu(), minlength=E)
     return dict(workload=f"prefill: T={T} tokens, top-8 over E=256 with Zipf(1.1) popularity, all experts at level 4, "
                          f"rows per expert max {int(cnt.max())} / median {int(cnt.median())}",
                 ms=round(dt * 1e3, 3), tflops=round(flops / dt / 1e12, 1), flop=flops, mfma_peak_tflops=MFMA_PEAK_TFLOPS,
-                mfma_frac=round(flops / dt / 1e12 / MFMA_PEAK_TFLOPS, 4), rel_err_vs_oracle=float(f"{rel:.2e}"), checked_tokens=toks,
+                mfma_frac=round(flops / dt / 1e12 / MFMA_PEAK_TFLOPS, 4), sclk_mhz_under_load=sclk,
+                mfma_frac_at_that_clock=round(flops / dt / 1e12 / (MFMA_PEAK_TFLOPS * sclk / 2400.0), 4) if sclk else None,
+                rel_err_vs_oracle=float(f"{rel:.2e}"), checked_tokens=toks,
                 launches_alone=parts,
                 with_hot_scratch=dict(ms=round(hot_ms, 3), result="bitwise equal", hot_experts=hot_parts["hot_experts"],
                                       wdecode_us=hot_parts["wdecode_us"], height_256=hot_parts["height_256"], sum_us=hot_parts["sum_us"]),
@@ -898,12 +929,18 @@ def main():
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / 1e3 / (nrep * R)
     kdt, kdt_in = timed_graph(gk), timed_graph(gk_in)
+
+    def replay_gk():
+        with torch.cuda.stream(s):
+            for _ in range(8):
+                gk.replay()
+    sclk = sclk_under_load(replay_gk)
     kbytes = sum(code_bytes(ex, levels, routes[i][2], "gu") for i in range(R)) / R
     achieved = kbytes / kdt / 1e9
     roofline = dict(bound="hbm", kernel="nq_gemv_k<0, false> (gate|up decode+GEMV)", achieved=round(achieved, 1), peak=HBM_PEAK_GBS, unit="GB/s",
                     frac=round(achieved / HBM_PEAK_GBS, 4), traffic=int(kbytes * TRAFFIC_RATIO), us_per_launch=round(kdt * 1e6, 2),
                     algorithmic_bytes_per_launch=int(kbytes), us_per_launch_inside_layer_call=round(kdt_in * 1e6, 2),
-                    frac_inside_layer_call=round(kbytes / kdt_in / 1e9 / HBM_PEAK_GBS, 4),
+                    frac_inside_layer_call=round(kbytes / kdt_in / 1e9 / HBM_PEAK_GBS, 4), sclk_mhz_under_load=sclk,
                     traffic_source=f"algorithmic bytes x {TRAFFIC_RATIO}: rocprofv3 FETCH_SIZE + WRITE_SIZE of this kernel, scaled by a 256 MiB copy "
                                    "(profiles/decode_gemv_hbm_traffic_pmc.txt), not a counter read in this run",
                     timed="the gate|up projection launch alone (which = 1 | 4: with its SwiGLU finisher, routing and rotated activations "
