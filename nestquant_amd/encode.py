@@ -25,6 +25,8 @@ it is not the reference's production encoder. What it restates, in plain torch t
     factored, units fitted along anti-diagonals from the far corner with the errors of the fitted units carried over by both
     factors, and the reference's inner iterations (accept-if-better tries with the errors fed back inside a chunk);
   * the second plane of the interleaved two-plane level 4 (window code 12) with the first plane frozen (viterbi_ring_given_p3).
+  * the low-rank plane (lr_detect, lr_metric, lr_fit; nq_encode.py:507-556): the strongest eigen-directions of the input second
+    moment, the metric that leaves them to the plane, and the least-squares coefficients per level.
 The reference's encoder depends on exllamav3 1.5.1, which is not available here, so bit parity with it is not claimed;
 the tests pin this encoder by brute force on a small trellis, by decode(encode) self-consistency and by the Gaussian
 distortion the reference reports for this code (MSE 0.068 at 2 bits, threads/03-nested-trellis-code/REPORT.md:21; base +
@@ -726,6 +728,60 @@ def proxy_loss2(Q, target, Hr, Go):
     """tr(Go E H' E^T) / tr(Go T H' T^T) with E = Q - T: the expected weighted output error relative to the output's"""
     E, T = Q.double() - target.double(), target.double()
     return float(((Go @ E @ Hr) * E).sum() / ((Go @ T @ Hr) * T).sum())
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# Low-rank plane: fp16 corrections U^T V on the un-rotated input side, for the few input directions that carry most of the
+# activations' energy (table words 14 .. 17; the layer adds (x V^T) U2 at every level and (x V^T) U4 at level 4)
+
+LR_TAU, LR_RMAX = 0.05, 4        # the reference's production setting (nq_encode.py:500-501); its sparsified variant is off there
+
+
+def dense_from_rotated(Q, su, sv):
+    """the dense weight a rotated-domain matrix Q [N, K] stands for: D(sv) B_N Q B_K D(su), fp32"""
+    return (blocked_had(blocked_had(Q.double(), 1), 0) * su.double()[None, :] * sv.double()[:, None]).float()
+
+
+def lr_detect(H, tau=LR_TAU, rmax=LR_RMAX):
+    """V fp16 [r, K], r <= rmax: the unit eigenvectors of the input second moment H [K, K] whose eigenvalue is at least tau of
+    the trace, largest first (reference nq_encode.py:507-520 without its sparsification step, which production leaves off)"""
+    w, Q = torch.linalg.eigh(H.double())
+    w, Q = w.flip(0), Q.flip(1)
+    share = w / w.clamp_min(0).sum()
+    r = int((share[:rmax] >= tau).sum())
+    return Q[:, :r].T.contiguous().half()
+
+
+def lr_metric(H, V):
+    """the input metric for the trellis fit when the error inside span(V) is corrected afterwards by the low-rank plane:
+    (I - P) H (I - P) + m P with P the projector on span(V) and m the mean diagonal of the first term, which keeps the metric
+    positive definite without asking the fit for anything inside the span (reference nq_encode.py:527-537)"""
+    if V.shape[0] == 0:
+        return H
+    Vd = V.to(H.device).double()
+    P = Vd.T @ torch.linalg.solve(Vd @ Vd.T, Vd)
+    R = torch.eye(H.shape[0], dtype=torch.float64, device=H.device) - P
+    Hp = R @ H.double() @ R
+    return (Hp + Hp.diagonal().mean() * P).to(H.dtype)
+
+
+def lr_fit(W, dense2, dense4, V):
+    """least-squares coefficients of the low-rank plane on the decoded levels (reference nq_encode.py:540-556): U2 fp16 [r, N]
+    minimises |W - dense2 - U2^T V| over matrices of that form (normal equations (V V^T) U = V E^T), U4 does the same for what
+    level 4 leaves once the U2 term has been added. -> (U2, U4, dense2 + U2^T V, dense4 + (U2 + U4)^T V); the last two, fp32
+    [N, K], are what the layer multiplies at levels 2 and 4 (both terms use the fp16-rounded coefficients)."""
+    Vd = V.to(W.device).double()
+    gram = Vd @ Vd.T
+
+    def coefficients(err):
+        return torch.linalg.solve(gram, Vd @ err.double().T).half()
+    term = lambda U: (U.double().T @ Vd).float()
+    Wf = W.float()
+    U2 = coefficients(Wf - dense2)
+    with2 = dense2 + term(U2)
+    base4 = dense4 + term(U2)
+    U4 = coefficients(Wf - base4)
+    return U2, U4, with2, base4 + term(U4)
 
 
 class EncodedProj(Proj):

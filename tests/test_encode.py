@@ -303,3 +303,49 @@ def test_two_sided_ldlq_identity_and_gain():
                 p3=O.unpack_words(r["p3"].numpy(), nrec, 64), d3=u32(r["d3"]))
     for level, key in ((2, "Q"), (3, "Q3"), (4, "Q4")):
         assert same_f16(O.dense_W(p, level), r[key].half().numpy()) == 0
+
+
+def test_low_rank_plane_detect_metric_fit():
+    """lr_detect / lr_metric / lr_fit (reference threads/12-reference-encoder/nq_encode.py:507-556), pinned by what the linear
+    algebra fixes: a second moment built from known orthonormal directions gives those directions back, in order, cut at the
+    share threshold and at rmax; the metric agrees with H off the span and is m * identity on it; the fitted coefficients
+    satisfy the normal equations (the residual has nothing left inside span(V)), any other coefficients fit worse, and the
+    expected output error under activations that live mostly in the span falls by the share the span holds."""
+    g = torch.Generator().manual_seed(9)
+    K, N = 128, 128
+    Qo, _ = torch.linalg.qr(torch.randn(K, K, generator=g).double())
+    v1, v2, v3 = Qo[:, 0], Qo[:, 1], Qo[:, 2]
+    H = torch.eye(K, dtype=torch.float64) + 40 * torch.outer(v1, v1) + 15 * torch.outer(v2, v2) + 0.5 * torch.outer(v3, v3)
+    V = EN.lr_detect(H)                                           # shares 41 / 183.5, 16 / 183.5, 1.5 / 183.5 (< 0.05), 1 / 183.5 ...
+    assert V.shape == (2, K) and V.dtype == torch.float16
+    assert abs(abs(float(V[0].double() @ v1)) - 1) < 1e-3 and abs(abs(float(V[1].double() @ v2)) - 1) < 1e-3
+    assert EN.lr_detect(H, rmax=1).shape[0] == 1 and EN.lr_detect(H, tau=0.3).shape[0] == 0
+    assert EN.lr_detect(H, tau=0.001, rmax=4).shape[0] == 4       # rmax caps what the threshold would let through
+    Vd = torch.stack([v1, v2])
+    Mx = EN.lr_metric(H, Vd)
+    w = Qo[:, 5] * 0.7 + Qo[:, 9] * 0.3                           # orthogonal to the span
+    assert abs(float(w @ Mx @ w) - float(w @ H @ w)) < 1e-9
+    P = Vd.T @ Vd
+    m = float(((torch.eye(K, dtype=torch.float64) - P) @ H @ (torch.eye(K, dtype=torch.float64) - P)).diagonal().mean())
+    assert torch.allclose(Mx @ v1, m * v1, atol=1e-9) and torch.allclose(Mx, Mx.T, atol=1e-12)
+    assert float(torch.linalg.eigvalsh(Mx).min()) > 0.5 and EN.lr_metric(H, Vd[:0]) is H
+    # fit on a quantised weight
+    W = torch.randn(N, K, generator=g)
+    r = EN.encode_nested(W, seed=4)
+    su, sv = r["su"], r["sv"]
+    back = EN.dense_from_rotated(r["target"], su, sv)
+    assert float((back - W).norm() / W.norm()) < 1e-5             # D(sv) B target B D(su) is the weight itself
+    d2, d4 = EN.dense_from_rotated(r["Q"], su, sv), EN.dense_from_rotated(r["Q4"], su, sv)
+    U2, U4, w2, w4 = EN.lr_fit(W, d2, d4, V)
+    assert U2.shape == U4.shape == (2, N) and U2.dtype == torch.float16
+    Vf = V.double()
+    for dense, fitted in ((d2, w2), (d4, w4)):
+        left = (W.double() - fitted.double()) @ Vf.T              # what the residual still has inside the span
+        was = (W.double() - dense.double()) @ Vf.T
+        assert float(left.norm()) < 0.02 * float(was.norm())      # fp16 coefficients: not zero, but two orders down
+    for _ in range(3):                                            # any other coefficients are worse
+        Uo = (U2.double() + 0.02 * torch.randn(2, N, generator=g).double())
+        assert float((W.double() - d2.double() - Uo.T @ Vf).norm()) > float((W.double() - w2.double()).norm())
+    cost = lambda D: float((((W.double() - D.double()) @ H) * (W.double() - D.double())).sum())
+    assert cost(w2) < 0.75 * cost(d2) and cost(w4) < 0.75 * cost(d4)   # the span holds 57 of H's trace of 183.5
+    assert w4.dtype == torch.float32 and float((w4 - d4 - (U2.float() + U4.float()).T @ V.float()).abs().max()) < 1e-3

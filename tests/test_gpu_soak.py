@@ -7,7 +7,8 @@ acknowledged, then a relaxed arrival counter, then device-scope loads in the las
 as a one-call / two-call difference, a result that is not repeatable, a counter that does not return to zero, or a distance
 from moe_ref above the tolerance; (2) the routing corner cases (repeated experts, zero weights, level 0, every row kind in one
 call) against an independent formulation (moe_ref: dense weights from the HIP decoder, plain torch fp32 layer math);
-(3) nq_moe_forward_static on the same calls. Shapes, levels, row kinds, token counts and tilings are drawn from a seeded
+(3) nq_moe_forward_static on the same calls; (4) the hoisted value map (every third call: repeatable, within 2e-3 of the default
+result, counters clean). Nested experts read their level 4 concatenated or interleaved at random. Shapes, levels, row kinds, token counts and tilings are drawn from a seeded
 generator, so a failure names a case that can be run again."""
 import random
 
@@ -31,7 +32,8 @@ def _random_layer(rng, g, Bmax=8):
     for i in range(NE):
         nested = rng.random() < 0.5
         rk = (0, 0) if nested else (rng.choice([0, 3, 6, 7, 9]), rng.choice([0, 2, 5, 8]))
-        e = F.Expert(H, I, seed=rng.randrange(10 ** 6), dev="cpu", rk_gu=rk[0], rk_dn=rk[1], nested=nested, var=(not nested and rng.random() < 0.3))
+        e = F.Expert(H, I, seed=rng.randrange(10 ** 6), dev="cpu", rk_gu=rk[0], rk_dn=rk[1], nested=nested, var=(not nested and rng.random() < 0.3),
+                     interleave=(nested and rng.random() < 0.4))
         if rng.random() < 0.25:
             rg, rd = rng.randint(0, 4), rng.randint(0, 4)
             if rg + rd:
@@ -56,7 +58,7 @@ def _random_layer(rng, g, Bmax=8):
 def test_decode_soak(seed):
     rng = random.Random(seed)
     g = torch.Generator().manual_seed(rng.randrange(1 << 30))
-    n = nref = 0; worst = 0.0
+    n = nref = 0; worst = worst_h = 0.0
     for _layer in range(DECODE_LAYERS):
         H, I, NE, topk, ex, L, levels = _random_layer(rng, g)
         for _ in range(4):
@@ -81,12 +83,21 @@ def test_decode_soak(seed):
             assert torch.equal(y3, ys), ("built-in scratch differs from caller workspaces", case)
             assert bool(torch.isfinite(y3).all()), ("not finite", case)
             assert not L.cnt_gu.any() and not L.cnt_d.any() and not L.cnt_h.any(), ("arrival counters not back at zero", case)
+            if n % 3 == 0:                                         # the hoisted value map: other roundings, same layer
+                yh = L(x, sel, rw, cfg_gu=cg, cfg_dn=cd, hoist=True).clone()
+                yh2 = L(x, sel, rw, cfg_gu=cg, cfg_dn=cd, hoist=True, out=torch.empty_like(yh), static_ws=True)
+                torch.cuda.synchronize()
+                assert torch.equal(yh, yh2), ("hoisted call not repeatable", case)
+                dh = ((yh - y3).norm() / (y3.norm() + 1e-20)).item()
+                worst_h = max(worst_h, dh)
+                assert dh < 2e-3 and not L.cnt_gu.any() and not L.cnt_d.any() and not L.cnt_h.any(), ("hoisted call far from the default", dh, case)
             if n % 6 == 0:
                 ref = M.moe_ref(ex, levels, x, sel, rw)
                 err = ((y3 - ref).norm() / (ref.norm() + 1e-20)).item()
                 worst = max(worst, err); nref += 1
                 assert err < 1e-3, ("far from moe_ref", err, case)
-    print(f"decode soak seed {seed}: {n} calls, {nref} compared with moe_ref, worst rel err {worst:.2e}")
+    print(f"decode soak seed {seed}: {n} calls, {nref} compared with moe_ref, worst rel err {worst:.2e}; "
+          f"hoisted value map at most {worst_h:.2e} from the default")
     assert n == 4 * DECODE_LAYERS
 
 

@@ -28,7 +28,7 @@ def test_step_offsets_cover_the_ring(code):
 
 
 def test_published_plane_sizes():
-    # TP8 shard I = 256 (reference INTEGRATION.md:26-33): gate|up [512, 6144], down [6144, 256]
+    # TP8 shard I = 256 (reference threads/13-moe-layer-kernel/INTEGRATION.md:26-33): gate|up [512, 6144], down [6144, 256]
     gu, dn = O.proj_sizes(512, 6144, rk=6), O.proj_sizes(6144, 256, rk=7)
     assert (gu["base"], dn["base"]) == (786432, 393216)
     assert (gu["p4"] - 4, dn["p4"] - 4) == (761856, 454656)           # payload; the tail sub-array adds a 4-byte pad
