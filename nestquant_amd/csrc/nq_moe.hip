@@ -503,10 +503,13 @@ __device__ __forceinline__ void finish_dn(const MoeArgs& a, const PickInfo& R, i
 // host says so, MoeArgs::common_rows). A run whose row is nevertheless of another kind is not decoded as if it were common:
 // its plane is not read and its partial sums are NaN, so every token that picked it comes out NaN. ANYROW = true also
 // carries the decode loops of the other base codes and of mask mode, which cost ~35 registers that the common kernel does
-// not have to pay for. Four wavefronts per SIMD is the measured optimum for both (three: +4 us per layer; five, which the
-// common kernel reaches at 92 registers: +1.5 us), so the register allocator is told to aim at exactly that.
+// not have to pay for. Four wavefronts per SIMD is the measured optimum for the gate|up launch (three: +4 us per layer; five,
+// which the common kernel reaches at 92 registers: +1.5 us), so the register allocator is told to aim at exactly that. The
+// common down launch gains from five (96 registers, three of them spilled): its 1536 workgroups then need 1.2 rounds instead of
+// 1.5 (-0.4 us per layer at one token, -2.5 us at four); six spills sixteen registers and loses 0.9 us.
 template <int MODE, bool ANYROW>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) nq_gemv_k(MoeArgs a, int NC)
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MODE == 1 && !ANYROW ? 5 : 4, MODE == 1 && !ANYROW ? 5 : 4)))
+nq_gemv_k(MoeArgs a, int NC)
 {
     extern __shared__ __align__(16) char smem[];
     __builtin_amdgcn_s_setprio(3);                               // the head is a chain of latencies (see progress_priority)

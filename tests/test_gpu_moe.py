@@ -565,15 +565,16 @@ def test_odd_shapes_decode_and_prefill_vs_full_oracle(H, I, NE, topk, seed):
 
 
 def test_occupancy_query_matches_the_launch_shape_the_layer_uses():
-    """moe.occ (the reference's M.occ): the common decode kernels are built for four wavefronts per SIMD, i.e. four resident
-    workgroups of four wavefronts per CU at the full shape's LDS use, and spill nothing"""
+    """moe.occ (the reference's M.occ): the common gate|up kernel is built for four wavefronts per SIMD, i.e. four resident
+    workgroups of four wavefronts per CU at the full shape's LDS use, and spills nothing; the common down kernel for five,
+    at the price of a few spilled registers (at most 16 bytes per lane)"""
     H, I, B = 6144, 2048, 1
     cfg_gu, cfg_dn = M.MoELayer.default_cfg(H, I)
     for mode, cf in ((0, cfg_gu), (1, cfg_dn)):
         nc, sb = cf[0] * cf[2], cf[1]
         shm = max(B * (nc * 256 + 16) + 256, sb * 512)
         wgs, regs, spill = M.occ(mode, sb, shm)
-        assert wgs * sb == 16 and 64 < regs <= 128 and spill == 0, (mode, wgs, regs, spill)
+        assert wgs * sb == (16, 20)[mode] and 64 < regs <= (128, 96)[mode] and spill <= (0, 16)[mode], (mode, wgs, regs, spill)
     assert M.occ(0, 4, 4096, any_rows=True)[0] >= 1
     with pytest.raises(RuntimeError, match="nq_occ"):
         M.occ(2, 4, 0)
