@@ -916,7 +916,7 @@ def main():
         for i in range(R):
             gu_only(i, 13)
     L.route, L.xrot = ws_main
-    nrep = max(1, (K + R - 1) // R)
+    nrep = max(8, (K + R - 1) // R)                               # at least 512 launches, however few steps the headline times
 
     def timed_graph(gr):
         with torch.cuda.stream(s):
