@@ -154,6 +154,13 @@ def test_hoisted_value_map_is_an_option_with_its_own_tolerance():
     x = (torch.randn(2, H, generator=g) * 0.05).half().to(DEV)
     assert torch.equal(L(x, sel, rw).clone(), L(x, sel, rw, hoist=True))
     print(f"hoisted value map: worst distance from the float64 oracle {worst:.2e}")
+    # a layer with a row of a rare kind (mask mode) runs the complete kernel, which has no hoisted loops: the option changes nothing
+    rare = to_dev([F.Expert(H, I, seed=830, dev="cpu"), F.Expert(H, I, seed=831, dev="cpu", nm_gu=3, nm_dn=2)])
+    L2 = M.MoELayer(2, H, I, Bmax=2, topk=2)
+    L2.set(0, rare[0], 2); L2.set(1, rare[1], 4)
+    sel2 = torch.tensor([[0, 1], [1, 0]], device=DEV)
+    rw2 = rw[:, :2].contiguous()
+    assert torch.equal(L2(x, sel2, rw2).clone(), L2(x, sel2, rw2, hoist=True))
 
 
 def test_golden_layer_fixture(golden_dir):
