@@ -102,7 +102,10 @@ def test_config5_full_size_churn(in_call):
             moved += len(routed & swapped)
             err = rel_err(y, oracle_out(st, X.level)[0])
             worst = max(worst, err)
-            assert err < 1e-4, (st, err)                         # a stale or mixed state is off by percents; the reference holds ~1e-4 (sm120/results/check_I512.txt)
+            # a stale or mixed state is off by percents (every expert has a level-4 sign vector of its own); which states the checks
+            # meet depends on when the copies land, and runs of this loop have reached 7e-5, so the bar is the one the reference's
+            # own racing check reaches (max_rel_err 1.8e-4, threads/13-moe-layer-kernel/levelswitch_mbox.json) with some room
+            assert err < 3e-4, (st, err)
             for e in sorted(swapped)[:6]:                         # bit-exact dequant after the swap, at the level the books say
                 if e in X.pend:
                     continue
